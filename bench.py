@@ -1,0 +1,179 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized Gram build (the hot path of hyacinTsvdFit) on one MI355X.
+
+A step = hyacinXquantizeScaleBatch + hyacinXherkBatch on a synthetic matrix that is already resident in
+HBM: per-column exponents, int8 CRT-residue / limb quantization, the int8 MFMA contraction and the
+reconstruction of the exact integer Gram.  Prints ONE JSON line:
+  value      effective Gram TFLOP/s = M N (N+1) (x4 complex) / step time  (the FP SYRK/HERK flops replaced)
+  roofline   the contraction kernel alone, timed with HIP events on its stream: algorithmic int8 ops / time
+             against the dense INT8 MFMA peak
+  cpu_baseline  the same limb / CRT algorithm compiled for the host (the oracle), timed on a row sample
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+INT8_PEAK_TOPS = 5000.0   # MI355X dense INT8 MFMA peak, 5.0 POP/s
+
+WORKLOADS = {
+    # name: (type, opA, M, N, K, eps, algorithm, description)
+    "target": (0, "N", 131072, 2048, 1024, 1e-12, b"A", "real FP64 M=131072 N=2048 eps=1e-12 (CRT real, 14 moduli)"),
+    "cfg1": (0, "N", 4096, 256, 256, 1e-10, b"L", "real FP64 M=4096 N=256 eps=1e-10 (limbs, 6 digits)"),
+    "cfg2": (2, "T", 65536, 1024, 512, 1e-5, b"A", "real FP32 opA=T M=65536 N=1024 eps=1e-5 (CRT real, 8 moduli)"),
+    "cfg3": (1, "N", 131072, 2048, 1024, 1e-12, b"A", "complex FP64 M=131072 N=2048 eps=1e-12 (CRT complex, 15 moduli)"),
+}
+
+
+def synth(torch, at, M, N, seed):
+    """Column-scaled Gaussian test matrix generated on the device, column-major M x N."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    real = torch.float64 if at in (0, 1) else torch.float32
+    comps = 2 if at & 1 else 1
+    scale = torch.pow(10.0, -torch.arange(N, device="cuda", dtype=torch.float64) / (N / 8.0)).to(real)
+    A = torch.randn((N, M, comps), generator=g, device="cuda", dtype=real) * scale[:, None, None]
+    return A.contiguous()
+
+
+def algorithmic_ops(alg, order, cplx, M, N):
+    if alg == "C":
+        if not cplx:
+            return order * M * N * (N + 1)
+        return min(order, 20) * 2 * M * N * N + max(order - 20, 0) * (M * N * (N + 1) + 2 * M * N * N)
+    ops = order * M * N * (N + 1) + order * (order - 1) * M * N * N
+    return ops + (order * order * 2 * M * N * N if cplx else 0)
+
+
+def cpu_baseline(at, M, N, eps, alg, order, u, sample_rows):
+    """The oracle's quantize + int8 Gram + reconstruction on the first sample_rows rows, all host cores."""
+    import numpy as np
+    from oracle import ho
+    rng = np.random.default_rng(3)
+    cplx = at & 1
+    A = rng.standard_normal((sample_rows, N)) * 10.0 ** (-np.arange(N) / (N / 8.0))
+    if cplx:
+        A = A + 1j * rng.standard_normal((sample_rows, N)) * 10.0 ** (-np.arange(N) / (N / 8.0))
+    A = A.astype({0: np.float64, 1: np.complex128, 2: np.float32, 3: np.complex64}[at])
+    ho.build()
+    t0 = time.perf_counter()
+    vexp = ho.quantize_scale_batch(A, 1, sample_rows, sample_rows, u)
+    kind = "crt" if alg == "C" else "limbs"
+    K = (sample_rows + 127) // 128 * 128
+    panels = ho.quantize(kind, A, order, vexp, ldb=K)
+    ho.i8herk(kind, cplx, N, order, panels, 0, 2)
+    dt = time.perf_counter() - t0
+    feff = sample_rows * N * (N + 1) * (4 if cplx else 1)
+    out = {"value": feff / dt / 1e12, "unit": "TFLOP/s (FP-equivalent Gram flops)", "cores": os.cpu_count(), "kind": "port",
+           "sample": "first %d of %d rows (int8 work is linear in rows), %s order %d, %.2f s" % (sample_rows, M, kind, order, dt)}
+    try:   # FP reference: SYRK / HERK from the BLAS scipy ships, on the same sample
+        from scipy.linalg import blas
+        t0 = time.perf_counter()
+        (blas.zherk if cplx else blas.dsyrk)(1.0, np.asfortranarray(A.astype(np.complex128 if cplx else np.float64)), trans=2 if cplx else 1)
+        out["fp_blas_tflops"] = feff / (time.perf_counter() - t0) / 1e12
+    except Exception as e:  # pragma: no cover
+        out["fp_blas_tflops"] = None
+        out["fp_blas_note"] = "BLAS unavailable: %s" % e
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="target", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-fit", action="store_true", help="skip the end-to-end hyacinTsvdFit timing")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--cpu-rows", type=int, default=4096)
+    ap.add_argument("--slab", type=int, default=0, help="K slab of the contraction kernel (64 or 128)")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        print("bench.py measures one GPU: the Gram path of this build has no multi-GPU leg (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import hyacinth_amd as ha
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    L = ha.lib()
+    at, opA, M, N, K, eps, alg, desc = WORKLOADS[a.workload]
+    if a.slab:
+        assert L.hykGramSetSlab(a.slab) == 0
+    stream = torch.cuda.current_stream().cuda_stream
+    h = ha.create_handle(stream=stream, GramMatrixAlgorithm=alg)
+    cplx = at & 1
+    A = synth(torch, at, M, N, 0x4859)          # stored column-major M x N; opA='T' workloads are benchmarked on the transposed copy the fit makes
+    lda = M
+    u, cP, lP, stride = ha.herk_batch_init(h, eps, M, N, at)
+    seg = min(h.GramSegmentK, M) if h.GramSegmentK > 0 else M
+    batches, lastM = (M + seg - 1) // seg, M - (M - 1) // seg * seg
+    vexp = torch.zeros((batches + 1) * N, dtype=torch.int32, device="cuda")
+    Cq = torch.zeros(cP * lP * stride, dtype=torch.int64, device="cuda")
+    pA, pV, pC = C.c_void_p(A.data_ptr()), C.c_void_p(vexp.data_ptr()), C.c_void_p(Cq.data_ptr())
+
+    def step():
+        L.hyacinXquantizeScaleBatch(C.byref(h), batches, seg, lastM, N, at, pA, lda, u, pV)
+        L.hyacinXherkBatch(C.byref(h), batches, seg, lastM, N, at, pA, lda, u, pV, 0, lP, pC)
+
+    for _ in range(a.warmup):
+        step()
+    torch.cuda.synchronize()
+    L.hykGramProfile(1)
+    t0 = time.perf_counter()
+    for _ in range(a.steps):
+        step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / a.steps
+    kms, kn = C.c_double(), C.c_int32()
+    L.hykGramProfileRead(C.byref(kms), C.byref(kn))
+    L.hykGramProfile(0)
+
+    # the plan the library followed (same planner, host side)
+    from oracle import ho
+    plan_alg, order, _ = ho.gram_algorithm(alg.decode(), M if batches <= 1 else M, u + cplx, cplx, h.TCGemmTargetK, h.StrideBatchPerfPenalty)
+    ops = algorithmic_ops(plan_alg, order, cplx, M, N)
+    feff = M * N * (N + 1) * (4 if cplx else 1)
+    launches_per_step = max(1, kn.value // a.steps)
+    t_kernel = kms.value / 1e3 / a.steps            # contraction kernel time per step
+    achieved = ops / t_kernel / 1e12 if t_kernel > 0 else 0.0
+
+    fit_ms = None
+    if not a.no_fit:
+        S = torch.zeros(K, dtype=torch.float64, device="cuda")
+        V = torch.zeros(N * K * (2 if cplx else 1), dtype=torch.float64 if at in (0, 1) else torch.float32, device="cuda")
+        times = []
+        for i in range(3):
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            rank = L.hyacinTsvdFit(C.byref(h), eps, b"N", M, N, K, pA, lda, C.c_void_p(S.data_ptr()), C.c_void_p(V.data_ptr()), N, 0, at)
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t1) * 1e3)
+        fit_ms = sorted(times[1:])[len(times[1:]) // 2]
+
+    out = {
+        "metric": "Gram-build effective TFLOPS (+ % INT8 MFMA peak; hyacinTsvdFit wall ms)",
+        "value": feff / dt / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 (i32 accumulate)", "data": "synthetic",
+        "config": {"workload": "%s: %s" % (a.workload, desc), "M": M, "N": N, "eps": eps, "algorithm": plan_alg, "order": order,
+                   "quant_bits": u, "gram_limbs": lP, "row_slices": batches},
+        "pct_int8_mfma_peak": 100.0 * achieved / INT8_PEAK_TOPS,
+        "tsvd_fit_ms": fit_ms,
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s", "frac": achieved / INT8_PEAK_TOPS, "traffic": None,
+                     "kernel": "gram_kernel", "ops": "int8 multiply-adds x2, upper triangle only", "launches_per_step": launches_per_step,
+                     "avg_launch_ms": kms.value / max(1, kn.value), "algorithmic_ops_per_step": ops},
+    }
+    if not a.no_cpu:
+        rows = min(a.cpu_rows, M)
+        out["cpu_baseline"] = cpu_baseline(at, M, N, eps, plan_alg, order, u, rows)
+    ha.destroy_handle(h)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,388 @@
+/*
+ * gram_mfma.hip -- the int8 Gram contraction on the CDNA4 matrix cores, and the
+ * kernels that turn its accumulators into the 63-bit-limb integer Gram.
+ *
+ * Replaces, in the reference, the cuBLAS int8 GEMMs of src/hyacin_herk.cpp:61-251
+ * together with the int32 -> accumulator kernels src/limbs_diag.cu,
+ * src/limbs_cross_real.cu, src/limbs_cross_imag.cu, src/crt_diag_real.cu,
+ * src/crt_rotate.cu, src/crt_extra_real.cu, src/crt_extra_imag.cu (all fused into
+ * the contraction's epilogue: the int32 products never reach HBM), and
+ * src/crt_reconstruct_real.cu / src/crt_reconstruct_complex.cu.
+ *
+ * Data layout.  int8 panels, K-contiguous: panel p, column j, row k at
+ * panels[p * panelStride + j * ldb + k]; K (rows) is a multiple of 128 with the
+ * padding rows zero.  Accumulators: plane q, packed-triangle entry
+ * y + x(x+1)/2 (y <= x) at acc[q * planeStride + entry]; uint32 sums of
+ * canonical residues for the CRT path, int64 sums for the limb path.
+ *
+ * Work decomposition.  A work item is (group, 256x256 tile (ta <= tb) of the
+ * upper block triangle, K split).  A group is a list of panel pairs
+ * (lanePanel, aPanel) whose products  W[y, x] = sum_k lanePanel[k, y] *
+ * aPanel[k, x]  (y in block ta, x in block tb) are summed in int32 on the
+ * MFMA accumulators, plus an epilogue rule that says which accumulator planes
+ * receive  +-W  or  (c * W) mod m.  Exact integer addition commutes, so items
+ * combine through atomics in any order and the result is bit-identical to any
+ * serial schedule.  Lower-triangle products (needed by the complex paths) are
+ * expressed as groups with the two panels swapped, so that the lane dimension of
+ * the MFMA output always runs along the contiguous index of the packed triangle.
+ *
+ * Mapping to the chip.  One 256-thread workgroup (4 wavefronts, 2x2, each
+ * 128x128 = 4x4 v_mfma_i32_32x32x32_i8 tiles, 256 accumulator registers per
+ * lane) per item; operand tiles staged through LDS in double-buffered K slabs
+ * with a padded row pitch that makes the 16-byte fragment reads conflict-free.
+ * Workgroups are dispatched round-robin over the 8 XCDs, so item =
+ * (blockIdx % 8) * itemsPerXcd + blockIdx / 8 keeps the items that run
+ * together on one XCD (one L2) on the same panels and K range.
+ */
+#include <vector>
+#include <hip/hip_runtime.h>
+#include "hyk_common.h"
+#include "crt_tables.h"
+#include "hyacin_kernels.h"
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int TILE = 256;        /* output tile edge per workgroup */
+constexpr int WAVE_TILE = 128;   /* output tile edge per wavefront */
+constexpr int G_THREADS = 256;
+constexpr int MAX_GROUPS = 48;
+constexpr int MAX_PAIRS = 192;
+constexpr int XCDS = 8;
+
+enum { EPI_MOD = 0, EPI_I64 = 1 };
+
+struct GramGroup {
+  uint16_t pairBegin, pairCount;
+  uint16_t planeRe, planeIm;
+  uint32_t m, d, c32;       /* EPI_MOD: modulus, floor(2^32/m), 2^32 mod m */
+  uint32_t mulRe, mulIm;    /* EPI_MOD: multipliers in [0, m), 0 = no contribution; EPI_I64: 0 none, 1 add, 2 subtract */
+};
+
+struct GramArgs {
+  const int8_t* panels; int64_t ldb, panelStride;
+  void* acc; int64_t planeStride;
+  int32_t N, nT, tileCount, kLen, kSplits, K, groupCount, totalItems, itemsPerXcd;
+  GramGroup groups[MAX_GROUPS];
+  uint32_t pairs[MAX_PAIRS];  /* lanePanel | aPanel << 16 */
+};
+
+/* element (i, j) of a 32x32 MFMA result held in accumulator register r of a lane */
+__device__ __forceinline__ int acc_row(int r, int lane) { return ((r >> 2) << 3) + ((lane >> 5) << 2) + (r & 3); }
+
+template <int BK> struct Slab {
+  static constexpr int PITCH = BK + 16;                 /* bytes per tile row in LDS; 16-byte pad => conflict-free b128 reads */
+  static constexpr int TILE_BYTES = TILE * PITCH;
+  static constexpr int PIECES = TILE * BK / 16;         /* 16-byte pieces per operand tile */
+  static constexpr int PER_THREAD = PIECES / G_THREADS; /* pieces each thread moves per operand tile */
+  static constexpr int PER_ROW = BK / 16;
+};
+
+template <int BK, int EPI>
+__global__ __launch_bounds__(G_THREADS, 1) void gram_kernel(const GramArgs args) {
+  using S = Slab<BK>;
+  extern __shared__ __align__(16) int8_t lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wy = wave & 1, wx = wave >> 1;
+
+  /* XCD-aware item mapping */
+  const int item = (int)(blockIdx.x % XCDS) * args.itemsPerXcd + (int)(blockIdx.x / XCDS);
+  if ((int)(blockIdx.x / XCDS) >= args.itemsPerXcd || item >= args.totalItems) { return; }
+  const int t = item % args.tileCount, gk = item / args.tileCount, ks = gk % args.kSplits, g = gk / args.kSplits;
+  int tb = (int)((__fsqrt_rn(8.f * (float)t + 1.f) - 1.f) * 0.5f);
+  while ((tb + 1) * (tb + 2) / 2 <= t) { ++tb; } while (tb * (tb + 1) / 2 > t) { --tb; }
+  const int ta = t - tb * (tb + 1) / 2;
+  const GramGroup grp = args.groups[g];
+  const int k0 = ks * args.kLen, kEnd = (k0 + args.kLen) < args.K ? (k0 + args.kLen) : args.K, slabs = (kEnd - k0) / BK;
+  const int y0 = ta * TILE, x0 = tb * TILE;
+
+  /* per-thread global source offsets (column clamped to N-1: out-of-range columns only feed masked outputs) */
+  int64_t srcLane[S::PER_THREAD], srcA[S::PER_THREAD]; int dstOff[S::PER_THREAD];
+  #pragma unroll
+  for (int r = 0; r < S::PER_THREAD; ++r) {
+    const int p = tid + r * G_THREADS, row = p / S::PER_ROW, kq = p % S::PER_ROW;
+    int cy = y0 + row; cy = cy < args.N ? cy : args.N - 1; int cx = x0 + row; cx = cx < args.N ? cx : args.N - 1;
+    srcLane[r] = (int64_t)cy * args.ldb + kq * 16; srcA[r] = (int64_t)cx * args.ldb + kq * 16; dstOff[r] = row * S::PITCH + kq * 16;
+  }
+
+  v16i acc[4][4];
+  #pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    #pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      #pragma unroll
+      for (int r = 0; r < 16; ++r) { acc[a][b][r] = 0; }
+    }
+  }
+
+  const int iters = slabs * grp.pairCount;
+  v4i regLane[S::PER_THREAD], regA[S::PER_THREAD];
+  /* position of the next slab to fetch: pair index within the group and slab within the K range (both wave-uniform) */
+  int nextPair = 0, nextSlab = 0; const int8_t* baseLane = args.panels; const int8_t* baseA = args.panels;
+  auto fetch = [&]() {
+    if (nextSlab == 0) {
+      const uint32_t pp = args.pairs[__builtin_amdgcn_readfirstlane(grp.pairBegin + nextPair)];
+      baseLane = args.panels + (int64_t)(pp & 0xffffu) * args.panelStride + k0; baseA = args.panels + (int64_t)(pp >> 16) * args.panelStride + k0;
+    }
+    #pragma unroll
+    for (int r = 0; r < S::PER_THREAD; ++r) { regLane[r] = *reinterpret_cast<const v4i*>(baseLane + srcLane[r]); }
+    #pragma unroll
+    for (int r = 0; r < S::PER_THREAD; ++r) { regA[r] = *reinterpret_cast<const v4i*>(baseA + srcA[r]); }
+    baseLane += BK; baseA += BK; if (++nextSlab == slabs) { nextSlab = 0; ++nextPair; }
+  };
+  auto stash = [&](int stage) {
+    int8_t* tileLane = lds + stage * 2 * S::TILE_BYTES; int8_t* tileA = tileLane + S::TILE_BYTES;
+    #pragma unroll
+    for (int r = 0; r < S::PER_THREAD; ++r) { *reinterpret_cast<v4i*>(tileLane + dstOff[r]) = regLane[r]; }
+    #pragma unroll
+    for (int r = 0; r < S::PER_THREAD; ++r) { *reinterpret_cast<v4i*>(tileA + dstOff[r]) = regA[r]; }
+  };
+
+  /* fragment base offsets: lanes 0-31 take K bytes [0,16), lanes 32-63 bytes [16,32) of each 32-deep MFMA step */
+  const int fragLane = (wy * WAVE_TILE + (lane & 31)) * S::PITCH + (lane >> 5) * 16;
+  const int fragA = (wx * WAVE_TILE + (lane & 31)) * S::PITCH + (lane >> 5) * 16;
+
+  if (iters > 0) { fetch(); stash(0); }
+  __syncthreads();
+  for (int it = 0; it < iters; ++it) {
+    const int stage = it & 1;
+    if (it + 1 < iters) { fetch(); }
+    const int8_t* tileLane = lds + stage * 2 * S::TILE_BYTES; const int8_t* tileA = tileLane + S::TILE_BYTES;
+    #pragma unroll
+    for (int kk = 0; kk < BK / 32; ++kk) {
+      v4i fl[4], fa[4];
+      #pragma unroll
+      for (int b = 0; b < 4; ++b) { fl[b] = *reinterpret_cast<const v4i*>(tileLane + fragLane + b * 32 * S::PITCH + kk * 32); }
+      #pragma unroll
+      for (int a = 0; a < 4; ++a) { fa[a] = *reinterpret_cast<const v4i*>(tileA + fragA + a * 32 * S::PITCH + kk * 32); }
+      #pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        #pragma unroll
+        for (int b = 0; b < 4; ++b) { acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[a], fl[b], acc[a][b], 0, 0, 0); }
+      }
+    }
+    if (it + 1 < iters) { stash(stage ^ 1); }
+    __syncthreads();
+  }
+
+  /* epilogue: lane dimension j <-> y (contiguous in the packed triangle), register dimension i <-> x */
+  const bool diagTile = (ta == tb);
+  #pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    #pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int y = y0 + wy * WAVE_TILE + b * 32 + (lane & 31);
+      #pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int x = x0 + wx * WAVE_TILE + a * 32 + acc_row(r, lane);
+        if (x < args.N && y < args.N && (!diagTile || y <= x)) {
+          const int64_t e = hyk::tri_index(y, x); const int32_t w = acc[a][b][r];
+          if constexpr (EPI == EPI_MOD) {
+            uint32_t* dst = reinterpret_cast<uint32_t*>(args.acc);
+            const uint32_t v = hyk::reduce_i32(w, grp.m, grp.d, grp.c32);
+            if (grp.mulRe) { atomicAdd(&dst[(int64_t)grp.planeRe * args.planeStride + e], grp.mulRe == 1u ? v : hyk::reduce_u32(v * grp.mulRe, grp.m, grp.d)); }
+            if (grp.mulIm) { atomicAdd(&dst[(int64_t)grp.planeIm * args.planeStride + e], grp.mulIm == 1u ? v : hyk::reduce_u32(v * grp.mulIm, grp.m, grp.d)); }
+          } else {
+            unsigned long long* dst = reinterpret_cast<unsigned long long*>(args.acc);
+            const unsigned long long pos = (unsigned long long)(long long)w, negv = (unsigned long long)(-(long long)w);
+            if (grp.mulRe) { atomicAdd(&dst[(int64_t)grp.planeRe * args.planeStride + e], grp.mulRe == 1u ? pos : negv); }
+            if (grp.mulIm) { atomicAdd(&dst[(int64_t)grp.planeIm * args.planeStride + e], grp.mulIm == 1u ? pos : negv); }
+          }
+        }
+      }
+    }
+  }
+}
+
+/* ------------------------------------------------------------------ CRT reconstruction */
+struct ReconTable {
+  int32_t order;
+  uint32_t m[HYK_CRT_CPLX_COUNT], d[HYK_CRT_CPLX_COUNT], minv[HYK_CRT_CPLX_COUNT];
+  uint64_t Pd[HYK_CRT_CPLX_COUNT][3], P[3];
+};
+
+/* entry e of plane z: residues from the uint32 sums, centred CRT lift, C (+)= value.  clear: zero the sums afterwards. */
+__global__ __launch_bounds__(256) void crt_reconstruct_kernel(const ReconTable tab, int64_t count, uint32_t* __restrict__ acc, int64_t planeStride, int32_t beta, int32_t orderC, uint64_t* __restrict__ C, int32_t clear) {
+  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; const int z = blockIdx.y;
+  if (e >= count) { return; }
+  hyk::I192 a; a.w[0] = a.w[1] = a.w[2] = 0;
+  for (int x = 0; x < tab.order; ++x) {
+    uint32_t* src = &acc[(int64_t)(z * tab.order + x) * planeStride + e];
+    const uint32_t r = hyk::reduce_u32(*src, tab.m[x], tab.d[x]); if (clear) { *src = 0u; }
+    const uint32_t tt = hyk::reduce_u32(r * tab.minv[x], tab.m[x], tab.d[x]);
+    hyk::I192 pd; pd.w[0] = tab.Pd[x][0]; pd.w[1] = tab.Pd[x][1]; pd.w[2] = tab.Pd[x][2];
+    /* keep |a| < P: add t * (P/m) when a < 0, (t - m) * (P/m) otherwise */
+    if (hyk::i192_is_neg(a)) { hyk::i192_add(a, hyk::i192_mul_small(pd, tt)); }
+    else { hyk::i192_add(a, hyk::i192_neg(hyk::i192_mul_small(pd, tab.m[x] - tt))); }
+  }
+  hyk::I192 P; P.w[0] = tab.P[0]; P.w[1] = tab.P[1]; P.w[2] = tab.P[2];
+  if (hyk::i192_is_neg(a)) { hyk::i192_add(a, P); }
+  hyk::I192 twice = a; hyk::i192_add(twice, a); hyk::I192 diff = twice; hyk::i192_add(diff, hyk::i192_neg(P));
+  if (!hyk::i192_is_neg(diff)) { hyk::i192_add(a, hyk::i192_neg(P)); }   /* 2a >= P  ->  a - P, result in [-P/2, P/2) */
+  uint64_t* out = &C[(int64_t)z * orderC * count + e];
+  if (beta) { hyk::I192 old = hyk::limbs_to_i192(orderC, out, count); hyk::i192_add(a, old); }
+  hyk::i192_to_limbs(a, orderC, out, count);
+}
+
+/* limb path: C (+)= sum_s T_s 2^(8 s) */
+__global__ __launch_bounds__(256) void limb_combine_kernel(int64_t count, int32_t levels, unsigned long long* __restrict__ acc, int64_t planeStride, int32_t beta, int32_t orderC, uint64_t* __restrict__ C, int32_t clear) {
+  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; const int z = blockIdx.y;
+  if (e >= count) { return; }
+  hyk::I192 a; a.w[0] = a.w[1] = a.w[2] = 0;
+  for (int s = 0; s < levels; ++s) {
+    unsigned long long* src = &acc[(int64_t)(z * levels + s) * planeStride + e];
+    const int64_t v = (int64_t)*src; if (clear) { *src = 0ull; }
+    hyk::i192_add_shifted_i64(a, v, 8u * (uint32_t)s);
+  }
+  uint64_t* out = &C[(int64_t)z * orderC * count + e];
+  if (beta) { hyk::I192 old = hyk::limbs_to_i192(orderC, out, count); hyk::i192_add(a, old); }
+  hyk::i192_to_limbs(a, orderC, out, count);
+}
+
+__global__ void fill_zero_kernel(uint4* __restrict__ p, int64_t n16) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; if (i < n16) { p[i] = make_uint4(0, 0, 0, 0); }
+}
+
+/* ------------------------------------------------------------------ host-side planning */
+struct Launch { GramArgs args; int epi; };
+
+int g_bk = 64;  /* K slab per LDS stage: 64 or 128 (set through hykGramSetSlab for tuning) */
+
+/* optional per-launch timing of the contraction kernel with HIP events on its own stream */
+struct Timed { hipEvent_t start, stop; };
+bool g_profile = false; std::vector<Timed> g_timed;
+
+template <int BK, int EPI> hipError_t launch_one(hipStream_t stream, const GramArgs& a) {
+  const int ldsBytes = 2 * 2 * Slab<BK>::TILE_BYTES;
+  static bool attr = false;
+  if (!attr) { hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gram_kernel<BK, EPI>), hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes); if (e != hipSuccess) { return e; } attr = true; }
+  const int blocks = a.itemsPerXcd * XCDS;
+  Timed t{ nullptr, nullptr };
+  if (g_profile) { if (hipEventCreate(&t.start) != hipSuccess || hipEventCreate(&t.stop) != hipSuccess) { return hipErrorUnknown; } (void)hipEventRecord(t.start, stream); }
+  gram_kernel<BK, EPI><<<blocks, G_THREADS, ldsBytes, stream>>>(a);
+  if (g_profile) { (void)hipEventRecord(t.stop, stream); g_timed.push_back(t); }
+  return hipGetLastError();
+}
+
+hipError_t launch_gram(hipStream_t stream, GramArgs& a, int epi, int maxProducts) {
+  /* K split: enough items to fill the chip a few times over, never more than maxProducts int8 products per int32 */
+  int maxPairs = 1; for (int g = 0; g < a.groupCount; ++g) { maxPairs = a.groups[g].pairCount > maxPairs ? a.groups[g].pairCount : maxPairs; }
+  const int bk = g_bk; int kCap = (maxProducts / maxPairs) / bk * bk; if (kCap < bk) { return hipErrorInvalidValue; }
+  const int64_t base = (int64_t)a.groupCount * a.tileCount; int splits = 1;
+  const int wanted = 1024;  /* about four waves of 256 workgroups */
+  if (base < wanted) { splits = (int)((wanted + base - 1) / base); }
+  int kLen = ((a.K + splits - 1) / splits + bk - 1) / bk * bk; if (kLen < 2048) { kLen = 2048; } if (kLen > kCap) { kLen = kCap; }
+  if (kLen > a.K) { kLen = a.K; }
+  a.kLen = kLen; a.kSplits = (a.K + kLen - 1) / kLen;
+  const int64_t total = base * a.kSplits; if (total > 0x7fffffff / 2) { return hipErrorInvalidValue; }
+  a.totalItems = (int)total; a.itemsPerXcd = (int)((total + XCDS - 1) / XCDS);
+  if (bk == 128) { return epi == EPI_MOD ? launch_one<128, EPI_MOD>(stream, a) : launch_one<128, EPI_I64>(stream, a); }
+  return epi == EPI_MOD ? launch_one<64, EPI_MOD>(stream, a) : launch_one<64, EPI_I64>(stream, a);
+}
+
+void base_args(GramArgs& a, const int8_t* panels, int64_t ldb, int32_t N, int32_t K, void* acc) {
+  a.panels = panels; a.ldb = ldb; a.panelStride = (int64_t)N * ldb; a.acc = acc; a.planeStride = ((int64_t)N * N + N) / 2;
+  a.N = N; a.nT = (N + TILE - 1) / TILE; a.tileCount = a.nT * (a.nT + 1) / 2; a.K = K; a.groupCount = 0;
+}
+
+struct GroupBuilder {
+  GramArgs a; int pairs = 0; int epi; int maxProducts; hipStream_t stream; hipError_t err = hipSuccess;
+  GroupBuilder(hipStream_t s, int epi_, int maxProducts_, const int8_t* panels, int64_t ldb, int32_t N, int32_t K, void* acc) : epi(epi_), maxProducts(maxProducts_), stream(s) { base_args(a, panels, ldb, N, K, acc); }
+  void flush() { if (a.groupCount > 0 && err == hipSuccess) { err = launch_gram(stream, a, epi, maxProducts); } a.groupCount = 0; pairs = 0; }
+  /* begins a group; flushes first when the tables are full */
+  GramGroup& begin(int npairs) {
+    if (a.groupCount == MAX_GROUPS || pairs + npairs > MAX_PAIRS) { flush(); }
+    GramGroup& g = a.groups[a.groupCount++]; g.pairBegin = (uint16_t)pairs; g.pairCount = 0; g.planeRe = g.planeIm = 0; g.m = 1; g.d = 0; g.c32 = 0; g.mulRe = g.mulIm = 0; return g;
+  }
+  void pair(GramGroup& g, int lanePanel, int aPanel) { a.pairs[pairs] = (uint32_t)lanePanel | ((uint32_t)aPanel << 16); ++pairs; ++g.pairCount; }
+};
+
+void set_mod(GramGroup& g, uint32_t m) { g.m = m; g.d = (uint32_t)(0x100000000ull / m); g.c32 = (uint32_t)(0x100000000ull % m); }
+
+hipError_t zero_fill(hipStream_t stream, void* p, size_t bytes) {
+  const int64_t n16 = (int64_t)((bytes + 15) / 16); if (n16 == 0) { return hipSuccess; }
+  fill_zero_kernel<<<(uint32_t)((n16 + 255) / 256), 256, 0, stream>>>(reinterpret_cast<uint4*>(p), n16); return hipGetLastError();
+}
+
+}  // namespace
+
+extern "C" int hykGramProfile(int32_t enable) {
+  for (Timed& t : g_timed) { (void)hipEventDestroy(t.start); (void)hipEventDestroy(t.stop); } g_timed.clear(); g_profile = enable != 0; return 0;
+}
+
+/* total milliseconds and number of contraction-kernel launches since hykGramProfile(1); waits for them to finish */
+extern "C" int hykGramProfileRead(double* totalMs, int32_t* launches) {
+  double sum = 0.; for (Timed& t : g_timed) { if (hipEventSynchronize(t.stop) != hipSuccess) { return -3; } float ms = 0.f; if (hipEventElapsedTime(&ms, t.start, t.stop) != hipSuccess) { return -3; } sum += ms; }
+  if (totalMs) { *totalMs = sum; } if (launches) { *launches = (int32_t)g_timed.size(); } return 0;
+}
+
+extern "C" int hykGramSetSlab(int32_t bk) { if (bk != 64 && bk != 128) { return -1; } g_bk = bk; return 0; }
+
+extern "C" size_t hykGramWorkspaceBytes(int32_t kind, int32_t Complex, int32_t N, int32_t orderA) {
+  if (N <= 0 || orderA <= 0) { return 0; }
+  const size_t T = ((size_t)N * (size_t)N + (size_t)N) / 2, planes = (size_t)(Complex ? 2 : 1);
+  size_t bytes = (kind == HYK_GRAM_LIMBS) ? planes * (size_t)(2 * orderA - 1) * T * 8 : planes * (size_t)orderA * T * 4;
+  return (bytes + 255) / 256 * 256;
+}
+
+/* Workspace must be zero on entry (hykGramWorkspaceClear) and is zero again on return. */
+extern "C" int hykGramWorkspaceClear(hipStream_t stream, void* workspace, size_t bytes) { return zero_fill(stream, workspace, bytes) == hipSuccess ? 0 : -3; }
+
+extern "C" int hykGramCrt(hipStream_t stream, int32_t Complex, int32_t N, int32_t orderA, const int8_t* panels, int64_t ldb, int32_t K, int32_t beta, int32_t orderC, uint64_t* C, void* workspace) {
+  if (N <= 0) { return 0; }
+  if (orderA < 1 || orderA > (Complex ? HYK_CRT_CPLX_COUNT : HYK_CRT_REAL_COUNT) || orderC < 1 || orderC > 3 || K <= 0 || (K & 127) || ldb < K || (ldb & 15) || ((uintptr_t)panels & 15)) { return -1; }
+  /* 131072 products per int32: residues of every modulus but 256 are at most 125 in magnitude, and mod 256 a wrap is harmless */
+  GroupBuilder gb(stream, EPI_MOD, 131072, panels, ldb, N, K, workspace);
+  ReconTable tab; tab.order = orderA;
+  if (!Complex) {
+    for (int x = 0; x < orderA; ++x) { GramGroup& g = gb.begin(1); set_mod(g, hyk_crt_real_mo[x]); g.mulRe = 1; g.planeRe = (uint16_t)x; gb.pair(g, x, x); }
+    for (int x = 0; x < orderA; ++x) { tab.m[x] = hyk_crt_real_mo[x]; tab.d[x] = (uint32_t)(0x100000000ull / tab.m[x]); tab.minv[x] = hyk_crt_real_minv[orderA - 1][x]; for (int k = 0; k < 3; ++k) { tab.Pd[x][k] = hyk_crt_real_Pd[orderA - 1][x][k]; } }
+    for (int k = 0; k < 3; ++k) { tab.P[k] = hyk_crt_real_P[orderA - 1][k]; }
+  } else {
+    const int rot = orderA < HYK_CRT_CPLX_SPLIT ? orderA : HYK_CRT_CPLX_SPLIT;
+    for (int x = 0; x < rot; ++x) {
+      /* W = P^T Q: elements on or above the diagonal are p = Re + i Im, the transposed ones q = Re - i Im (mod m);
+       * Re = (p + q)/2, Im = (p - q)/(2 i).  On the diagonal both groups contribute: Re gets p, Im gets 0. */
+      const uint32_t m = hyk_crt_cplx_mo[x], inv2 = (m + 1) / 2, iminv = hyk_crt_cplx_iminv[x];
+      GramGroup& g0 = gb.begin(1); set_mod(g0, m); g0.mulRe = inv2; g0.mulIm = iminv; g0.planeRe = (uint16_t)x; g0.planeIm = (uint16_t)(orderA + x); gb.pair(g0, 2 * x, 2 * x + 1);
+      GramGroup& g1 = gb.begin(1); set_mod(g1, m); g1.mulRe = inv2; g1.mulIm = m - iminv; g1.planeRe = (uint16_t)x; g1.planeIm = (uint16_t)(orderA + x); gb.pair(g1, 2 * x + 1, 2 * x);
+    }
+    for (int x = HYK_CRT_CPLX_SPLIT; x < orderA; ++x) {
+      /* 3M scheme mod m: Re = S^T S - (R^T I + I^T R), Im = R^T I - I^T R with S = R + I */
+      const uint32_t m = hyk_crt_cplx_mo[x]; const int base = 2 * HYK_CRT_CPLX_SPLIT + 3 * (x - HYK_CRT_CPLX_SPLIT);
+      GramGroup& gs = gb.begin(1); set_mod(gs, m); gs.mulRe = 1; gs.planeRe = (uint16_t)x; gb.pair(gs, base, base);
+      GramGroup& g0 = gb.begin(1); set_mod(g0, m); g0.mulRe = m - 1; g0.mulIm = 1; g0.planeRe = (uint16_t)x; g0.planeIm = (uint16_t)(orderA + x); gb.pair(g0, base + 1, base + 2);
+      GramGroup& g1 = gb.begin(1); set_mod(g1, m); g1.mulRe = m - 1; g1.mulIm = m - 1; g1.planeRe = (uint16_t)x; g1.planeIm = (uint16_t)(orderA + x); gb.pair(g1, base + 2, base + 1);
+    }
+    for (int x = 0; x < orderA; ++x) { tab.m[x] = hyk_crt_cplx_mo[x]; tab.d[x] = (uint32_t)(0x100000000ull / tab.m[x]); tab.minv[x] = hyk_crt_cplx_minv[orderA - 1][x]; for (int k = 0; k < 3; ++k) { tab.Pd[x][k] = hyk_crt_cplx_Pd[orderA - 1][x][k]; } }
+    for (int k = 0; k < 3; ++k) { tab.P[k] = hyk_crt_cplx_P[orderA - 1][k]; }
+  }
+  gb.flush(); if (gb.err != hipSuccess) { return -3; }
+  const int64_t T = ((int64_t)N * N + N) / 2; dim3 grid((uint32_t)((T + 255) / 256), Complex ? 2u : 1u);
+  crt_reconstruct_kernel<<<grid, 256, 0, stream>>>(tab, T, reinterpret_cast<uint32_t*>(workspace), T, beta, orderC, C, 1);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+extern "C" int hykGramLimbs(hipStream_t stream, int32_t Complex, int32_t N, int32_t orderA, const int8_t* panels, int64_t ldb, int32_t K, int32_t beta, int32_t orderC, uint64_t* C, void* workspace) {
+  if (N <= 0) { return 0; }
+  if (orderA < 1 || orderA > 12 || orderC < 1 || orderC > 3 || K <= 0 || (K & 127) || ldb < K || (ldb & 15) || ((uintptr_t)panels & 15)) { return -1; }
+  const int levels = 2 * orderA - 1;
+  /* 131071 products of magnitude <= 2^14 fit an int32 */
+  GroupBuilder gb(stream, EPI_I64, 131071, panels, ldb, N, K, workspace);
+  /* heaviest levels first so the tail of the launch is made of short items */
+  for (int cnt = orderA; cnt >= 1; --cnt) for (int s = 0; s < levels; ++s) {
+    const int lo = s < orderA ? 0 : s - orderA + 1, hi = s < orderA ? s : orderA - 1; if (hi - lo + 1 != cnt) { continue; }
+    /* digits group 0 (real input: the only one; complex input: re + im): T_s = sum_{i+j=s} A_i^T A_j, upper triangle */
+    GramGroup& g = gb.begin(cnt); g.mulRe = 1; g.planeRe = (uint16_t)s; for (int i = lo; i <= hi; ++i) { gb.pair(g, i, s - i); }
+    if (Complex) {
+      /* X_s = sum_{i+j=s} R_i^T I_j: Re -= X[y,x] + X[x,y], Im += X[y,x] - X[x,y] (3M scheme) */
+      GramGroup& g0 = gb.begin(cnt); g0.mulRe = 2; g0.mulIm = 1; g0.planeRe = (uint16_t)s; g0.planeIm = (uint16_t)(levels + s); for (int i = lo; i <= hi; ++i) { gb.pair(g0, orderA + i, 2 * orderA + (s - i)); }
+      GramGroup& g1 = gb.begin(cnt); g1.mulRe = 2; g1.mulIm = 2; g1.planeRe = (uint16_t)s; g1.planeIm = (uint16_t)(levels + s); for (int i = lo; i <= hi; ++i) { gb.pair(g1, 2 * orderA + (s - i), orderA + i); }
+    }
+  }
+  gb.flush(); if (gb.err != hipSuccess) { return -3; }
+  const int64_t T = ((int64_t)N * N + N) / 2; dim3 grid((uint32_t)((T + 255) / 256), Complex ? 2u : 1u);
+  limb_combine_kernel<<<grid, 256, 0, stream>>>(T, levels, reinterpret_cast<unsigned long long*>(workspace), T, beta, orderC, C, 1);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}

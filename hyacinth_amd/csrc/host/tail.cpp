@@ -1,0 +1,109 @@
+/*
+ * tail.cpp -- hyacinXGevd (truncated SVD from the Gram matrix) and hyacinXGinterp
+ * (interpolative decomposition from the Gram matrix).
+ *
+ * Mirrors the reference's src/gram_evd.cu:94-194 (tsvd, find_srank_kernel, hyacinXGevd) and
+ * src/gram_id.cpp:28-101 (interp, hyacinXGinterp).  The factorization itself runs in the HIP kernels of
+ * potrfp.hip and tail.hip; no vendor solver is involved.  Differences that are visible to a caller:
+ *  - an FP32 Gram is widened to FP64 before the Cholesky (the reference factors it in FP32);
+ *  - the SVD always runs in FP64, also for FP32 / FP16 storage (the reference uses FP32 there);
+ *  - JacobiSVDSweeps == 0 (the reference's "bidiagonalization backend") runs Jacobi to convergence.
+ * G is left untouched (the reference overwrites it with the factor).
+ */
+#include <numeric>
+#include <cfloat>
+#include "common.hpp"
+
+namespace {
+
+double storage_eps(int Atype) { return (Atype == HYACIN_F64 || Atype == HYACIN_F64_COMPLEX) ? DBL_EPSILON : (double)FLT_EPSILON; }
+int factor_type(int Gtype) { const int c = Gtype & 1; return ((Gtype & ~1) == HYACIN_DD ? HYACIN_DD : HYACIN_F64) + c; }
+
+struct Factor {
+  hyh::Scratch widened, Rt, work; const void* G; int64_t ldg; int type; int32_t ldr; size_t rtBytes;
+  Factor(const hyacinHandle_t* h, int32_t N, int32_t Kmax, int Gtype, const void* Gin, int64_t ldgIn)
+    : widened(h, ((Gtype & ~1) == HYACIN_F32) ? (size_t)N * N * 8 * (1 + (Gtype & 1)) : 0),
+      Rt(h, (size_t)N * (size_t)std::min(N, Kmax + 1) * (size_t)hyh::elem_bytes(factor_type(Gtype))),
+      work(h, hykPotrfpWorkspaceBytes(N, factor_type(Gtype))) {
+    type = factor_type(Gtype); ldr = std::min(N, Kmax + 1); rtBytes = (size_t)N * ldr * hyh::elem_bytes(type); G = Gin; ldg = ldgIn;
+    if (widened.p) { HYH_KERNEL(hykMatcopy(h->hipStream, 'A', N, N, Gtype, Gin, ldgIn, HYACIN_F64 + (Gtype & 1), widened.p, N)); G = widened.p; ldg = N; }
+    HYH_KERNEL(hykGramWorkspaceClear(h->hipStream, Rt.p, rtBytes));
+  }
+};
+
+const char* type_tag(int t) { switch (t) { case HYACIN_F64: return "FP64"; case HYACIN_F64_COMPLEX: return "FP64-COMPLEX"; case HYACIN_DD: return "FP128-DD"; default: return "FP128-DD-COMPLEX"; } }
+
+int32_t run_potrfp(const hyacinHandle_t* h, Factor& f, double eps, int32_t K, int32_t N, int32_t* jpiv) {
+  int32_t* word = (int32_t*)h->pinnedWorkspace; *word = 0;
+  HYH_KERNEL(hykPotrfp(h->hipStream, h->DeviceSMs, eps, K, N, f.type, f.G, f.ldg, f.Rt.p, f.ldr, jpiv, f.work.p, word));
+  HYH_CHECK(hipStreamSynchronize(h->hipStream));
+  const int32_t rank = *word;
+  if (h->logger) { std::fprintf((FILE*)h->logger, "POTRFP-%s [eps=%.1le] [N=%d] [K=%d] [Cholesky-rank=%d]\n", type_tag(f.type), eps, N, K, rank); }
+  return rank;
+}
+
+}  // namespace
+
+extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t N, int32_t K, hyacinPrecision_t Atype, void* X, int32_t ldx, void* S, hyacinPrecision_t Gtype, void* G, int32_t ldg) {
+  if (N <= 0) { return 0; }
+  K = K <= 0 ? N : std::min(N, K);
+  if ((int)Atype < 0 || (int)Atype > HYACIN_F16_COMPLEX || ((int)Atype & 1) != ((int)Gtype & 1)) { return 0; }
+  const int gbase = (int)Gtype & ~1; if (gbase != HYACIN_F64 && gbase != HYACIN_F32 && gbase != HYACIN_DD) { return 0; }
+  hipStream_t s = handle->hipStream; hyh::timer_mark(handle, hyh::Segment::rep_kernel);
+  const int32_t lrqr = handle->QRCPTruncateRank, jac = std::abs(handle->JacobiSVDSweeps), bid = std::abs(std::min(0, handle->JacobiSVDSweeps));
+  const int32_t sweeps = lrqr ? jac : bid;   /* FP64-capable device: the same rule for every storage type (src/gram_evd.cu:148-150) */
+  const int Complex = (int)Atype & 1; const double machineEps = storage_eps((int)Atype);
+  eps = std::min(std::max(std::fabs(eps), machineEps), 1.);
+
+  hyh::Scratch jpiv(handle, sizeof(int32_t) * (size_t)N);
+  int32_t rank;
+  { Factor f(handle, N, N, (int)Gtype, G, ldg);
+    rank = run_potrfp(handle, f, lrqr ? eps : 0., N, N, jpiv.as<int32_t>());
+    if (rank <= 0) { return rank; }
+    /* B = (R P^T)^H, N x rank, FP64 */
+    hyh::Scratch B(handle, (size_t)N * rank * 8 * (1 + Complex)), sigma(handle, sizeof(double) * (size_t)rank), counter(handle, 64);
+    HYH_KERNEL(hykFactorToB(s, N, rank, f.type, f.Rt.p, f.ldr, B.as<double>()));
+    const int32_t maxSweeps = sweeps > 0 ? sweeps : 30; int32_t used = 0;
+    for (int32_t sw = 0; sw < maxSweeps && rank > 1; ++sw) {
+      HYH_KERNEL(hykGramWorkspaceClear(s, counter.p, 64));
+      HYH_KERNEL(hykJacobiSweep(s, Complex, N, rank, B.as<double>(), machineEps, counter.as<int32_t>())); ++used;
+      int32_t rotations = 0; HYH_CHECK(hipMemcpyAsync(&rotations, counter.p, sizeof(int32_t), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
+      if (rotations == 0) { break; }
+    }
+    HYH_KERNEL(hykColumnNorms(s, Complex, N, rank, B.as<double>(), sigma.as<double>()));
+    std::vector<double> sig((size_t)rank); HYH_CHECK(hipMemcpyAsync(sig.data(), sigma.p, sizeof(double) * (size_t)rank, hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
+    std::vector<int32_t> order((size_t)rank); std::iota(order.begin(), order.end(), 0);
+    std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return sig[a] > sig[b]; });
+    /* rank cut (reference: find_srank_kernel, src/gram_evd.cu:44-70): keep i < K while sum_{j>=i} sigma_j^2 > eps^2 sum_j sigma_j^2 */
+    std::vector<double> suffix((size_t)rank + 1, 0.); for (int32_t i = rank - 1; i >= 0; --i) { const double v = sig[order[i]]; suffix[i] = std::fma(v, v, suffix[i + 1]); }
+    const double resid = eps * eps * suffix[0]; std::vector<double> Sout((size_t)K, 0.); int32_t kept = 0;
+    for (int32_t i = 0; i < K; ++i) { if (i < rank && resid < suffix[i]) { Sout[i] = sig[order[i]]; ++kept; } }
+    const int32_t svdRank = kept; rank = std::min(rank, kept);
+    hyh::Scratch dS(handle, sizeof(double) * (size_t)K), dOrder(handle, sizeof(int32_t) * (size_t)std::max(1, rank));
+    HYH_CHECK(hipMemcpyAsync(dS.p, Sout.data(), sizeof(double) * (size_t)K, hipMemcpyHostToDevice, s));
+    if (rank > 0) { HYH_CHECK(hipMemcpyAsync(dOrder.p, order.data(), sizeof(int32_t) * (size_t)rank, hipMemcpyHostToDevice, s)); }
+    HYH_KERNEL(hykValuesOut(s, K, (int32_t)Atype, dS.as<double>(), S));
+    if (rank > 0) { HYH_KERNEL(hykBasisOut(s, N, rank, (int32_t)Atype, B.as<double>(), sigma.as<double>(), dOrder.as<int32_t>(), X, ldx)); }
+    HYH_CHECK(hipStreamSynchronize(s));   /* Sout / order are host temporaries */
+    if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ-%s [eps=%.1le] [M=%d] [N=%d] [K=%d] [sweeps=%d] [SVD-rank=%d]\n", Complex ? "FP64-COMPLEX" : "FP64", eps, N, rank, K, used, svdRank); }
+  }
+  return rank;
+}
+
+extern "C" int32_t hyacinXGinterp(const hyacinHandle_t* handle, double eps, int32_t N, int32_t K, hyacinPrecision_t Atype, void* X, int32_t ldx, int32_t* jpiv, hyacinPrecision_t Gtype, void* G, int32_t ldg) {
+  if (N <= 0) { return 0; }
+  K = K <= 0 ? N : std::min(N, K);
+  if ((int)Atype < 0 || (int)Atype > HYACIN_F16_COMPLEX || ((int)Atype & 1) != ((int)Gtype & 1)) { return 0; }
+  const int gbase = (int)Gtype & ~1; if (gbase != HYACIN_F64 && gbase != HYACIN_F32 && gbase != HYACIN_DD) { return 0; }
+  hipStream_t s = handle->hipStream; hyh::timer_mark(handle, hyh::Segment::rep_kernel);
+  const int Complex = (int)Atype & 1; eps = std::min(std::max(std::fabs(eps), storage_eps((int)Atype)), 1.);
+  Factor f(handle, N, K, (int)Gtype, G, ldg);
+  const int32_t rank = run_potrfp(handle, f, eps, K, N, jpiv);
+  if (rank <= 0) { return rank; }
+  if (rank >= N) { HYH_KERNEL(hykInterpOut(s, N, N, (int32_t)Atype, jpiv, nullptr, X, ldx)); return N; }
+  hyh::Scratch Rp(handle, (size_t)rank * N * 8 * (1 + Complex)), Tt(handle, (size_t)rank * (N - rank) * 8 * (1 + Complex));
+  HYH_KERNEL(hykInterpSolve(s, N, rank, f.type, f.Rt.p, f.ldr, jpiv, Rp.as<double>(), Tt.as<double>()));
+  HYH_KERNEL(hykInterpOut(s, N, rank, (int32_t)Atype, jpiv, Tt.as<double>(), X, ldx));
+  if (handle->logger) { std::fprintf((FILE*)handle->logger, "TRSM-LEFT-%s [M=%d] [N=%d]\n", Complex ? "FP64-COMPLEX" : "FP64", rank, N - rank); }
+  return rank;
+}

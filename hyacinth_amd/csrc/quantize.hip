@@ -1,0 +1,200 @@
+/*
+ * quantize.hip -- floating point -> int8 limb / CRT-residue panels (HBM-bound).
+ *
+ * Replaces the reference's src/quantize_limbs.cu, src/quantize_crt_real.cu and
+ * src/quantize_crt_complex.cu.  Every element x of column j becomes the integer
+ * q = RNE(x * 2^vexp[j]) (96-bit two's complement) and is written as
+ *   limbs:        balanced base-256 digits d_l in [-128, 127], q = sum d_l 256^l;
+ *                 complex writes three digit groups, of re + im, re and im;
+ *   CRT real:     q mod m_x, stored in int8 (values above 127 wrap by -m_x);
+ *   CRT complex:  moduli x < 20: (re - i_x im) mod m_x and (re + i_x im) mod m_x with i_x^2 = -1;
+ *                 moduli x >= 20: (re + im) mod m_x, re mod m_x, im mod m_x.
+ * A column with vexp[j] == INT_MAX is all zero.
+ *
+ * Output layout (same as the reference): panel p, column j, row k at
+ * B[p * N * ldb + j * ldb + k]; rows are the contraction dimension of the Gram
+ * kernel, so every MFMA operand fetch is a contiguous run of K.
+ *
+ * One thread quantizes four consecutive rows of one column and stores one
+ * packed dword per panel (byte stores when B + row is not 4-byte aligned).
+ */
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include "hyk_common.h"
+#include "crt_tables.h"
+#include "hyacin_kernels.h"
+
+namespace {
+
+constexpr int Q_THREADS = 256;
+constexpr int Q_ROWS = 4;
+
+/* loaders: element -> decomposed real / imaginary parts */
+struct ElemF64 { static constexpr int cplx = 0; using T = uint64_t; static __device__ __forceinline__ void load(const T* p, hyk::Dec& re, hyk::Dec& im) { re = hyk::decompose_f64(*p); im = hyk::Dec{ 0, 0, 0 }; } };
+struct ElemF32 { static constexpr int cplx = 0; using T = uint32_t; static __device__ __forceinline__ void load(const T* p, hyk::Dec& re, hyk::Dec& im) { re = hyk::decompose_f32(*p); im = hyk::Dec{ 0, 0, 0 }; } };
+struct ElemF16 { static constexpr int cplx = 0; using T = uint16_t; static __device__ __forceinline__ void load(const T* p, hyk::Dec& re, hyk::Dec& im) { re = hyk::decompose_f16(*p); im = hyk::Dec{ 0, 0, 0 }; } };
+struct ElemF64C { static constexpr int cplx = 1; using T = ulonglong2; static __device__ __forceinline__ void load(const T* p, hyk::Dec& re, hyk::Dec& im) { T v = *p; re = hyk::decompose_f64(v.x); im = hyk::decompose_f64(v.y); } };
+struct ElemF32C { static constexpr int cplx = 1; using T = uint2; static __device__ __forceinline__ void load(const T* p, hyk::Dec& re, hyk::Dec& im) { T v = *p; re = hyk::decompose_f32(v.x); im = hyk::decompose_f32(v.y); } };
+struct ElemF16C { static constexpr int cplx = 1; using T = uint32_t; static __device__ __forceinline__ void load(const T* p, hyk::Dec& re, hyk::Dec& im) { T v = *p; re = hyk::decompose_f16(v & 0xffffu); im = hyk::decompose_f16(v >> 16); } };
+
+__device__ __forceinline__ void store_panel(int8_t* dst, uint32_t packed, int valid, bool aligned) {
+  if (aligned && valid == Q_ROWS) { *reinterpret_cast<uint32_t*>(dst) = packed; }
+  else { for (int r = 0; r < valid; ++r) { dst[r] = (int8_t)(packed >> (8 * r)); } }
+}
+
+/* ------------------------------------------------------------------ limbs */
+template <typename E>
+__global__ __launch_bounds__(Q_THREADS) void quantize_limbs_kernel(int32_t M, int32_t order, const typename E::T* __restrict__ A, int64_t lda, const int32_t* __restrict__ vexp, int8_t* __restrict__ B, int64_t ldb, int64_t strideB) {
+  const int32_t j = blockIdx.y; const int64_t i0 = ((int64_t)blockIdx.x * Q_THREADS + threadIdx.x) * Q_ROWS;
+  if (i0 >= M) { return; }
+  const int valid = (M - i0) < Q_ROWS ? (int)(M - i0) : Q_ROWS; const int32_t expon = vexp[j];
+  int8_t* out = B + (int64_t)j * ldb + i0; const bool aligned = ((uintptr_t)out & 3u) == 0;
+  constexpr int GROUPS = E::cplx ? 3 : 1;
+  if (expon == HYK_INT_MAX) { for (int p = 0; p < order * GROUPS; ++p) { store_panel(out + p * strideB, 0u, valid, aligned); } return; }
+  hyk::I96 q[GROUPS][Q_ROWS];
+  #pragma unroll
+  for (int r = 0; r < Q_ROWS; ++r) {
+    hyk::Dec re{ 0, 0, 0 }, im{ 0, 0, 0 }; if (r < valid) { E::load(&A[(int64_t)j * lda + i0 + r], re, im); }
+    if constexpr (E::cplx) { hyk::I96 a = hyk::round_scaled(re, expon), b = hyk::round_scaled(im, expon); q[0][r] = hyk::i96_add(a, b); q[1][r] = a; q[2][r] = b; }
+    else { q[0][r] = hyk::round_scaled(re, expon); }
+  }
+  #pragma unroll
+  for (int g = 0; g < GROUPS; ++g) {
+    uint32_t carry[Q_ROWS] = { 0, 0, 0, 0 };
+    #pragma unroll
+    for (int l = 0; l < 12; ++l) {
+      if (l < order) {
+        uint32_t packed = 0;
+        #pragma unroll
+        for (int r = 0; r < Q_ROWS; ++r) { uint32_t t = hyk::i96_byte(q[g][r], l) + carry[r]; packed |= (t & 0xffu) << (8 * r); carry[r] = (t >> 8) + ((t >> 7) & 1u); }
+        store_panel(out + (int64_t)(g * order + l) * strideB, packed, valid, aligned);
+      }
+    }
+  }
+}
+
+/* ------------------------------------------------------------------ CRT */
+template <int X> struct RealMod { static constexpr hyk::Mod k = hyk::make_mod(hyk_crt_real_mo[X]); };
+template <int X> struct CplxMod { static constexpr hyk::Mod k = hyk::make_mod(hyk_crt_cplx_mo[X]); static constexpr uint32_t im = hyk_crt_cplx_im[X]; };
+
+template <typename E, int WORDS, int X>
+__device__ __forceinline__ void crt_real_step(int32_t order, const hyk::I96 (&q)[Q_ROWS], int8_t* out, int64_t strideB, int valid, bool aligned) {
+  if constexpr (X < HYK_CRT_REAL_COUNT) {
+    if (X < order) {
+      constexpr hyk::Mod k = RealMod<X>::k; uint32_t packed = 0;
+      #pragma unroll
+      for (int r = 0; r < Q_ROWS; ++r) { packed |= ((uint32_t)(uint8_t)hyk::residue_to_i8(hyk::reduce_i96<WORDS>(q[r], k), k.m)) << (8 * r); }
+      store_panel(out + (int64_t)X * strideB, packed, valid, aligned);
+      crt_real_step<E, WORDS, X + 1>(order, q, out, strideB, valid, aligned);
+    }
+  }
+}
+
+template <typename E, int WORDS>
+__global__ __launch_bounds__(Q_THREADS) void quantize_crt_real_kernel(int32_t M, int32_t order, const typename E::T* __restrict__ A, int64_t lda, const int32_t* __restrict__ vexp, int8_t* __restrict__ B, int64_t ldb, int64_t strideB) {
+  const int32_t j = blockIdx.y; const int64_t i0 = ((int64_t)blockIdx.x * Q_THREADS + threadIdx.x) * Q_ROWS;
+  if (i0 >= M) { return; }
+  const int valid = (M - i0) < Q_ROWS ? (int)(M - i0) : Q_ROWS; const int32_t expon = vexp[j];
+  int8_t* out = B + (int64_t)j * ldb + i0; const bool aligned = ((uintptr_t)out & 3u) == 0;
+  if (expon == HYK_INT_MAX) { for (int p = 0; p < order; ++p) { store_panel(out + p * strideB, 0u, valid, aligned); } return; }
+  hyk::I96 q[Q_ROWS];
+  #pragma unroll
+  for (int r = 0; r < Q_ROWS; ++r) { hyk::Dec re{ 0, 0, 0 }, im{ 0, 0, 0 }; if (r < valid) { E::load(&A[(int64_t)j * lda + i0 + r], re, im); } q[r] = hyk::round_scaled(re, expon); }
+  crt_real_step<E, WORDS, 0>(order, q, out, strideB, valid, aligned);
+}
+
+template <typename E, int WORDS, int X>
+__device__ __forceinline__ void crt_cplx_step(int32_t order, const hyk::I96 (&qr)[Q_ROWS], const hyk::I96 (&qi)[Q_ROWS], int8_t* out, int64_t strideB, int valid, bool aligned) {
+  if constexpr (X < HYK_CRT_CPLX_COUNT) {
+    if (X < order) {
+      constexpr hyk::Mod k = CplxMod<X>::k; constexpr uint32_t im = CplxMod<X>::im; uint32_t p0 = 0, p1 = 0, p2 = 0;
+      #pragma unroll
+      for (int r = 0; r < Q_ROWS; ++r) {
+        uint32_t a = hyk::reduce_i96<WORDS>(qr[r], k), b = hyk::reduce_i96<WORDS>(qi[r], k);
+        if constexpr (X < HYK_CRT_CPLX_SPLIT) {
+          uint32_t p = hyk::reduce_u32(a + (k.m - im) * b, k.m, k.d), q = hyk::reduce_u32(a + im * b, k.m, k.d);
+          p0 |= ((uint32_t)(uint8_t)hyk::residue_to_i8(p, k.m)) << (8 * r); p1 |= ((uint32_t)(uint8_t)hyk::residue_to_i8(q, k.m)) << (8 * r);
+        } else {
+          uint32_t s = a + b; s = s >= k.m ? s - k.m : s;
+          p0 |= ((uint32_t)(uint8_t)hyk::residue_to_i8(s, k.m)) << (8 * r); p1 |= ((uint32_t)(uint8_t)hyk::residue_to_i8(a, k.m)) << (8 * r); p2 |= ((uint32_t)(uint8_t)hyk::residue_to_i8(b, k.m)) << (8 * r);
+        }
+      }
+      if constexpr (X < HYK_CRT_CPLX_SPLIT) {
+        store_panel(out + (int64_t)(2 * X) * strideB, p0, valid, aligned); store_panel(out + (int64_t)(2 * X + 1) * strideB, p1, valid, aligned);
+      } else {
+        constexpr int base = 2 * HYK_CRT_CPLX_SPLIT + 3 * (X - HYK_CRT_CPLX_SPLIT);
+        store_panel(out + (int64_t)base * strideB, p0, valid, aligned); store_panel(out + (int64_t)(base + 1) * strideB, p1, valid, aligned); store_panel(out + (int64_t)(base + 2) * strideB, p2, valid, aligned);
+      }
+      crt_cplx_step<E, WORDS, X + 1>(order, qr, qi, out, strideB, valid, aligned);
+    }
+  }
+}
+
+template <typename E, int WORDS>
+__global__ __launch_bounds__(Q_THREADS) void quantize_crt_cplx_kernel(int32_t M, int32_t order, const typename E::T* __restrict__ A, int64_t lda, const int32_t* __restrict__ vexp, int8_t* __restrict__ B, int64_t ldb, int64_t strideB) {
+  const int32_t j = blockIdx.y; const int64_t i0 = ((int64_t)blockIdx.x * Q_THREADS + threadIdx.x) * Q_ROWS;
+  if (i0 >= M) { return; }
+  const int valid = (M - i0) < Q_ROWS ? (int)(M - i0) : Q_ROWS; const int32_t expon = vexp[j];
+  int8_t* out = B + (int64_t)j * ldb + i0; const bool aligned = ((uintptr_t)out & 3u) == 0;
+  const int panels = order <= HYK_CRT_CPLX_SPLIT ? 2 * order : 3 * order - HYK_CRT_CPLX_SPLIT;
+  if (expon == HYK_INT_MAX) { for (int p = 0; p < panels; ++p) { store_panel(out + p * strideB, 0u, valid, aligned); } return; }
+  hyk::I96 qr[Q_ROWS], qi[Q_ROWS];
+  #pragma unroll
+  for (int r = 0; r < Q_ROWS; ++r) { hyk::Dec re{ 0, 0, 0 }, im{ 0, 0, 0 }; if (r < valid) { E::load(&A[(int64_t)j * lda + i0 + r], re, im); } qr[r] = hyk::round_scaled(re, expon); qi[r] = hyk::round_scaled(im, expon); }
+  crt_cplx_step<E, WORDS, 0>(order, qr, qi, out, strideB, valid, aligned);
+}
+
+/* rows [row0, row1) of `panels` panels set to zero: the Gram kernel contracts over whole 128-row blocks */
+__global__ void zero_rows_kernel(int8_t* __restrict__ B, int64_t ldb, int64_t cols, int32_t row0, int32_t row1) {
+  const int64_t c = blockIdx.x; const int32_t len = row1 - row0; int8_t* p = B + c * ldb + row0;
+  for (int32_t i = threadIdx.x; i < len; i += blockDim.x) { p[i] = 0; }
+  (void)cols;
+}
+
+}  // namespace
+
+#define HYK_QGRID dim3 grid((uint32_t)((M + Q_THREADS * Q_ROWS - 1) / (Q_THREADS * Q_ROWS)), (uint32_t)N)
+
+extern "C" int hykQuantizeLimbs(hipStream_t stream, int32_t M, int32_t N, int32_t orderA, int32_t Atype, const void* A, int64_t lda, const int32_t* vexp, int8_t* B, int64_t ldb) {
+  if (M <= 0 || N <= 0) { return 0; }
+  if (orderA < 1 || orderA > 12 || N > 65535 || ldb < M) { return -1; }
+  const int64_t strideB = (int64_t)N * ldb; HYK_QGRID;
+  switch (Atype) {
+    case HYK_F64: quantize_limbs_kernel<ElemF64><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const uint64_t*)A, lda, vexp, B, ldb, strideB); break;
+    case HYK_F32: quantize_limbs_kernel<ElemF32><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const uint32_t*)A, lda, vexp, B, ldb, strideB); break;
+    case HYK_F16: quantize_limbs_kernel<ElemF16><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const uint16_t*)A, lda, vexp, B, ldb, strideB); break;
+    case HYK_F64C: quantize_limbs_kernel<ElemF64C><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const ulonglong2*)A, lda, vexp, B, ldb, strideB); break;
+    case HYK_F32C: quantize_limbs_kernel<ElemF32C><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const uint2*)A, lda, vexp, B, ldb, strideB); break;
+    case HYK_F16C: quantize_limbs_kernel<ElemF16C><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const uint32_t*)A, lda, vexp, B, ldb, strideB); break;
+    default: return -1;
+  }
+  return 0;
+}
+
+/* maxBits: an upper bound on the bit length of |q| (u + 1 covers re + im as well); <= 0 means unknown */
+extern "C" int hykQuantizeCrt(hipStream_t stream, int32_t M, int32_t N, int32_t orderA, int32_t Atype, const void* A, int64_t lda, const int32_t* vexp, int8_t* B, int64_t ldb, int32_t maxBits) {
+  if (M <= 0 || N <= 0) { return 0; }
+  const int cplx = Atype & 1;
+  if (orderA < 1 || orderA > (cplx ? HYK_CRT_CPLX_COUNT : HYK_CRT_REAL_COUNT) || N > 65535 || ldb < M) { return -1; }
+  const int64_t strideB = (int64_t)N * ldb; HYK_QGRID; const bool narrow = (0 < maxBits && maxBits <= 48);
+  #define HYK_LAUNCH_CRT(KERNEL, ELEM, TYPE) \
+    if (narrow) { KERNEL<ELEM, 3><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const TYPE*)A, lda, vexp, B, ldb, strideB); } \
+    else { KERNEL<ELEM, 6><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const TYPE*)A, lda, vexp, B, ldb, strideB); }
+  switch (Atype) {
+    case HYK_F64: HYK_LAUNCH_CRT(quantize_crt_real_kernel, ElemF64, uint64_t) break;
+    case HYK_F32: HYK_LAUNCH_CRT(quantize_crt_real_kernel, ElemF32, uint32_t) break;
+    case HYK_F16: HYK_LAUNCH_CRT(quantize_crt_real_kernel, ElemF16, uint16_t) break;
+    case HYK_F64C: HYK_LAUNCH_CRT(quantize_crt_cplx_kernel, ElemF64C, ulonglong2) break;
+    case HYK_F32C: HYK_LAUNCH_CRT(quantize_crt_cplx_kernel, ElemF32C, uint2) break;
+    case HYK_F16C: HYK_LAUNCH_CRT(quantize_crt_cplx_kernel, ElemF16C, uint32_t) break;
+    default: return -1;
+  }
+  #undef HYK_LAUNCH_CRT
+  return 0;
+}
+
+extern "C" int hykZeroRows(hipStream_t stream, int8_t* B, int64_t ldb, int64_t cols, int32_t row0, int32_t row1) {
+  if (cols <= 0 || row1 <= row0) { return 0; }
+  if (cols > 2147483647ll) { return -1; }
+  zero_rows_kernel<<<(uint32_t)cols, 128, 0, stream>>>(B, ldb, cols, row0, row1); return 0;
+}

@@ -1,0 +1,237 @@
+/*
+ * tail.hip -- the small N x N tail after the pivoted Cholesky: SVD of the
+ * Cholesky factor (truncated-SVD fit) and the triangular solve + scatter of the
+ * interpolative decomposition.
+ *
+ * Replaces, in the reference, the cuSOLVER gesvdj / gesvd call and
+ * find_srank_kernel of src/gram_evd.cu:44-142, the cuBLAS trsm of
+ * src/gram_id.cpp:8-15,45 and the pivot-scatter modes of src/matcopy.cu:48-52.
+ *
+ * SVD: one-sided (Hestenes) Jacobi on B = (R P^T)^H, N x r, in FP64.  After the
+ * pivoted Cholesky the columns of B are already graded, which is the
+ * preconditioning under which a few sweeps reach machine precision (the
+ * reference caps its Jacobi at 3 sweeps for the same reason).  Rounds follow
+ * the round-robin tournament, so the r/2 column pairs of a round are disjoint:
+ * one workgroup per pair, one launch per round.  Column j of the result has
+ * norm sigma_j and direction u_j; the right basis of op(A) is V = U.
+ *
+ * R arrives column-wise: Rt[c * ldr + k] = R[k, c] for physical column c.
+ */
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include "hyk_common.h"
+#include "hyacin_kernels.h"
+
+namespace {
+
+constexpr int T_THREADS = 256;
+
+__device__ __forceinline__ double block_sum(double v, double* scratch) {
+  for (int off = 32; off > 0; off >>= 1) { v += __shfl_xor(v, off, 64); }
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) { scratch[threadIdx.x >> 6] = v; }
+  __syncthreads();
+  double s = 0.; for (int w = 0; w < T_THREADS / 64; ++w) { s += scratch[w]; }
+  return s;
+}
+
+/* B[c + k*N] = conj(R[k, c]) from the (possibly double-double) column-wise factor; WE doubles per element, WR per real part */
+template <bool CPLX>
+__global__ void factor_to_b_kernel(int32_t N, int32_t rank, const double* __restrict__ Rt, int32_t ldr, int WE, int WR, double* __restrict__ B) {
+  const int c = blockIdx.x * T_THREADS + threadIdx.x, k = blockIdx.y; if (c >= N) { return; }
+  const double* src = &Rt[((int64_t)c * ldr + k) * WE];
+  if constexpr (CPLX) { B[2 * ((int64_t)c + (int64_t)k * N)] = src[0]; B[2 * ((int64_t)c + (int64_t)k * N) + 1] = -src[WR]; } else { B[(int64_t)c + (int64_t)k * N] = src[0]; }
+}
+
+template <bool CPLX>
+__global__ __launch_bounds__(T_THREADS) void jacobi_round_kernel(int32_t N, int32_t n, int32_t r, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations) {
+  __shared__ double scratch[T_THREADS / 64];
+  const int i = blockIdx.x; int p, q;
+  if (i == 0) { p = n - 1; q = round; } else { p = (round + i) % (n - 1); q = (round - i + (n - 1)) % (n - 1); }
+  if (p >= r || q >= r) { return; }
+  if (p > q) { int t = p; p = q; q = t; }
+  constexpr int W = CPLX ? 2 : 1;
+  double* bp = &B[(int64_t)p * N * W]; double* bq = &B[(int64_t)q * N * W];
+  double alpha = 0., beta = 0., gre = 0., gim = 0.;
+  for (int k = threadIdx.x; k < N; k += T_THREADS) {
+    if constexpr (CPLX) {
+      const double pr = bp[2 * k], pi = bp[2 * k + 1], qr = bq[2 * k], qi = bq[2 * k + 1];
+      alpha += pr * pr + pi * pi; beta += qr * qr + qi * qi; gre += pr * qr + pi * qi; gim += pr * qi - pi * qr;   /* conj(p) q */
+    } else { const double pv = bp[k], qv = bq[k]; alpha += pv * pv; beta += qv * qv; gre += pv * qv; }
+  }
+  alpha = block_sum(alpha, scratch); beta = block_sum(beta, scratch); gre = block_sum(gre, scratch); if constexpr (CPLX) { gim = block_sum(gim, scratch); }
+  const double g2 = gre * gre + gim * gim;
+  if (!(g2 > tol * tol * alpha * beta) || !(g2 > 0.)) { return; }
+  const double gabs = sqrt(g2), zeta = (beta - alpha) / (2. * gabs);
+  const double t = (zeta >= 0. ? 1. : -1.) / (fabs(zeta) + sqrt(1. + zeta * zeta)), cs = 1. / sqrt(1. + t * t), sn = cs * t;
+  const double er = gre / gabs, ei = gim / gabs;   /* e^{i phi}; column q is first multiplied by e^{-i phi} so that the cross term is real */
+  for (int k = threadIdx.x; k < N; k += T_THREADS) {
+    if constexpr (CPLX) {
+      const double pr = bp[2 * k], pi = bp[2 * k + 1], q0 = bq[2 * k], q1 = bq[2 * k + 1];
+      const double qr = q0 * er + q1 * ei, qi = q1 * er - q0 * ei;
+      bp[2 * k] = cs * pr - sn * qr; bp[2 * k + 1] = cs * pi - sn * qi; bq[2 * k] = sn * pr + cs * qr; bq[2 * k + 1] = sn * pi + cs * qi;
+    } else { const double pv = bp[k], qv = bq[k] * er; bp[k] = cs * pv - sn * qv; bq[k] = sn * pv + cs * qv; }
+  }
+  if (threadIdx.x == 0) { atomicAdd(rotations, 1); }
+}
+
+template <bool CPLX>
+__global__ __launch_bounds__(T_THREADS) void column_norm_kernel(int32_t N, const double* __restrict__ B, double* __restrict__ sigma) {
+  __shared__ double scratch[T_THREADS / 64]; constexpr int W = CPLX ? 2 : 1;
+  const double* b = &B[(int64_t)blockIdx.x * N * W]; double s = 0.;
+  for (int k = threadIdx.x; k < N * W; k += T_THREADS) { s += b[k] * b[k]; }
+  s = block_sum(s, scratch); if (threadIdx.x == 0) { sigma[blockIdx.x] = sqrt(s); }
+}
+
+template <typename T> __device__ __forceinline__ void store_real(T* p, double v);
+template <> __device__ __forceinline__ void store_real<double>(double* p, double v) { *p = v; }
+template <> __device__ __forceinline__ void store_real<float>(float* p, double v) { *p = (float)v; }
+template <> __device__ __forceinline__ void store_real<__half>(__half* p, double v) { __half_raw r; r.data = static_cast<_Float16>(v); *p = r; }
+
+/* X[:, j] = B[:, order[j]] / sigma[order[j]] converted to the storage type, j < rank */
+template <typename T, bool CPLX>
+__global__ void basis_out_kernel(int32_t N, const double* __restrict__ B, const double* __restrict__ sigma, const int32_t* __restrict__ order, T* __restrict__ X, int64_t ldx) {
+  const int k = blockIdx.x * T_THREADS + threadIdx.x, j = blockIdx.y; if (k >= N) { return; }
+  const int src = order[j]; const double s = sigma[src], inv = s > 0. ? 1. / s : 0.;
+  if constexpr (CPLX) { const double* b = &B[2 * ((int64_t)src * N + k)]; T* x = &X[2 * ((int64_t)j * ldx + k)]; store_real<T>(x, b[0] * inv); store_real<T>(x + 1, b[1] * inv); }
+  else { store_real<T>(&X[(int64_t)j * ldx + k], B[(int64_t)src * N + k] * inv); }
+}
+
+/* column j <- column j / sigma_j in place (a zero column stays zero) */
+__global__ void normalize_columns_kernel(int32_t N, int W, double* B, const double* sigma) {
+  const int k = blockIdx.x * T_THREADS + threadIdx.x, j = blockIdx.y; if (k >= N * W) { return; }
+  const double s = sigma[j]; B[(int64_t)j * N * W + k] *= (s > 0. ? 1. / s : 0.);
+}
+
+template <typename T> __global__ void values_out_kernel(int32_t K, const double* __restrict__ S, T* __restrict__ out) { const int i = blockIdx.x * T_THREADS + threadIdx.x; if (i < K) { store_real<T>(&out[i], S[i]); } }
+
+/* Rp[k + x*K] = R[k, jpiv[x]-1] (high word), K x N upper trapezoid in pivot order */
+template <bool CPLX>
+__global__ void gather_factor_kernel(int32_t N, int32_t K, const double* __restrict__ Rt, int32_t ldr, int WE, int WR, const int32_t* __restrict__ jpiv, double* __restrict__ Rp) {
+  const int k = blockIdx.x * T_THREADS + threadIdx.x, x = blockIdx.y; if (k >= K) { return; }
+  const double* src = &Rt[((int64_t)(jpiv[x] - 1) * ldr + k) * WE]; const bool low = k > x;
+  if constexpr (CPLX) { Rp[2 * ((int64_t)k + (int64_t)x * K)] = low ? 0. : src[0]; Rp[2 * ((int64_t)k + (int64_t)x * K) + 1] = low ? 0. : src[WR]; } else { Rp[(int64_t)k + (int64_t)x * K] = low ? 0. : src[0]; }
+}
+
+/* back substitution R11 T = R12, one thread per right-hand side; Tt[col + i*ncols] = T[i, col] */
+template <bool CPLX>
+__global__ void upper_solve_kernel(int32_t K, int32_t ncols, const double* __restrict__ Rp, double* __restrict__ Tt) {
+  const int col = blockIdx.x * T_THREADS + threadIdx.x; if (col >= ncols) { return; }
+  constexpr int W = CPLX ? 2 : 1; const double* rhs = &Rp[(int64_t)(K + col) * K * W];
+  for (int i = K - 1; i >= 0; --i) {
+    double sr = rhs[(int64_t)i * W], si = CPLX ? rhs[(int64_t)i * W + 1] : 0.;
+    for (int j = i + 1; j < K; ++j) {
+      const double* rij = &Rp[((int64_t)i + (int64_t)j * K) * W]; const double* xj = &Tt[((int64_t)col + (int64_t)j * ncols) * W];
+      if constexpr (CPLX) { sr -= rij[0] * xj[0] - rij[1] * xj[1]; si -= rij[0] * xj[1] + rij[1] * xj[0]; } else { sr -= rij[0] * xj[0]; }
+    }
+    const double d = Rp[((int64_t)i + (int64_t)i * K) * W];   /* the diagonal of R is real */
+    double* out = &Tt[((int64_t)col + (int64_t)i * ncols) * W]; out[0] = sr / d; if constexpr (CPLX) { out[1] = si / d; }
+  }
+}
+
+/* X[jpiv[x]-1, y] = (x < K) ? (x == y) : conj(T[y, x-K]) for y < K (reference: scatter mode 'I', src/matcopy.cu:48-52) */
+template <typename T, bool CPLX>
+__global__ void interp_out_kernel(int32_t N, int32_t K, const int32_t* __restrict__ jpiv, const double* __restrict__ Tt, T* __restrict__ X, int64_t ldx) {
+  const int y = blockIdx.x * T_THREADS + threadIdx.x, x = blockIdx.y; if (y >= K) { return; }
+  const int64_t row = jpiv[x] - 1; double vr, vi = 0.;
+  if (x < K) { vr = (x == y) ? 1. : 0.; } else { const int ncols = N - K; const double* t = &Tt[((int64_t)(x - K) + (int64_t)y * ncols) * (CPLX ? 2 : 1)]; vr = t[0]; if constexpr (CPLX) { vi = -t[1]; } }
+  if constexpr (CPLX) { T* o = &X[2 * (row + (int64_t)y * ldx)]; store_real<T>(o, vr); store_real<T>(o + 1, vi); } else { store_real<T>(&X[row + (int64_t)y * ldx], vr); }
+}
+
+}  // namespace
+
+extern "C" int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t Gtype, const void* Rt, int32_t ldr, double* B) {
+  if (N <= 0 || rank <= 0) { return 0; }
+  const bool dd = (Gtype & ~1) == HYK_DD, cplx = Gtype & 1; const int WR = dd ? 2 : 1, WE = WR * (cplx ? 2 : 1);
+  dim3 grid((N + T_THREADS - 1) / T_THREADS, rank);
+  if (cplx) { factor_to_b_kernel<true><<<grid, T_THREADS, 0, stream>>>(N, rank, (const double*)Rt, ldr, WE, WR, B); } else { factor_to_b_kernel<false><<<grid, T_THREADS, 0, stream>>>(N, rank, (const double*)Rt, ldr, WE, WR, B); }
+  return 0;
+}
+
+/* one sweep = n-1 rounds over the r columns of B (N x r, FP64, complex interleaved); rotations counts the rotations applied */
+extern "C" int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations) {
+  if (N <= 0 || r <= 1) { return 0; }
+  const int n = (r + 1) & ~1;
+  for (int round = 0; round < n - 1; ++round) {
+    if (Complex) { jacobi_round_kernel<true><<<n / 2, T_THREADS, 0, stream>>>(N, n, r, round, B, tol, rotations); } else { jacobi_round_kernel<false><<<n / 2, T_THREADS, 0, stream>>>(N, n, r, round, B, tol, rotations); }
+  }
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+extern "C" int hykColumnNorms(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, const double* B, double* sigma) {
+  if (N <= 0 || r <= 0) { return 0; }
+  if (Complex) { column_norm_kernel<true><<<r, T_THREADS, 0, stream>>>(N, B, sigma); } else { column_norm_kernel<false><<<r, T_THREADS, 0, stream>>>(N, B, sigma); }
+  return 0;
+}
+
+extern "C" int hykBasisOut(hipStream_t stream, int32_t N, int32_t rank, int32_t Atype, const double* B, const double* sigma, const int32_t* order, void* X, int64_t ldx) {
+  if (N <= 0 || rank <= 0) { return 0; }
+  dim3 grid((N + T_THREADS - 1) / T_THREADS, rank);
+  switch (Atype) {
+    case HYK_F64: basis_out_kernel<double, false><<<grid, T_THREADS, 0, stream>>>(N, B, sigma, order, (double*)X, ldx); break;
+    case HYK_F32: basis_out_kernel<float, false><<<grid, T_THREADS, 0, stream>>>(N, B, sigma, order, (float*)X, ldx); break;
+    case HYK_F16: basis_out_kernel<__half, false><<<grid, T_THREADS, 0, stream>>>(N, B, sigma, order, (__half*)X, ldx); break;
+    case HYK_F64C: basis_out_kernel<double, true><<<grid, T_THREADS, 0, stream>>>(N, B, sigma, order, (double*)X, ldx); break;
+    case HYK_F32C: basis_out_kernel<float, true><<<grid, T_THREADS, 0, stream>>>(N, B, sigma, order, (float*)X, ldx); break;
+    case HYK_F16C: basis_out_kernel<__half, true><<<grid, T_THREADS, 0, stream>>>(N, B, sigma, order, (__half*)X, ldx); break;
+    default: return -1;
+  }
+  return 0;
+}
+
+extern "C" int hykValuesOut(hipStream_t stream, int32_t K, int32_t Atype, const double* S, void* out) {
+  if (K <= 0) { return 0; }
+  const int grid = (K + T_THREADS - 1) / T_THREADS;
+  switch (Atype & ~1) {
+    case HYK_F64: values_out_kernel<double><<<grid, T_THREADS, 0, stream>>>(K, S, (double*)out); break;
+    case HYK_F32: values_out_kernel<float><<<grid, T_THREADS, 0, stream>>>(K, S, (float*)out); break;
+    case HYK_F16: values_out_kernel<__half><<<grid, T_THREADS, 0, stream>>>(K, S, (__half*)out); break;
+    default: return -1;
+  }
+  return 0;
+}
+
+/* interpolation: Rp (K x N, FP64) and Tt ((N-K) x K) are scratch */
+extern "C" int hykInterpSolve(hipStream_t stream, int32_t N, int32_t K, int32_t Gtype, const void* Rt, int32_t ldr, const int32_t* jpiv, double* Rp, double* Tt) {
+  if (N <= 0 || K <= 0 || K >= N) { return 0; }
+  const bool dd = (Gtype & ~1) == HYK_DD, cplx = Gtype & 1; const int WR = dd ? 2 : 1, WE = WR * (cplx ? 2 : 1);
+  dim3 grid((K + T_THREADS - 1) / T_THREADS, N); const int ncols = N - K, sgrid = (ncols + T_THREADS - 1) / T_THREADS;
+  if (cplx) { gather_factor_kernel<true><<<grid, T_THREADS, 0, stream>>>(N, K, (const double*)Rt, ldr, WE, WR, jpiv, Rp); upper_solve_kernel<true><<<sgrid, T_THREADS, 0, stream>>>(K, ncols, Rp, Tt); }
+  else { gather_factor_kernel<false><<<grid, T_THREADS, 0, stream>>>(N, K, (const double*)Rt, ldr, WE, WR, jpiv, Rp); upper_solve_kernel<false><<<sgrid, T_THREADS, 0, stream>>>(K, ncols, Rp, Tt); }
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+extern "C" int hykInterpOut(hipStream_t stream, int32_t N, int32_t K, int32_t Atype, const int32_t* jpiv, const double* Tt, void* X, int64_t ldx) {
+  if (N <= 0 || K <= 0) { return 0; }
+  dim3 grid((K + T_THREADS - 1) / T_THREADS, N);
+  switch (Atype) {
+    case HYK_F64: interp_out_kernel<double, false><<<grid, T_THREADS, 0, stream>>>(N, K, jpiv, Tt, (double*)X, ldx); break;
+    case HYK_F32: interp_out_kernel<float, false><<<grid, T_THREADS, 0, stream>>>(N, K, jpiv, Tt, (float*)X, ldx); break;
+    case HYK_F16: interp_out_kernel<__half, false><<<grid, T_THREADS, 0, stream>>>(N, K, jpiv, Tt, (__half*)X, ldx); break;
+    case HYK_F64C: interp_out_kernel<double, true><<<grid, T_THREADS, 0, stream>>>(N, K, jpiv, Tt, (double*)X, ldx); break;
+    case HYK_F32C: interp_out_kernel<float, true><<<grid, T_THREADS, 0, stream>>>(N, K, jpiv, Tt, (float*)X, ldx); break;
+    case HYK_F16C: interp_out_kernel<__half, true><<<grid, T_THREADS, 0, stream>>>(N, K, jpiv, Tt, (__half*)X, ldx); break;
+    default: return -1;
+  }
+  return 0;
+}
+
+/* Orthonormal basis of the column space by one-sided Jacobi: V W = U Sigma; the columns are rotated until mutually
+ * orthogonal, then normalised in place (a zero column stays zero and drops out of the projector).
+ * work: at least 64 + 8 r bytes of device memory. */
+extern "C" int hykOrthonormalize(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* V, int64_t ldv, double* work) {
+  if (N <= 0 || r <= 0) { return 0; }
+  if (ldv != N) { return -1; }
+  int32_t* counter = reinterpret_cast<int32_t*>(work); double* sigma = work + 8;
+  for (int sweep = 0; sweep < 40 && r > 1; ++sweep) {
+    if (hipMemsetAsync(counter, 0, 64, stream) != hipSuccess) { return -3; }
+    if (hykJacobiSweep(stream, Complex, N, r, V, 2.220446049250313e-16, counter) != 0) { return -3; }
+    int32_t rotations = 0;
+    if (hipMemcpyAsync(&rotations, counter, sizeof(int32_t), hipMemcpyDeviceToHost, stream) != hipSuccess || hipStreamSynchronize(stream) != hipSuccess) { return -3; }
+    if (rotations == 0) { break; }
+  }
+  if (hykColumnNorms(stream, Complex, N, r, V, sigma) != 0) { return -3; }
+  const int W = Complex ? 2 : 1; dim3 grid((N * W + T_THREADS - 1) / T_THREADS, r);
+  normalize_columns_kernel<<<grid, T_THREADS, 0, stream>>>(N, W, V, sigma);
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}

@@ -1,0 +1,105 @@
+/*
+ * hyacin_kernels.h -- the thin C-ABI layer of hand-written HIP kernels under
+ * the hyacin.h API.  Plain pointers and sizes only; every device pointer is HBM
+ * memory, every function enqueues on the given stream and returns 0 on success,
+ * a negative value for invalid arguments (-1, -2) or a failed launch (-3).
+ * The host C++ of the library calls exactly these; tests bind them with ctypes.
+ * Precision arguments take hyacinPrecision_t values.
+ */
+#pragma once
+#include <stdint.h>
+#include <stddef.h>
+#include <hip/hip_runtime_api.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HYK_GRAM_LIMBS 0
+#define HYK_GRAM_CRT 1
+
+/* Per-column scales.  Replaces src/fp_exponent.cu:23-51 (init / per-slice exponent / min-reduce kernels).
+ * vexp: (batches + 1) * N int32 = [global | slice 0 | slice 1 | ...]. lda in elements. */
+int hykColumnExponents(hipStream_t stream, int32_t batches, int32_t segM, int32_t lastM, int32_t N, int32_t Atype, const void* A, int64_t lda, int32_t u, int32_t* vexp);
+
+/* Bits needed per row slice.  Replaces internal::int8::vector_range, src/fp_exponent.cu:67-76. */
+int hykSliceRange(hipStream_t stream, int32_t batches, int32_t N, int32_t u, const int32_t* vexp, int32_t* segU);
+
+/* Limb panels.  Replaces internal::int8::quantize_limbs, src/quantize_limbs.cu:46-101.
+ * B: panels of N columns x ldb rows int8, panel stride N * ldb; real orderA panels, complex 3 * orderA. */
+int hykQuantizeLimbs(hipStream_t stream, int32_t M, int32_t N, int32_t orderA, int32_t Atype, const void* A, int64_t lda, const int32_t* vexp, int8_t* B, int64_t ldb);
+
+/* CRT residue panels.  Replaces internal::int8::quantize_crt, src/quantize_crt_real.cu:63-112 and
+ * src/quantize_crt_complex.cu:72-123.  maxBits: bound on the bit length of the quantized magnitudes (<= 0: unknown). */
+int hykQuantizeCrt(hipStream_t stream, int32_t M, int32_t N, int32_t orderA, int32_t Atype, const void* A, int64_t lda, const int32_t* vexp, int8_t* B, int64_t ldb, int32_t maxBits);
+
+/* Rows [row0, row1) of `cols` consecutive panel columns set to zero.  Replaces the cudaMemset2DAsync padding of
+ * src/hyacin_herk.cpp:154,261,275. */
+int hykZeroRows(hipStream_t stream, int8_t* B, int64_t ldb, int64_t cols, int32_t row0, int32_t row1);
+
+/* Accumulator workspace of the Gram kernels: size, and clearing (the Gram calls expect it zero and leave it zero). */
+size_t hykGramWorkspaceBytes(int32_t kind, int32_t Complex, int32_t N, int32_t orderA);
+int hykGramWorkspaceClear(hipStream_t stream, void* workspace, size_t bytes);
+
+/* C (+)= exact integer Gram of CRT residue panels (K rows, multiple of 128, padding rows zero).
+ * Replaces i8herk_crt, src/hyacin_herk.cpp:163-281: int8 GEMMs + crt_diag_real / crt_rotate / crt_extra_* + reconstruct_*. */
+int hykGramCrt(hipStream_t stream, int32_t Complex, int32_t N, int32_t orderA, const int8_t* panels, int64_t ldb, int32_t K, int32_t beta, int32_t orderC, uint64_t* C, void* workspace);
+
+/* C (+)= exact integer Gram of limb panels.  Replaces i8herk_limbs, src/hyacin_herk.cpp:61-161: int8 GEMMs +
+ * limbs_diag / limbs_cross_real / limbs_cross_imag. */
+int hykGramLimbs(hipStream_t stream, int32_t Complex, int32_t N, int32_t orderA, const int8_t* panels, int64_t ldb, int32_t K, int32_t beta, int32_t orderC, uint64_t* C, void* workspace);
+
+/* Measurement hooks (no counterpart in the reference): time every launch of the contraction kernel with HIP events on
+ * its stream.  hykGramProfile(1) starts a fresh record, hykGramProfile(0) stops; Read waits for the recorded launches. */
+int hykGramProfile(int32_t enable);
+int hykGramProfileRead(double* totalMs, int32_t* launches);
+
+/* K slab staged in LDS per step of the Gram kernel: 64 or 128 bytes (tuning knob; default 64). */
+int hykGramSetSlab(int32_t bk);
+
+/* Bit length of the dominant diagonal entry of the integer Gram.  Replaces gram_range_kernel, src/fp_i63tp_dequantize.cu:17-26. */
+int hykGramRange(hipStream_t stream, int32_t N, int32_t orderC, const uint64_t* C, const int32_t* vexp, int32_t* out);
+
+/* Packed integer Gram -> full Hermitian floating Gram.  Replaces triangle_unpack_dequantize_kernel, src/fp_i63tp_dequantize.cu:121-159. */
+int hykDequantize(hipStream_t stream, int32_t N, int32_t orderC, const uint64_t* C, const int32_t* vexp, int32_t Gtype, void* G, int64_t ldg);
+
+/* Pivoted Cholesky.  Replaces internal::Cholesky::potrfp, src/hyacin_potrfp.cu:119-343.
+ * G: N x N (FP64 / FP64 complex / double-double / double-double complex), read only.
+ * Rt: zero-initialised, column-wise factor Rt[c * ldr + k] = R[k, c] in the type of G, ldr >= min(N, K + 1).
+ * jpiv: N 1-based pivots in the reference's swap order.  rankOut: device-visible int32 (pinned host memory). */
+size_t hykPotrfpWorkspaceBytes(int32_t N, int32_t Gtype);
+int hykPotrfp(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, int32_t N, int32_t Gtype, const void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, void* workspace, int32_t* rankOut);
+
+/* SVD tail.  Replaces the cuSOLVER gesvdj call and the copies around it, src/gram_evd.cu:110-137. */
+int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t Gtype, const void* Rt, int32_t ldr, double* B);
+int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations);
+int hykColumnNorms(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, const double* B, double* sigma);
+int hykBasisOut(hipStream_t stream, int32_t N, int32_t rank, int32_t Atype, const double* B, const double* sigma, const int32_t* order, void* X, int64_t ldx);
+int hykValuesOut(hipStream_t stream, int32_t K, int32_t Atype, const double* S, void* out);
+
+/* Interpolation tail.  Replaces cuBLAS trsm + scatter modes 'U' / 'I', src/gram_id.cpp:40-46, src/matcopy.cu:48-52. */
+int hykInterpSolve(hipStream_t stream, int32_t N, int32_t K, int32_t Gtype, const void* Rt, int32_t ldr, const int32_t* jpiv, double* Rp, double* Tt);
+int hykInterpOut(hipStream_t stream, int32_t N, int32_t K, int32_t Atype, const int32_t* jpiv, const double* Tt, void* X, int64_t ldx);
+
+/* Converting copy / transpose.  Replaces scatter_matcopy modes 'A', 'T', 'C', src/matcopy.cu:23-44,58-96. */
+int hykMatcopy(hipStream_t stream, char mode, int64_t M, int64_t N, int32_t srcType, const void* A, int64_t lda, int32_t dstType, void* B, int64_t ldb);
+
+/* *out += sum of squares.  Replaces cublasDnrm2_64, src/lra.cpp:170,204. */
+int hykSumSquares(hipStream_t stream, int64_t M, int64_t N, const double* A, int64_t lda, double* out);
+
+/* Complex FP16 matrix product C = op(A) B on interleaved half pairs, FP32 accumulation on the MFMA units.
+ * Replaces internal::matmul_cf16_{cn,tn,nn}, src/matmul_fp16_complex.cu:21-89. opA: 'N', 'T' or 'C'. */
+int hykMatmulCf16(hipStream_t stream, char opA, int32_t M, int32_t N, int32_t K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C, int64_t ldc);
+
+/* Real / complex matrix product C = op(A) B in the storage type (FP64, FP32, FP16 and complex FP64 / FP32), used by the
+ * column-segmented fit and the residual check.  Replaces the cuBLAS gemm calls of src/lra.cpp:86-105,202-203.
+ * alpha/beta are real scalars. opA 'N' | 'T' | 'C', opB 'N' | 'T' | 'C'. */
+int hykGemm(hipStream_t stream, char opA, char opB, int32_t M, int32_t N, int32_t K, double alpha, int32_t type, const void* A, int64_t lda, const void* B, int64_t ldb, double beta, void* C, int64_t ldc);
+
+/* Householder QR, Q factor only: V (N x r, FP64 or complex FP64, interleaved) is overwritten by an orthonormal basis of
+ * its column space.  Replaces cuSOLVER geqrf + orgqr/ungqr, src/lra.cpp:176-191. work: r * sizeof(element) + 64 bytes. */
+int hykOrthonormalize(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* V, int64_t ldv, double* work);
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,74 @@
+/* Host build of the integer device helpers (hyk_common.h) so their arithmetic can be checked on a CPU
+ * against the oracle before any kernel runs: rounding, balanced digits, residues, limb encoding. */
+#include <cstring>
+#include "hyk_common.h"
+#include "crt_tables.h"
+
+using namespace hyk;
+
+static Dec dec_of(int type, const void* p, int64_t i, int part) {
+  switch (type & ~1) {
+    case HYK_F64: { uint64_t b; std::memcpy(&b, (const char*)p + (i * (1 + (type & 1)) + part) * 8, 8); return decompose_f64(b); }
+    case HYK_F32: { uint32_t b; std::memcpy(&b, (const char*)p + (i * (1 + (type & 1)) + part) * 4, 4); return decompose_f32(b); }
+    default: { uint16_t b; std::memcpy(&b, (const char*)p + (i * (1 + (type & 1)) + part) * 2, 2); return decompose_f16(b); }
+  }
+}
+
+extern "C" {
+
+/* out[i] = {lo64, hi32 sign-extended to 64} of RNE(x_i 2^expon) */
+void hm_round(int type, const void* x, int64_t n, int32_t expon, int64_t* out) {
+  for (int64_t i = 0; i < n; ++i) { I96 q = round_scaled(dec_of(type, x, i, 0), expon); out[2 * i] = (int64_t)q.lo; out[2 * i + 1] = (int64_t)(int32_t)q.hi; }
+}
+
+void hm_digits(int type, const void* x, int64_t n, int32_t expon, int order, int8_t* out) {
+  for (int64_t i = 0; i < n; ++i) {
+    I96 q = round_scaled(dec_of(type, x, i, 0), expon); uint32_t carry = 0;
+    for (int l = 0; l < order; ++l) { uint32_t t = i96_byte(q, l) + carry; out[i * order + l] = (int8_t)(t & 0xffu); carry = (t >> 8) + ((t >> 7) & 1u); }
+  }
+}
+
+void hm_residues(int cplxTable, int words, int type, const void* x, int64_t n, int32_t expon, int order, int8_t* out) {
+  for (int64_t i = 0; i < n; ++i) {
+    I96 q = round_scaled(dec_of(type, x, i, 0), expon);
+    for (int m = 0; m < order; ++m) {
+      Mod k = make_mod(cplxTable ? hyk_crt_cplx_mo[m] : hyk_crt_real_mo[m]);
+      uint32_t r = words == 3 ? reduce_i96<3>(q, k) : reduce_i96<6>(q, k);
+      out[i * order + m] = residue_to_i8(r, k.m);
+    }
+  }
+}
+
+int32_t hm_frexp(int type, const void* x) {
+  switch (type & ~1) {
+    case HYK_F64: { uint64_t b; std::memcpy(&b, x, 8); return frexp_exp_f64(b & 0x7fffffffffffffffull); }
+    case HYK_F32: { uint32_t b; std::memcpy(&b, x, 4); return frexp_exp_f32(b & 0x7fffffffu); }
+    default: { uint16_t b; std::memcpy(&b, x, 2); return frexp_exp_f16(b & 0x7fffu); }
+  }
+}
+
+/* limbs (L x 1, stride 1) -> 192-bit -> (+ v << sh) -> limbs */
+void hm_limb_roundtrip(int L, const uint64_t* in, int64_t v, uint32_t sh, uint64_t* out, uint64_t* words) {
+  I192 a = limbs_to_i192(L, in, 1); i192_add_shifted_i64(a, v, sh); i192_to_limbs(a, L, out, 1); words[0] = a.w[0]; words[1] = a.w[1]; words[2] = a.w[2];
+}
+
+int32_t hm_reduce_i32(int32_t v, uint32_t m) { return (int32_t)reduce_i32(v, m, (uint32_t)(0x100000000ull / m), (uint32_t)(0x100000000ull % m)); }
+
+/* centred CRT lift as in the reconstruction kernel; residues canonical; returns three 64-bit words */
+void hm_crt_lift(int cplxTable, int order, const uint32_t* residues, uint64_t* words) {
+  I192 a; a.w[0] = a.w[1] = a.w[2] = 0;
+  for (int x = 0; x < order; ++x) {
+    const uint32_t m = cplxTable ? hyk_crt_cplx_mo[x] : hyk_crt_real_mo[x], d = (uint32_t)(0x100000000ull / m);
+    const uint32_t minv = cplxTable ? hyk_crt_cplx_minv[order - 1][x] : hyk_crt_real_minv[order - 1][x];
+    const uint32_t tt = reduce_u32(reduce_u32(residues[x], m, d) * minv, m, d);
+    I192 pd; for (int k = 0; k < 3; ++k) { pd.w[k] = cplxTable ? hyk_crt_cplx_Pd[order - 1][x][k] : hyk_crt_real_Pd[order - 1][x][k]; }
+    if (i192_is_neg(a)) { i192_add(a, i192_mul_small(pd, tt)); } else { i192_add(a, i192_neg(i192_mul_small(pd, m - tt))); }
+  }
+  I192 P; for (int k = 0; k < 3; ++k) { P.w[k] = cplxTable ? hyk_crt_cplx_P[order - 1][k] : hyk_crt_real_P[order - 1][k]; }
+  if (i192_is_neg(a)) { i192_add(a, P); }
+  I192 twice = a; i192_add(twice, a); I192 diff = twice; i192_add(diff, i192_neg(P));
+  if (!i192_is_neg(diff)) { i192_add(a, i192_neg(P)); }
+  words[0] = a.w[0]; words[1] = a.w[1]; words[2] = a.w[2];
+}
+
+}

@@ -1,0 +1,256 @@
+"""The hyacin.h entry points on the GPU against the oracle pipeline: bit-exact integer Gram, singular values and
+Gram within 10*eps, fitted bases within 2x of the oracle's own projection residual."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from util import as_complex, haar, rand_matrix
+
+pytestmark = pytest.mark.gpu
+
+NP_OF = {0: np.float64, 1: np.complex128, 2: np.float32, 3: np.complex64, 4: np.float16, 5: np.float16}
+
+
+@pytest.fixture(scope="module")
+def env():
+    import torch
+    import hyacinth_amd as ha
+    from gpu_util import stream
+    h = ha.create_handle(stream=stream().value)
+    yield ha, h
+    ha.destroy_handle(h)
+
+
+def low_rank(rng, M, N, decay, cplx=False, noise=0.0):
+    U, V = haar(rng, M, N, cplx), haar(rng, N, N, cplx)
+    s = decay ** np.arange(N)
+    A = (U * s) @ V.conj().T
+    if noise:
+        A = A + noise * (rng.standard_normal((M, N)) + (1j * rng.standard_normal((M, N)) if cplx else 0))
+    return A, s
+
+
+def to_storage(A, at):
+    if at in (0, 1):
+        return A.astype(NP_OF[at])
+    if at in (2, 3):
+        return A.astype(NP_OF[at])
+    if at == 4:
+        return A.real.astype(np.float16)
+    return np.stack([A.real, A.imag], axis=-1).astype(np.float16)
+
+
+def dev_matrix(A, opA):
+    """Device copy of op^-1(A) so that op(stored) == A; returns (tensor, lda)."""
+    from gpu_util import dev
+    if A.ndim == 3:                       # complex half [M, N, 2]
+        if opA == "N":
+            return dev(np.ascontiguousarray(np.transpose(A, (1, 0, 2)))), A.shape[0]
+        S = A.copy()
+        if opA == "C":
+            S[..., 1] = -S[..., 1]
+        return dev(np.ascontiguousarray(S)), A.shape[1]      # stored N x M column-major == [m][n][2]
+    if opA == "N":
+        return dev(np.ascontiguousarray(A.T)), A.shape[0]
+    S = A.conj() if opA == "C" else A
+    return dev(np.ascontiguousarray(S)), A.shape[1]          # stored N x M column-major: element (n, m) at n + m*N
+
+
+def run_tsvd(env, A, eps, K, opA="N", segmented=False):
+    from gpu_util import zeros, ptr, sync, host
+    from oracle import ho
+    ha, h = env
+    at = ho.atype_of(A)
+    M, N = A.shape[0], A.shape[1]
+    dA, lda = dev_matrix(A, opA)
+    eb = {0: 8, 1: 16, 2: 4, 3: 8, 4: 2, 5: 4}[at]
+    sb = eb // (1 + (at & 1))
+    S, V = zeros(sb * K), zeros(eb * N * K)
+    fn = ha.lib().hyacinTsvdFitSegmentN if segmented else ha.lib().hyacinTsvdFit
+    rank = fn(C.byref(h), eps, opA.encode(), M, N, K, ptr(dA), lda, ptr(S), ptr(V), N, 0, at)
+    sync()
+    real = {8: np.float64, 4: np.float32, 2: np.float16}[sb]
+    Sh = host(S, real).astype(np.float64)
+    Vh = host(V, real).astype(np.float64)
+    Vh = (Vh.reshape(K, N, 2)[..., 0] + 1j * Vh.reshape(K, N, 2)[..., 1]).T if at & 1 else Vh.reshape(K, N).T
+    err = ha.lib().hyacinCheckNorm(C.byref(h), opA.encode(), M, N, ptr(dA), lda, rank, ptr(V), N, at)
+    nrm = ha.lib().hyacinCheckNorm(C.byref(h), opA.encode(), M, N, ptr(dA), lda, 0, None, N, at)
+    return rank, Sh, Vh[:, :rank], err, nrm
+
+
+CASES = [
+    # (type, M, N, K, eps, decay, alg, opA)
+    (0, 2048, 96, 96, 1e-10, 10 ** (-1 / 6), b"L", "N"),
+    (0, 2048, 96, 96, 1e-10, 10 ** (-1 / 6), b"A", "N"),
+    (2, 4096, 128, 64, 1e-5, 2 ** (-1 / 4), b"A", "T"),
+    (1, 3000, 80, 40, 1e-12, 10 ** (-1 / 5), b"A", "N"),
+    (5, 4096, 96, 32, 1e-3, 0.8, b"L", "C"),
+    (3, 1500, 70, 70, 1e-6, 0.7, b"A", "C"),
+    (4, 1024, 64, 64, 1e-3, 0.85, b"A", "N"),
+    (1, 1200, 60, 60, 1e-9, 0.6, b"L", "N"),
+]
+
+
+@pytest.mark.parametrize("at,M,N,K,eps,decay,alg,opA", CASES)
+def test_tsvd_fit_parity(env, oracle, at, M, N, K, eps, decay, alg, opA):
+    ha, h = env
+    rng = np.random.default_rng(41)
+    A0, s = low_rank(rng, M, N, decay, cplx=bool(at & 1), noise=eps * 1e-2)
+    A = to_storage(A0, at)
+    h.GramMatrixAlgorithm = alg
+    print("tsvd", at, M, N, K, eps, alg, opA, flush=True)
+    try:
+        rank, S, V, err, nrm = run_tsvd(env, A, eps, K, opA)
+    finally:
+        h.GramMatrixAlgorithm = b"A"
+    r_o, S_o, V_o, g = oracle.tsvd_fit(A, eps, K, alg=alg.decode())
+    Ac = as_complex(A).astype(np.complex128 if at & 1 else np.float64)
+    assert abs(nrm - np.linalg.norm(Ac) ** 2) <= 1e-10 * nrm
+    # rank: the energy cut is decided on sigma values that agree to rounding; allow one at the threshold
+    assert abs(rank - r_o) <= 1
+    tol = 10 * max(eps, {0: 2.2e-16, 1: 2.2e-16, 2: 1.2e-7, 3: 1.2e-7, 4: 9.8e-4, 5: 9.8e-4}[at]) * S_o[0]
+    k = min(rank, r_o)
+    assert np.abs(S[:k] - S_o[:k]).max() <= tol
+    assert not S[rank:].any()
+    # projection residual: own CheckNorm agrees with the closed form, and is within 2x of the oracle basis' residual
+    mine = oracle.check_norm(Ac, V)
+    assert abs(err - mine) <= 1e-6 * nrm + 0.05 * mine
+    ref = oracle.check_norm(Ac, V_o[:, :k]) if k else nrm
+    floor = (10 * tol) ** 2
+    assert oracle.check_norm(Ac, V[:, :k]) <= 2 * ref + floor
+    assert mine <= max(2 * ref, (2 * eps) ** 2 * nrm) + floor
+
+
+def test_gram_api_bit_exact_sliced(env, oracle):
+    """hyacinXquantizeScaleBatch + hyacinXherkBatch against the oracle, sliced rows with uneven scales, beta chaining."""
+    from gpu_util import dev, zeros, ptr, sync, host, colmajor_bytes
+    ha, h = env
+    rng = np.random.default_rng(42)
+    for kind, alg in (("f64", b"A"), ("c128", b"A"), ("f32", b"L"), ("c64", b"C"), ("f16", b"A"), ("c32h", b"L")):
+        M, N, seg = 3000, 150, 512
+        A = rand_matrix(rng, M, N, kind, 1.5)
+        A[512:1024] *= 2.0 ** -12
+        A[2048:2560] = 0
+        A[:, 7] = 0
+        at = oracle.atype_of(A)
+        h.GramMatrixAlgorithm = alg; h.GramSegmentK = seg
+        try:
+            pl = oracle.fit_plan(M, N, 1e-9, at, segK=seg)
+            u, cP, lP, stride = ha.herk_batch_init(h, 1e-9, M, N, at)
+            assert (u, cP, lP, stride) == (pl["u"], pl["cP"], pl["lP"], pl["stride"])
+            dA, lda, _ = colmajor_bytes(A)
+            vexp = zeros(4 * (pl["batches"] + 1) * N)
+            ha.lib().hyacinXquantizeScaleBatch(C.byref(h), pl["batches"], seg, pl["lastM"], N, at, ptr(dA), lda, u, ptr(vexp))
+            Cd = zeros(8 * cP * lP * stride)
+            print("gram api", kind, alg, pl, flush=True)
+            ha.lib().hyacinXherkBatch(C.byref(h), pl["batches"], seg, pl["lastM"], N, at, ptr(dA), lda, u, ptr(vexp), 0, lP, ptr(Cd))
+            sync()
+            v_o = oracle.quantize_scale_batch(A, pl["batches"], seg, pl["lastM"], u)
+            assert np.array_equal(host(vexp, np.int32), v_o)
+            C_o = oracle.herk_batch(A, pl["batches"], seg, pl["lastM"], u, v_o, lP, alg=alg.decode())
+            assert np.array_equal(host(Cd, np.uint64), C_o)
+            # dequantize: type choice and values
+            gt, gb = C.c_int(), C.c_int32()
+            ha.lib().hyacinXdequantizeInit(C.byref(h), N, lP, ptr(Cd), ptr(vexp), at, C.byref(gt), C.byref(gb))
+            g_o, b_o, _ = oracle.dequantize_init(N, lP, C_o, v_o, at)
+            assert (gt.value, gb.value) == (g_o, b_o)
+        finally:
+            h.GramMatrixAlgorithm = b"A"; h.GramSegmentK = 8192
+
+
+@pytest.mark.parametrize("at,opA", [(0, "N"), (1, "N"), (2, "T"), (5, "C")])
+def test_interpolate_fit(env, oracle, at, opA):
+    from gpu_util import zeros, ptr, sync, host
+    ha, h = env
+    rng = np.random.default_rng(43)
+    M, N, K, eps = 2000, 90, 30, {0: 1e-8, 1: 1e-8, 2: 1e-4, 5: 1e-2}[at]
+    A0, _ = low_rank(rng, M, N, 0.6, cplx=bool(at & 1))
+    A0 = A0 * np.exp(rng.uniform(-6, 6, N) if at < 4 else rng.uniform(-1, 1, N))     # badly scaled columns stress the exponent path
+    A = to_storage(A0, at)
+    dA, lda = dev_matrix(A, opA)
+    eb = {0: 8, 1: 16, 2: 4, 5: 4}[at]
+    X, jp = zeros(eb * N * K), zeros(4 * N)
+    print("interp", at, opA, flush=True)
+    rank = ha.lib().hyacinInterpolateFit(C.byref(h), eps, opA.encode(), M, N, K, ptr(dA), lda, ptr(jp), ptr(X), N, 0, at)
+    sync()
+    jpiv = host(jp, np.int32)
+    assert sorted(jpiv.tolist()) == list(range(1, N + 1))
+    r_o, jp_o, X_o, g = oracle.interpolate_fit(A, eps, K)
+    assert abs(rank - r_o) <= 1 and 0 < rank <= K
+    real = {8: np.float64, 16: np.float64, 4: np.float32 if at == 2 else np.float16}[eb]
+    Xh = host(X, real).astype(np.float64)
+    Xh = (Xh.reshape(K, N, 2)[..., 0] + 1j * Xh.reshape(K, N, 2)[..., 1]).T if at & 1 else Xh.reshape(K, N).T
+    Xh = Xh[:, :rank]
+    Ac = as_complex(A).astype(np.complex128 if at & 1 else np.float64)
+    sel = jpiv[:rank] - 1
+    assert np.allclose(Xh[sel], np.eye(rank), atol=1e-3 if at == 5 else 1e-12)
+    resid = np.linalg.norm(Ac - Ac[:, sel] @ Xh.conj().T)
+    sel_o = jp_o[:r_o] - 1
+    resid_o = np.linalg.norm(Ac - Ac[:, sel_o] @ X_o.conj().T)
+    storage_eps = {0: 2.2e-16, 1: 2.2e-16, 2: 1.2e-7, 5: 9.8e-4}[at]
+    assert resid <= 2 * resid_o + 50 * max(eps, storage_eps) * np.linalg.norm(Ac)
+
+
+def test_segmented_fit(env, oracle):
+    ha, h = env
+    rng = np.random.default_rng(44)
+    for at, opA in ((0, "N"), (3, "C"), (5, "C")):
+        M, N, K = 3000, 640, 40                       # floor(sqrt(640/40)) = 4 segments
+        eps = {0: 1e-8, 3: 1e-4, 5: 1e-2}[at]
+        A0, s = low_rank(rng, M, N, 0.75, cplx=bool(at & 1))
+        A = to_storage(A0, at)
+        print("segmented", at, opA, flush=True)
+        rank, S, V, err, nrm = run_tsvd(env, A, eps, K, opA, segmented=True)
+        rank1, S1, V1, err1, _ = run_tsvd(env, A, eps, K, opA, segmented=False)
+        assert 0 < rank <= K and abs(rank - rank1) <= 2
+        k = min(rank, rank1)
+        storage_eps = {0: 2.2e-16, 3: 1.2e-7, 5: 9.8e-4}[at]
+        assert np.abs(S[:k] - S1[:k]).max() <= 20 * max(eps, storage_eps) * S1[0]
+        assert err <= 4 * err1 + (20 * max(eps, storage_eps)) ** 2 * nrm
+
+
+def test_degenerate_inputs(env, oracle):
+    from gpu_util import dev, zeros, ptr, sync, host
+    ha, h = env
+    A = np.zeros((300, 20))
+    dA = dev(A.T.copy())
+    S, V = zeros(8 * 20), zeros(8 * 20 * 20)
+    L = ha.lib()
+    assert L.hyacinTsvdFit(C.byref(h), 1e-8, b"N", 300, 20, 0, ptr(dA), 300, ptr(S), ptr(V), 20, 0, 0) == 0       # K <= 0
+    assert L.hyacinTsvdFit(C.byref(h), 1e-8, b"N", 300, 20, 20, ptr(dA), 300, ptr(S), ptr(V), 20, 0, 99) == 0     # unknown precision
+    assert L.hyacinTsvdFit(C.byref(h), 1e-8, b"N", 300, 20, 20, ptr(dA), 300, ptr(S), ptr(V), 20, 0, 0) == 0      # zero matrix
+    sync()
+    jp = zeros(4 * 20)
+    assert L.hyacinInterpolateFit(C.byref(h), 1e-8, b"N", 300, 20, 5, ptr(dA), 300, ptr(jp), ptr(V), 20, 0, 0) == 0
+    assert L.hyacinCheckNorm(C.byref(h), b"N", 300, 20, ptr(dA), 300, 0, None, 20, 0) == 0.0
+    # timers: off by default -> sync only
+    ms = (C.c_double * 3)(ord("D"), ord("R"), ord("C"))
+    L.hyacinSync_TimerSegments(C.byref(h), ms, 3)
+    # a single non-zero column: rank 1, exact direction
+    A[:, 3] = np.arange(300) + 1.0
+    dA = dev(A.T.copy())
+    assert L.hyacinTsvdFit(C.byref(h), 1e-8, b"N", 300, 20, 20, ptr(dA), 300, ptr(S), ptr(V), 20, 0, 0) == 1
+    sync()
+    Sh, Vh = host(S, np.float64), host(V, np.float64).reshape(20, 20).T
+    assert abs(Sh[0] - np.linalg.norm(A[:, 3])) <= 1e-9 * Sh[0] and abs(abs(Vh[3, 0]) - 1) < 1e-12
+
+
+def test_timer_segments(oracle):
+    import os
+    import hyacinth_amd as ha
+    from gpu_util import dev, zeros, ptr, sync, stream
+    os.environ["HYACIN_CREATE_TIMER"] = "1"
+    try:
+        h = ha.create_handle(stream=stream().value)
+    finally:
+        del os.environ["HYACIN_CREATE_TIMER"]
+    rng = np.random.default_rng(45)
+    A = rng.standard_normal((4000, 64))
+    dA = dev(A.T.copy())
+    S, V = zeros(8 * 64), zeros(8 * 64 * 64)
+    assert ha.lib().hyacinTsvdFit(C.byref(h), 1e-6, b"N", 4000, 64, 64, ptr(dA), 4000, ptr(S), ptr(V), 64, 0, 0) > 0
+    ms = (C.c_double * 4)(ord("D"), ord("R"), ord("C"), ord("x"))
+    ha.lib().hyacinSync_TimerSegments(C.byref(h), ms, 4)
+    assert ms[0] > 0 and ms[1] > 0 and ms[2] == 0 and ms[3] == 0
+    ha.destroy_handle(h)

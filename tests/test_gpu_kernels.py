@@ -1,0 +1,180 @@
+"""HIP kernel layer against the CPU oracle, through the C ABI. Integer results must be bit-exact."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from util import ALL_KINDS, INT_MAX, rand_matrix
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gl():
+    from gpu_util import Lib
+    return Lib()
+
+
+def special(rng, M, N, kind):
+    A = rand_matrix(rng, M, N, kind, 2.0)
+    flat = A
+    flat[:, 1] = 0
+    flat[min(3, M - 1), 2] = 0
+    return A
+
+
+@pytest.mark.parametrize("kind", ALL_KINDS)
+def test_column_exponents(gl, oracle, kind):
+    rng = np.random.default_rng(31)
+    for (M, N, segM) in [(70, 9, 16), (1000, 33, 256), (513, 5, 513)]:
+        A = special(rng, M, N, kind)
+        batches, lastM = (M + segM - 1) // segM, M - (M - 1) // segM * segM
+        for u in (23, 46, -1):
+            got = gl.column_exponents(A, batches, segM, lastM, u)
+            want = oracle.quantize_scale_batch(A, batches, segM, lastM, u)
+            n = len(want) if u >= 0 else N
+            print("exponents", kind, M, N, segM, u, flush=True)
+            assert np.array_equal(got[:n], want[:n])
+
+
+def test_slice_range_and_gram_range(gl, oracle):
+    import torch
+    from gpu_util import dev, zeros, ptr, stream, sync, host
+    rng = np.random.default_rng(32)
+    A = rand_matrix(rng, 640, 40, "f64", 1.0)
+    A[128:256] *= 1e-5
+    A[384:512] = 0
+    vexp = oracle.quantize_scale_batch(A, 5, 128, 128, 33)
+    dv, segU = dev(vexp), zeros(4 * 5)
+    assert gl.L.hykSliceRange(stream(), 5, 40, 33, ptr(dv), ptr(segU)) == 0
+    sync()
+    assert np.array_equal(host(segU, np.int32), oracle.vector_range(5, 40, 33, vexp))
+    for lP, eps in ((1, 1e-3), (2, 1e-10), (3, 1e-15)):
+        pl = oracle.fit_plan(640, 40, eps, 0, corr=7 if lP < 3 else 20, segK=128)
+        v = oracle.quantize_scale_batch(A, 5, 128, 128, pl["u"])
+        Cq = oracle.herk_batch(A, 5, 128, 128, pl["u"], v, pl["lP"])
+        out = zeros(4)
+        assert gl.L.hykGramRange(stream(), 40, pl["lP"], ptr(dev(Cq)), ptr(dev(v)), ptr(out)) == 0
+        sync()
+        assert host(out, np.int32)[0] == oracle.dequantize_init(40, pl["lP"], Cq, v, 0)[2]
+
+
+@pytest.mark.parametrize("kind", ALL_KINDS)
+def test_quantize_panels_bit_exact(gl, oracle, kind):
+    rng = np.random.default_rng(33)
+    cplx = kind.startswith("c")
+    for (M, N) in [(37, 5), (1029, 12)]:
+        A = special(rng, M, N, kind)
+        for u in (5, 23, 46, 62, 81):
+            vexp = oracle.quantize_scale_batch(A, 1, M, M, u)
+            for order in (1, 3, 6, 11):
+                print("limbs", kind, M, N, u, order, flush=True)
+                want = oracle.quantize("limbs", A, order, vexp, ldb=M + 11)
+                got = gl.quantize("limbs", A, order, vexp, ldb=M + 11)
+                assert np.array_equal(got, want)
+            for order in ((1, 7, 15, 20, 21, 25) if cplx else (1, 8, 14, 24)):
+                print("crt", kind, M, N, u, order, flush=True)
+                want = oracle.quantize("crt", A, order, vexp, ldb=M + 3)
+                for mb in (0, u + 1):
+                    got = gl.quantize("crt", A, order, vexp, ldb=M + 3, max_bits=mb)
+                    assert np.array_equal(got, want)
+    # rows appended at an odd offset of an existing panel set (byte-store path)
+    A = special(rng, 50, 4, kind)
+    vexp = oracle.quantize_scale_batch(A, 1, 50, 50, 30)
+    want = oracle.quantize("limbs", A, 4, vexp)
+    got = gl.quantize("limbs", A, 4, vexp, ldb=64, row_offset=7)
+    assert np.array_equal(got[:, :, 7:57], want) and not got[:, :, :7].any() and not got[:, :, 57:].any()
+
+
+def random_panels(rng, p, N, K, rows, lo=-128, hi=128):
+    P = rng.integers(lo, hi, size=(p, N, K), dtype=np.int64).astype(np.int8)
+    P[:, :, rows:] = 0
+    return P
+
+
+GRAM_SHAPES = [(7, 128, 128), (130, 384, 300), (300, 1152, 1100), (513, 256, 256)]
+
+
+@pytest.mark.parametrize("N,K,rows", GRAM_SHAPES)
+@pytest.mark.parametrize("cplx,order", [(0, 1), (0, 14), (1, 2), (1, 15), (1, 22)])
+def test_gram_crt_bit_exact(gl, oracle, N, K, rows, cplx, order):
+    if N > 300 and order > 15:
+        pytest.skip("covered at the smaller sizes")
+    rng = np.random.default_rng(34)
+    panels = random_panels(rng, oracle.n_panels("crt", order, cplx), N, K, rows, -125, 126)
+    orderC = 3
+    print("gram crt", N, K, rows, cplx, order, flush=True)
+    want = oracle.i8herk("crt", cplx, N, order, panels, 0, orderC)
+    got = gl.gram("crt", cplx, N, order, panels, orderC)
+    assert np.array_equal(got, want)
+    want2 = oracle.i8herk("crt", cplx, N, order, panels, 1, orderC, Cin=want)
+    got2 = gl.gram("crt", cplx, N, order, panels, orderC, beta=1, Cin=got)
+    assert np.array_equal(got2, want2)
+
+
+@pytest.mark.parametrize("N,K,rows", GRAM_SHAPES)
+@pytest.mark.parametrize("cplx,order", [(0, 1), (0, 6), (1, 3), (0, 11), (1, 6)])
+def test_gram_limbs_bit_exact(gl, oracle, N, K, rows, cplx, order):
+    if N > 300 and order > 6:
+        pytest.skip("covered at the smaller sizes")
+    rng = np.random.default_rng(35)
+    panels = random_panels(rng, oracle.n_panels("limbs", order, cplx), N, K, rows)
+    orderC = 3 if order > 6 else 2
+    print("gram limbs", N, K, rows, cplx, order, flush=True)
+    want = oracle.i8herk("limbs", cplx, N, order, panels, 0, orderC)
+    got = gl.gram("limbs", cplx, N, order, panels, orderC)
+    assert np.array_equal(got, want)
+    want2 = oracle.i8herk("limbs", cplx, N, order, panels, 1, orderC, Cin=want)
+    got2 = gl.gram("limbs", cplx, N, order, panels, orderC, beta=1, Cin=got)
+    assert np.array_equal(got2, want2)
+
+
+def test_gram_extreme_values_and_long_k(gl, oracle):
+    """All -128 digits over a K that needs several int32-safe splits; all-(-125) residues over K = 131072 rows are covered by the bound."""
+    N, K = 20, 16384 * 3
+    panels = np.full((2, N, K), -128, np.int8)
+    want = oracle.i8herk("limbs", 0, N, 2, panels, 0, 2)
+    assert np.array_equal(gl.gram("limbs", 0, N, 2, panels, 2), want)
+    panels = np.full((2, N, K), -125, np.int8)
+    panels[0] = -128
+    want = oracle.i8herk("crt", 0, N, 2, panels, 0, 2)
+    assert np.array_equal(gl.gram("crt", 0, N, 2, panels, 2), want)
+
+
+def test_gram_slab_128(gl, oracle):
+    rng = np.random.default_rng(36)
+    panels = random_panels(rng, 3, 270, 640, 600, -125, 126)
+    want = oracle.i8herk("crt", 0, 270, 3, panels, 0, 2)
+    try:
+        assert gl.L.hykGramSetSlab(128) == 0
+        got = gl.gram("crt", 0, 270, 3, panels, 2)
+    finally:
+        gl.L.hykGramSetSlab(64)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("cplx", [0, 1])
+def test_dequantize(gl, oracle, cplx):
+    from gpu_util import dev, zeros, ptr, stream, sync, host
+    rng = np.random.default_rng(37)
+    N = 45
+    A = rand_matrix(rng, 300, N, "c128" if cplx else "f64", 2.0)
+    A[:, 4] = 0
+    at = oracle.atype_of(A)
+    for eps, corr in ((1e-3, 7), (1e-10, 7), (1e-15, 20)):
+        pl = oracle.fit_plan(300, N, eps, at, corr=corr)
+        vexp = oracle.quantize_scale_batch(A, 1, 300, 300, pl["u"])
+        Cq = oracle.herk_batch(A, 1, 300, 300, pl["u"], vexp, pl["lP"])
+        for gtype in (oracle.F32 + cplx, oracle.F64 + cplx, oracle.DD + cplx):
+            want = oracle.dequantize(N, pl["lP"], Cq, vexp, gtype)
+            G = zeros(want.nbytes)
+            assert gl.L.hykDequantize(stream(), N, pl["lP"], ptr(dev(Cq)), ptr(dev(vexp)), gtype, ptr(G), N) == 0
+            sync()
+            got = host(G, want.dtype, want.shape)
+            if gtype in (oracle.DD, oracle.DDC):
+                # double-double: compare the represented values (hi + lo) to 2^-100 relative, exactly where the lo word is zero
+                assert np.array_equal(got[..., 0::2], want[..., 0::2])
+                scale = np.abs(want[..., 0::2]).max()
+                assert (np.abs(got[..., 1::2] - want[..., 1::2]) <= scale * 2.0**-100).all()
+            else:
+                assert np.array_equal(got, want)

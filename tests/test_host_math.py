@@ -1,0 +1,127 @@
+"""The integer helpers the HIP kernels are built from (hyk_common.h), compiled for the host and checked against exact arithmetic."""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from oracle import closed_form as cf
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+SRC = os.path.join(ROOT, "tests", "host_math", "host_math.cpp")
+LIB = os.path.join(ROOT, "tests", "host_math", "libhost_math.so")
+
+
+@pytest.fixture(scope="module")
+def hm():
+    hdr = os.path.join(ROOT, "hyacinth_amd", "csrc", "hyk_common.h")
+    if not os.path.exists(LIB) or os.path.getmtime(LIB) < max(os.path.getmtime(SRC), os.path.getmtime(hdr)):
+        subprocess.check_call(["g++", "-O2", "-std=c++17", "-shared", "-fPIC", "-I", os.path.join(ROOT, "hyacinth_amd", "csrc"), SRC, "-o", LIB])
+    L = C.CDLL(LIB)
+    L.hm_frexp.restype = C.c_int32
+    L.hm_reduce_i32.restype = C.c_int32
+    return L
+
+
+def _p(a):
+    return a.ctypes.data_as(C.c_void_p)
+
+
+def samples(rng, dtype, n=400):
+    x = rng.standard_normal(n) * np.exp(rng.standard_normal(n) * 8)
+    x = np.clip(x, -float(np.finfo(dtype).max), float(np.finfo(dtype).max)).astype(dtype)
+    tiny = np.finfo(dtype).tiny
+    special = np.array([0.0, -0.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 3.5, tiny, tiny / 2, -tiny / 4, 1.0, -1.0, 255.5, -128.5, 0.99999], dtype=dtype)
+    return np.concatenate([special, x])
+
+
+TYPES = [(0, np.float64), (2, np.float32), (4, np.float16)]
+
+
+@pytest.mark.parametrize("tcode,dtype", TYPES)
+def test_round_scaled(hm, tcode, dtype):
+    rng = np.random.default_rng(21)
+    x = samples(rng, dtype)
+    for expon in (-30, -3, 0, 1, 17, 40, 62, 81):
+        xs = x[np.abs(x.astype(np.float64)) * 2.0**expon < 2.0**90]
+        out = np.zeros(2 * len(xs), np.int64)
+        hm.hm_round(tcode, _p(xs), C.c_int64(len(xs)), C.c_int32(expon), _p(out))
+        for i, v in enumerate(xs):
+            got = (int(out[2 * i]) & (2**64 - 1)) + (int(out[2 * i + 1]) << 64)
+            assert got == cf.rne_scaled(float(v), expon), (float(v), expon)
+
+
+@pytest.mark.parametrize("tcode,dtype", TYPES)
+def test_digits_and_residues(hm, tcode, dtype):
+    rng = np.random.default_rng(22)
+    x = samples(rng, dtype, 200)
+    for expon in (0, 20, 44):
+        xs = x[np.abs(x.astype(np.float64)) * 2.0**expon < 2.0**47]
+        q = [cf.rne_scaled(float(v), expon) for v in xs]
+        for order in (1, 4, 8, 12):
+            out = np.zeros(len(xs) * order, np.int8)
+            hm.hm_digits(tcode, _p(xs), C.c_int64(len(xs)), C.c_int32(expon), order, _p(out))
+            assert out.reshape(len(xs), order).tolist() == [cf.balanced_digits(v, order) for v in q]
+        for table, moduli in ((0, cf.REAL_MODULI), (1, cf.CPLX_MODULI)):
+            for words in (3, 6):
+                out = np.zeros(len(xs) * len(moduli), np.int8)
+                hm.hm_residues(table, words, tcode, _p(xs), C.c_int64(len(xs)), C.c_int32(expon), len(moduli), _p(out))
+                assert out.reshape(len(xs), len(moduli)).tolist() == [[cf.signed_residue(v, m) for m in moduli] for v in q]
+    # wide values need all six 16-bit words
+    big = np.array([1.0, -1.0, 0.75, -0.3, 1 - 2.0**-52], dtype=np.float64).astype(dtype)
+    for expon in (60, 75, 81):
+        q = [cf.rne_scaled(float(v), expon) for v in big]
+        out = np.zeros(len(big) * 24, np.int8)
+        hm.hm_residues(0, 6, tcode, _p(big), C.c_int64(len(big)), C.c_int32(expon), 24, _p(out))
+        assert out.reshape(len(big), 24).tolist() == [[cf.signed_residue(v, m) for m in cf.REAL_MODULI] for v in q]
+
+
+def test_frexp_exponents(hm):
+    import math
+    for tcode, dtype, minnorm in ((0, np.float64, 2.0**-1022), (2, np.float32, 2.0**-126), (4, np.float16, 0.0)):
+        for v in [1.0, 0.5, 0.75, 3.0, 1e-5, 65504.0 if dtype == np.float16 else 1e30, np.finfo(dtype).tiny, np.finfo(dtype).tiny / 4, 0.0, 6e-8]:
+            x = np.array([v], dtype=dtype)
+            want = cf.column_exponent(abs(float(x[0])), 0, minnorm if dtype != np.float16 else 2.0**-126)
+            got = hm.hm_frexp(tcode, _p(x))
+            assert got == (cf.INT_MAX if want == cf.INT_MAX else -want)
+
+
+def test_reduce_i32_and_limbs(hm):
+    rng = np.random.default_rng(23)
+    for m in cf.REAL_MODULI + cf.CPLX_MODULI:
+        for v in [0, 1, -1, 2**31 - 1, -2**31, m, -m, 16384 * 131071] + [int(t) for t in rng.integers(-2**31, 2**31, 40)]:
+            assert hm.hm_reduce_i32(C.c_int32(v), C.c_uint32(m)) == v % m
+    for L in (1, 2, 3):
+        bits = 63 * (L - 1) + 64
+        for _ in range(200):
+            base = int(rng.integers(-2**62, 2**62)) << int(rng.integers(0, max(1, bits - 64)))
+            v, sh = int(rng.integers(-2**40, 2**40)), int(rng.integers(0, bits - 42))
+            enc = np.zeros(L, np.uint64)
+            t = base
+            for l in range(L - 1):
+                enc[l] = t & (2**63 - 1); t >>= 63
+            enc[L - 1] = t & (2**64 - 1)
+            out, words = np.zeros(L, np.uint64), np.zeros(3, np.uint64)
+            hm.hm_limb_roundtrip(L, _p(enc), C.c_int64(v), C.c_uint32(sh), _p(out), _p(words))
+            want = base + (v << sh)
+            got = sum(int(out[l]) << (63 * l) for l in range(L - 1)) + ((int(out[L - 1]) - (2**64 if int(out[L - 1]) >= 2**63 else 0)) << (63 * (L - 1)))
+            assert got == want
+
+
+@pytest.mark.parametrize("table,moduli", [(0, cf.REAL_MODULI), (1, cf.CPLX_MODULI)])
+def test_crt_lift(hm, table, moduli):
+    rng = np.random.default_rng(24)
+    for order in range(1, len(moduli) + 1):
+        P = 1
+        for m in moduli[:order]:
+            P *= m
+        vals = [0, 1, -1, P // 2 - 1, -(P // 2)] + [int(rng.integers(-2**62, 2**62)) * int(rng.integers(1, 2**62)) % P - P // 2 for _ in range(10)]
+        for v in vals:
+            # un-reduced residue sums, as the accumulators hold them
+            res = np.array([(v % m) + m * int(rng.integers(0, 1000)) for m in moduli[:order]], np.uint32)
+            words = np.zeros(3, np.uint64)
+            hm.hm_crt_lift(table, order, _p(res), _p(words))
+            got = sum(int(words[k]) << (64 * k) for k in range(3))
+            got -= (1 << 192) if got >= (1 << 191) else 0
+            assert got == v, (order, v)
