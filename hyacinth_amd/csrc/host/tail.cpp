@@ -7,7 +7,9 @@
  * potrfp.hip and tail.hip; no vendor solver is involved.  Differences that are visible to a caller:
  *  - an FP32 Gram is widened to FP64 before the Cholesky (the reference factors it in FP32);
  *  - the SVD always runs in FP64, also for FP32 / FP16 storage (the reference uses FP32 there);
- *  - JacobiSVDSweeps == 0 (the reference's "bidiagonalization backend") runs Jacobi to convergence.
+ *  - the Jacobi iteration stops as soon as a sweep applies no rotation; a sweep here is one plain round-robin pass over all
+ *    column pairs, which does less work than a sweep of the vendor's blocked solver, so the cap is 5 x |JacobiSVDSweeps|
+ *    plain sweeps (15 by default); JacobiSVDSweeps == 0 (the reference's "bidiagonalization backend") caps at 30.
  * G is left untouched (the reference overwrites it with the factor).
  */
 #include <numeric>
@@ -63,7 +65,7 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
     /* B = (R P^T)^H, N x rank, FP64 */
     hyh::Scratch B(handle, (size_t)N * rank * 8 * (1 + Complex)), sigma(handle, sizeof(double) * (size_t)rank), counter(handle, 64);
     HYH_KERNEL(hykFactorToB(s, N, rank, f.type, f.Rt.p, f.ldr, B.as<double>()));
-    const int32_t maxSweeps = sweeps > 0 ? sweeps : 30; int32_t used = 0;
+    const int32_t maxSweeps = sweeps > 0 ? 5 * sweeps : 30; int32_t used = 0;
     for (int32_t sw = 0; sw < maxSweeps && rank > 1; ++sw) {
       HYH_KERNEL(hykGramWorkspaceClear(s, counter.p, 64));
       HYH_KERNEL(hykJacobiSweep(s, Complex, N, rank, B.as<double>(), machineEps, counter.as<int32_t>())); ++used;
