@@ -35,6 +35,7 @@
  * together on one XCD (one L2) on the same panels and K range.
  */
 #include <vector>
+#include <type_traits>
 #include <hip/hip_runtime.h>
 #include "hyk_common.h"
 #include "crt_tables.h"
@@ -65,6 +66,7 @@ struct GramArgs {
   const int8_t* panels; int64_t ldb, panelStride;
   void* acc; int64_t planeStride;
   int32_t N, nT, tileCount, kLen, kSplits, K, groupCount, totalItems, itemsPerXcd;
+  uint32_t tileMagic, splitMagic;   /* floor(2^32 / d) + 1: x / d == mulhi(x, magic) while x * d < 2^32 (checked on the host); 0 for d == 1 */
   GramGroup groups[MAX_GROUPS];
   uint32_t pairs[MAX_PAIRS];  /* lanePanel | aPanel << 16 */
 };
@@ -73,11 +75,18 @@ struct GramArgs {
 __device__ __forceinline__ int acc_row(int r, int lane) { return ((r >> 2) << 3) + ((lane >> 5) << 2) + (r & 3); }
 
 template <int BK> struct Slab {
-  static constexpr int PITCH = BK + 16;                 /* bytes per tile row in LDS; 16-byte pad => conflict-free b128 reads */
+  static constexpr int PITCH = BK;                      /* bytes per tile row in LDS, unpadded; 16-byte slots are XOR-swizzled per row */
   static constexpr int TILE_BYTES = TILE * PITCH;
   static constexpr int PIECES = TILE * BK / 16;         /* 16-byte pieces per operand tile */
   static constexpr int PER_THREAD = PIECES / G_THREADS; /* pieces each thread moves per operand tile */
   static constexpr int PER_ROW = BK / 16;
+  /* Slot swizzle: piece kq of row r sits in slot kq ^ swz(r).  Fragment reads touch the same kq of 8 (or 16) consecutive
+   * rows: the swizzle spreads them over all 32 (or 64) banks; a parked row still occupies its own contiguous BK bytes, so
+   * the writes are conflict-free as well. */
+  __device__ static __forceinline__ int swz(int row) {
+    if constexpr (BK == 64) { return (((row >> 1) ^ (row >> 3)) & 1) | (((row >> 2) & 1) << 1); }
+    else { return ((row ^ (row >> 3)) & 1) | (row & 6); }
+  }
 };
 
 template <int BK, int EPI>
@@ -86,12 +95,13 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_kernel(const GramArgs args)
   extern __shared__ __align__(16) int8_t lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wy = wave & 1, wx = wave >> 1;
 
-  /* XCD-aware item mapping */
+  /* XCD-aware item mapping.  Everything derived from the item is wave-uniform and stays in scalar registers: divisions go
+   * through host-made reciprocals (the hardware divides on the vector ALU), the triangular root is a short scalar search. */
   const int item = (int)(blockIdx.x % XCDS) * args.itemsPerXcd + (int)(blockIdx.x / XCDS);
   if ((int)(blockIdx.x / XCDS) >= args.itemsPerXcd || item >= args.totalItems) { return; }
-  const int t = item % args.tileCount, gk = item / args.tileCount, ks = gk % args.kSplits, g = gk / args.kSplits;
-  int tb = (int)((__fsqrt_rn(8.f * (float)t + 1.f) - 1.f) * 0.5f);
-  while ((tb + 1) * (tb + 2) / 2 <= t) { ++tb; } while (tb * (tb + 1) / 2 > t) { --tb; }
+  const int gk = args.tileMagic ? (int)(((uint64_t)(uint32_t)item * args.tileMagic) >> 32) : item, t = item - gk * args.tileCount;
+  const int g = args.splitMagic ? (int)(((uint64_t)(uint32_t)gk * args.splitMagic) >> 32) : gk, ks = gk - g * args.kSplits;
+  int tb = 0; while ((tb + 1) * (tb + 2) / 2 <= t) { ++tb; }
   const int ta = t - tb * (tb + 1) / 2;
   const GramGroup grp = args.groups[g];
   const int k0 = ks * args.kLen, kEnd = (k0 + args.kLen) < args.K ? (k0 + args.kLen) : args.K, slabs = (kEnd - k0) / BK;
@@ -103,7 +113,7 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_kernel(const GramArgs args)
   for (int r = 0; r < S::PER_THREAD; ++r) {
     const int p = tid + r * G_THREADS, row = p / S::PER_ROW, kq = p % S::PER_ROW;
     int cy = y0 + row; cy = cy < args.N ? cy : args.N - 1; int cx = x0 + row; cx = cx < args.N ? cx : args.N - 1;
-    srcLane[r] = (int64_t)cy * args.ldb + kq * 16; srcA[r] = (int64_t)cx * args.ldb + kq * 16; dstOff[r] = row * S::PITCH + kq * 16;
+    srcLane[r] = (int64_t)cy * args.ldb + kq * 16; srcA[r] = (int64_t)cx * args.ldb + kq * 16; dstOff[r] = row * S::PITCH + ((kq ^ S::swz(row)) << 4);
   }
 
   v16i acc[4][4];
@@ -117,54 +127,97 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_kernel(const GramArgs args)
   }
 
   const int iters = slabs * grp.pairCount;
-  v4i regLane[S::PER_THREAD], regA[S::PER_THREAD];
-  /* position of the next slab to fetch: pair index within the group and slab within the K range (both wave-uniform) */
-  int nextPair = 0, nextSlab = 0; const int8_t* baseLane = args.panels; const int8_t* baseA = args.panels;
-  auto fetch = [&]() {
-    if (nextSlab == 0) {
-      const uint32_t pp = args.pairs[__builtin_amdgcn_readfirstlane(grp.pairBegin + nextPair)];
-      baseLane = args.panels + (int64_t)(pp & 0xffffu) * args.panelStride + k0; baseA = args.panels + (int64_t)(pp >> 16) * args.panelStride + k0;
-    }
-    #pragma unroll
-    for (int r = 0; r < S::PER_THREAD; ++r) { regLane[r] = *reinterpret_cast<const v4i*>(baseLane + srcLane[r]); }
-    #pragma unroll
-    for (int r = 0; r < S::PER_THREAD; ++r) { regA[r] = *reinterpret_cast<const v4i*>(baseA + srcA[r]); }
-    baseLane += BK; baseA += BK; if (++nextSlab == slabs) { nextSlab = 0; ++nextPair; }
+  /* Global -> register -> LDS pipeline.  HBM / L2 latency is longer than one slab of MFMA work, so the loads of a slab are
+   * issued three slabs ahead into one of two register sets, parked in LDS one slab ahead, and contracted from LDS. */
+  v4i stg[2][2 * S::PER_THREAD];
+  /* Position of the slab requested last (pair within the group, slab within the K range) and its panel addresses; all
+   * wave-uniform and kept in scalar registers.  The loop body has no control flow: past the last slab the position stays
+   * put and the loads re-read the last slab (never parked), so the outstanding-load counter can be waited on exactly.
+   * peek() loads the descriptor of the following pair early; advance() consumes it right after a barrier, where the
+   * LDS / scalar-load counter is drained anyway. */
+  int curPair = 0, curSlab = 0, issued = 1; uint32_t ppNext = args.pairs[grp.pairBegin];
+  const int8_t* baseLane = args.panels + (int64_t)(ppNext & 0xffffu) * args.panelStride + k0;
+  const int8_t* baseA = args.panels + (int64_t)(ppNext >> 16) * args.panelStride + k0;
+  auto peek = [&]() { const int q = curPair + 1 < (int)grp.pairCount ? curPair + 1 : (int)grp.pairCount - 1; ppNext = args.pairs[grp.pairBegin + q]; };
+  auto advance = [&]() {
+    const bool more = issued < iters, wrap = more && (curSlab + 1 == slabs);
+    const int8_t* candLane = args.panels + (int64_t)(ppNext & 0xffffu) * args.panelStride + k0;
+    const int8_t* candA = args.panels + (int64_t)(ppNext >> 16) * args.panelStride + k0;
+    baseLane = wrap ? candLane : baseLane + (more ? BK : 0); baseA = wrap ? candA : baseA + (more ? BK : 0);
+    curSlab = wrap ? 0 : curSlab + (more ? 1 : 0); curPair += wrap ? 1 : 0; issued += more ? 1 : 0;
   };
-  auto stash = [&](int stage) {
+  auto issue = [&](v4i (&reg)[2 * S::PER_THREAD]) {
+    #pragma unroll
+    for (int r = 0; r < S::PER_THREAD; ++r) { reg[r] = *reinterpret_cast<const v4i*>(baseLane + srcLane[r]); }
+    #pragma unroll
+    for (int r = 0; r < S::PER_THREAD; ++r) { reg[S::PER_THREAD + r] = *reinterpret_cast<const v4i*>(baseA + srcA[r]); }
+  };
+  auto stash = [&](const v4i (&reg)[2 * S::PER_THREAD], int stage) {
     int8_t* tileLane = lds + stage * 2 * S::TILE_BYTES; int8_t* tileA = tileLane + S::TILE_BYTES;
     #pragma unroll
-    for (int r = 0; r < S::PER_THREAD; ++r) { *reinterpret_cast<v4i*>(tileLane + dstOff[r]) = regLane[r]; }
+    for (int r = 0; r < S::PER_THREAD; ++r) { *reinterpret_cast<v4i*>(tileLane + dstOff[r]) = reg[r]; }
     #pragma unroll
-    for (int r = 0; r < S::PER_THREAD; ++r) { *reinterpret_cast<v4i*>(tileA + dstOff[r]) = regA[r]; }
+    for (int r = 0; r < S::PER_THREAD; ++r) { *reinterpret_cast<v4i*>(tileA + dstOff[r]) = reg[S::PER_THREAD + r]; }
   };
 
-  /* fragment base offsets: lanes 0-31 take K bytes [0,16), lanes 32-63 bytes [16,32) of each 32-deep MFMA step */
-  const int fragLane = (wy * WAVE_TILE + (lane & 31)) * S::PITCH + (lane >> 5) * 16;
-  const int fragA = (wx * WAVE_TILE + (lane & 31)) * S::PITCH + (lane >> 5) * 16;
-
-  if (iters > 0) { fetch(); stash(0); }
-  __syncthreads();
-  for (int it = 0; it < iters; ++it) {
-    const int stage = it & 1;
-    if (it + 1 < iters) { fetch(); }
+  /* fragment addressing: lanes 0-31 take K bytes [0,16), lanes 32-63 bytes [16,32) of each 32-deep MFMA step; the row of a
+   * lane is lane & 31 plus a multiple of 32, so its swizzle is a per-lane constant */
+  constexpr int KSTEPS = BK / 32;
+  const int rowLane = (wy * WAVE_TILE + (lane & 31)) * S::PITCH, rowA = (wx * WAVE_TILE + (lane & 31)) * S::PITCH, sw = S::swz(lane & 31), hi = lane >> 5;
+  int kOff[KSTEPS];
+  #pragma unroll
+  for (int kk = 0; kk < KSTEPS; ++kk) { kOff[kk] = ((2 * kk + hi) ^ sw) << 4; }
+  v4i fl[2][4], fa[2][4];
+  auto frags = [&](int stage, int kk, int set) {
     const int8_t* tileLane = lds + stage * 2 * S::TILE_BYTES; const int8_t* tileA = tileLane + S::TILE_BYTES;
     #pragma unroll
-    for (int kk = 0; kk < BK / 32; ++kk) {
-      v4i fl[4], fa[4];
+    for (int b = 0; b < 4; ++b) { fl[set][b] = *reinterpret_cast<const v4i*>(tileLane + rowLane + b * 32 * S::PITCH + kOff[kk]); }
+    #pragma unroll
+    for (int a = 0; a < 4; ++a) { fa[set][a] = *reinterpret_cast<const v4i*>(tileA + rowA + a * 32 * S::PITCH + kOff[kk]); }
+  };
+  auto mfmas = [&](int set) {
+    #pragma unroll
+    for (int a = 0; a < 4; ++a) {
       #pragma unroll
-      for (int b = 0; b < 4; ++b) { fl[b] = *reinterpret_cast<const v4i*>(tileLane + fragLane + b * 32 * S::PITCH + kk * 32); }
-      #pragma unroll
-      for (int a = 0; a < 4; ++a) { fa[a] = *reinterpret_cast<const v4i*>(tileA + fragA + a * 32 * S::PITCH + kk * 32); }
-      #pragma unroll
-      for (int a = 0; a < 4; ++a) {
-        #pragma unroll
-        for (int b = 0; b < 4; ++b) { acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[a], fl[b], acc[a][b], 0, 0, 0); }
-      }
+      for (int b = 0; b < 4; ++b) { acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[set][a], fl[set][b], acc[a][b], 0, 0, 0); }
     }
-    if (it + 1 < iters) { stash(stage ^ 1); }
-    __syncthreads();
-  }
+  };
+  /* One slab, software-pipelined.  On entry the fragments of its first K step are already on their way (set 0).
+   * While the matrix cores work through a K step, the LDS pipe fetches the fragments of the next step and parks the next
+   * slab in the other buffer; one barrier before the last K step publishes that slab, whose first fragments are then
+   * requested under the last step's MFMAs together with the global loads of the slab three ahead.
+   * sched_group_barrier pins the interleaving: masks 0x8 MFMA, 0x100 LDS read, 0x200 LDS write, 0x20 global read. */
+  auto slab = [&](auto parity) {
+    constexpr int cur = decltype(parity)::value, nxt = cur ^ 1;
+    peek();
+    #pragma unroll
+    for (int kk = 0; kk < KSTEPS; ++kk) {
+      const bool last = (kk == KSTEPS - 1);
+      if (!last) { frags(cur, kk + 1, (kk + 1) & 1); } else { frags(nxt, 0, 0); issue(stg[nxt]); }
+      mfmas(kk & 1);
+      if (kk == 0) { stash(stg[nxt], nxt); }
+      #pragma unroll
+      for (int i = 0; i < 8; ++i) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); }
+      if (kk == 0) {
+        #pragma unroll
+        for (int i = 0; i < 8; ++i) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x200, (2 * S::PER_THREAD) / 8, 0); }
+      } else if (last) {
+        #pragma unroll
+        for (int i = 0; i < 8; ++i) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x020, (2 * S::PER_THREAD) / 8, 0); }
+      }
+      if (kk == KSTEPS - 2) { __syncthreads(); advance(); }
+    }
+  };
+
+  /* prologue: slabs 0 and 1 requested, slab 0 parked, slab 2 requested, first fragments on their way */
+  issue(stg[0]); peek(); advance(); issue(stg[1]);
+  stash(stg[0], 0);
+  peek(); advance(); issue(stg[0]);
+  __syncthreads();
+  frags(0, 0, 0);
+  int it = 0;
+  for (; it + 1 < iters; it += 2) { slab(std::integral_constant<int, 0>{}); slab(std::integral_constant<int, 1>{}); }
+  if (it < iters) { slab(std::integral_constant<int, 0>{}); }
 
   /* epilogue: lane dimension j <-> y (contiguous in the packed triangle), register dimension i <-> x */
   const bool diagTile = (ta == tb);
@@ -277,6 +330,8 @@ hipError_t launch_gram(hipStream_t stream, GramArgs& a, int epi, int maxProducts
   a.kLen = kLen; a.kSplits = (a.K + kLen - 1) / kLen;
   const int64_t total = base * a.kSplits; if (total > 0x7fffffff / 2) { return hipErrorInvalidValue; }
   a.totalItems = (int)total; a.itemsPerXcd = (int)((total + XCDS - 1) / XCDS);
+  if (total * a.tileCount >= (1ll << 32) || total * a.kSplits >= (1ll << 32)) { return hipErrorInvalidValue; }
+  a.tileMagic = a.tileCount > 1 ? (uint32_t)((1ull << 32) / (uint32_t)a.tileCount) + 1u : 0u; a.splitMagic = a.kSplits > 1 ? (uint32_t)((1ull << 32) / (uint32_t)a.kSplits) + 1u : 0u;
   if (bk == 128) { return epi == EPI_MOD ? launch_one<128, EPI_MOD>(stream, a) : launch_one<128, EPI_I64>(stream, a); }
   return epi == EPI_MOD ? launch_one<64, EPI_MOD>(stream, a) : launch_one<64, EPI_I64>(stream, a);
 }
