@@ -91,7 +91,7 @@ def main():
     ap.add_argument("--no-fit", action="store_true", help="skip the end-to-end hyacinTsvdFit timing")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--cpu-rows", type=int, default=4096)
-    ap.add_argument("--slab", type=int, default=0, help="K slab of the contraction kernel (64 or 128)")
+    ap.add_argument("--slab", type=int, default=-1, help="contraction kernel variant: 0 direct-to-LDS (default), 64 / 128 register-staged with that K slab")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU: the Gram path of this build has no multi-GPU leg (run with --gpus 1)", file=sys.stderr)
@@ -102,7 +102,7 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     L = ha.lib()
     at, opA, M, N, K, eps, alg, desc = WORKLOADS[a.workload]
-    if a.slab:
+    if a.slab >= 0:
         assert L.hykGramSetSlab(a.slab) == 0
     stream = torch.cuda.current_stream().cuda_stream
     h = ha.create_handle(stream=stream, GramMatrixAlgorithm=alg)

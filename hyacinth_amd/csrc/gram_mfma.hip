@@ -248,6 +248,166 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_kernel(const GramArgs args)
   }
 }
 
+/* ------------------------------------------------------------------ contraction with direct global -> LDS loads
+ * Same work items, same epilogue.  The operand slabs (64 K bytes deep) travel from HBM / L2 straight into a ring of four
+ * LDS stages with global_load_lds_dwordx4: no staging registers, no LDS store instructions (at one wavefront per SIMD the
+ * 16-byte LDS stores cost more issue time than the fragment reads).  The hardware writes the 64 lanes of such a load to
+ * 64 consecutive 16-byte slots, so the slot swizzle is applied on the global side: the lane that owns slot s of row r
+ * fetches K piece s ^ swz(r).  The loads are issued from inline assembly: the compiler would otherwise make every LDS
+ * read wait for all direct loads in flight.  Their completion is tracked by hand with the vector-memory counter: every
+ * slab step issues exactly 8 loads per lane (past the end of the K range it re-requests the last slab into a stage
+ * nobody reads again), so "slab j + 1 has landed" is always "at most 16 loads outstanding". */
+constexpr int DMA_BK = 64, DMA_STAGES = 4, DMA_TILE_BYTES = TILE * DMA_BK, DMA_STAGE_BYTES = 2 * DMA_TILE_BYTES;
+
+__device__ __forceinline__ void dma16(uint32_t ldsAddr, const int8_t* src) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(ldsAddr), "v"(src) : "memory");
+}
+
+template <int EPI>
+__global__ __launch_bounds__(G_THREADS, 1) void gram_dma_kernel(const GramArgs args) {
+  using S = Slab<DMA_BK>;
+  constexpr int BK = DMA_BK;
+  extern __shared__ __align__(16) int8_t lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wy = wave & 1, wx = wave >> 1;
+
+  const int item = (int)(blockIdx.x % XCDS) * args.itemsPerXcd + (int)(blockIdx.x / XCDS);
+  if ((int)(blockIdx.x / XCDS) >= args.itemsPerXcd || item >= args.totalItems) { return; }
+  const int gk = args.tileMagic ? (int)(((uint64_t)(uint32_t)item * args.tileMagic) >> 32) : item, t = item - gk * args.tileCount;
+  const int g = args.splitMagic ? (int)(((uint64_t)(uint32_t)gk * args.splitMagic) >> 32) : gk, ks = gk - g * args.kSplits;
+  int tb = 0; while ((tb + 1) * (tb + 2) / 2 <= t) { ++tb; }
+  const int ta = t - tb * (tb + 1) / 2;
+  const GramGroup grp = args.groups[g];
+  const int k0 = ks * args.kLen, kEnd = (k0 + args.kLen) < args.K ? (k0 + args.kLen) : args.K, slabs = (kEnd - k0) / BK;
+  const int y0 = ta * TILE, x0 = tb * TILE;
+
+  /* lane tid of load r fills LDS slot p = tid + 256 r of a tile (row p / 4, slot p % 4) */
+  int64_t srcLane[S::PER_THREAD], srcA[S::PER_THREAD];
+  #pragma unroll
+  for (int r = 0; r < S::PER_THREAD; ++r) {
+    const int p = tid + r * G_THREADS, row = p / S::PER_ROW, kq = (p % S::PER_ROW) ^ S::swz(row);
+    int cy = y0 + row; cy = cy < args.N ? cy : args.N - 1; int cx = x0 + row; cx = cx < args.N ? cx : args.N - 1;
+    srcLane[r] = (int64_t)cy * args.ldb + kq * 16; srcA[r] = (int64_t)cx * args.ldb + kq * 16;
+  }
+  const uint32_t ldsBase = (uint32_t)(size_t)(__attribute__((address_space(3))) int8_t*)lds;
+  const uint32_t dmaBase = __builtin_amdgcn_readfirstlane(ldsBase + (uint32_t)wave * 1024u);
+
+  v16i acc[4][4];
+  #pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    #pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      #pragma unroll
+      for (int r = 0; r < 16; ++r) { acc[a][b][r] = 0; }
+    }
+  }
+
+  const int iters = slabs * grp.pairCount;
+  int curPair = 0, curSlab = 0, issued = 1; uint32_t ppNext = args.pairs[grp.pairBegin];
+  const int8_t* baseLane = args.panels + (int64_t)(ppNext & 0xffffu) * args.panelStride + k0;
+  const int8_t* baseA = args.panels + (int64_t)(ppNext >> 16) * args.panelStride + k0;
+  auto peek = [&]() { const int q = curPair + 1 < (int)grp.pairCount ? curPair + 1 : (int)grp.pairCount - 1; ppNext = args.pairs[grp.pairBegin + q]; };
+  auto advance = [&]() {
+    const bool more = issued < iters, wrap = more && (curSlab + 1 == slabs);
+    const int8_t* candLane = args.panels + (int64_t)(ppNext & 0xffffu) * args.panelStride + k0;
+    const int8_t* candA = args.panels + (int64_t)(ppNext >> 16) * args.panelStride + k0;
+    baseLane = wrap ? candLane : baseLane + (more ? BK : 0); baseA = wrap ? candA : baseA + (more ? BK : 0);
+    curSlab = wrap ? 0 : curSlab + (more ? 1 : 0); curPair += wrap ? 1 : 0; issued += more ? 1 : 0;
+  };
+  /* load i (0..7) of the current slab position into the stage at byte offset stageOff */
+  auto dma = [&](int i, uint32_t stageOff) {
+    const int r = i & 3; const bool second = i >= 4;
+    dma16(dmaBase + stageOff + (second ? (uint32_t)DMA_TILE_BYTES : 0u) + (uint32_t)r * 4096u, (second ? baseA + srcA[r] : baseLane + srcLane[r]));
+  };
+
+  constexpr int KSTEPS = BK / 32;
+  static_assert(KSTEPS == 2, "the slab step below is written for two MFMA K steps");
+  const int rowLane = (wy * WAVE_TILE + (lane & 31)) * S::PITCH, rowA = DMA_TILE_BYTES + (wx * WAVE_TILE + (lane & 31)) * S::PITCH, sw = S::swz(lane & 31), hi = lane >> 5;
+  const int k0Off = ((0 + hi) ^ sw) << 4, k1Off = ((2 + hi) ^ sw) << 4;
+  v4i fl[2][4], fa[2][4];
+  /* fragment read i (0..3 lane operand, 4..7 A operand) of K step kk from the stage at stageOff into register set `set` */
+  auto rd = [&](int i, int set, int kk, uint32_t stageOff) {
+    const int8_t* base = lds + stageOff + (kk ? k1Off : k0Off);
+    if (i < 4) { fl[set][i] = *reinterpret_cast<const v4i*>(base + rowLane + i * 32 * S::PITCH); }
+    else { fa[set][i - 4] = *reinterpret_cast<const v4i*>(base + rowA + (i - 4) * 32 * S::PITCH); }
+  };
+  auto mm = [&](int n, int set) { const int a = n >> 2, b = n & 3; acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[set][a], fl[set][b], acc[a][b], 0, 0, 0); };
+
+  /* prologue: four slabs on their way, the first one landed and published, its first fragments requested */
+  #pragma unroll
+  for (int st = 0; st < DMA_STAGES; ++st) {
+    if (st) { peek(); advance(); }
+    #pragma unroll
+    for (int i = 0; i < 8; ++i) { dma(i, (uint32_t)st * DMA_STAGE_BYTES); }
+  }
+  asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+  __syncthreads();
+  #pragma unroll
+  for (int i = 0; i < 8; ++i) { rd(i, 0, 0, 0u); }
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+
+  for (int it = 0; it < iters; ++it) {
+    const uint32_t curOff = (uint32_t)(it & (DMA_STAGES - 1)) * DMA_STAGE_BYTES, nxtOff = (uint32_t)((it + 1) & (DMA_STAGES - 1)) * DMA_STAGE_BYTES;
+    /* first K step: MFMAs on set 0; the fragments of the second K step go into set 1 under the first eight of them, four
+     * more cover the latency of the last read before the barrier */
+    #pragma unroll
+    for (int i = 0; i < 8; ++i) { rd(i, 1, 1, curOff); }
+    peek();
+    #pragma unroll
+    for (int n = 0; n < 12; ++n) { mm(n, 0); }
+    #pragma unroll
+    for (int i = 0; i < 8; ++i) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); }
+    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    /* slab it + 1 has landed (own loads) and every wave is done reading stage `cur`: publish */
+    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    #pragma unroll
+    for (int n = 12; n < 16; ++n) { mm(n, 0); }
+    advance();
+    __builtin_amdgcn_sched_barrier(0);
+    /* second K step: MFMAs on set 1; first fragments of the next slab into set 0, then stage `cur` is refilled with slab it + 4 */
+    #pragma unroll
+    for (int i = 0; i < 8; ++i) { rd(i, 0, 0, nxtOff); }
+    #pragma unroll
+    for (int n = 0; n < 8; ++n) { mm(n, 1); }
+    #pragma unroll
+    for (int i = 0; i < 8; ++i) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); }
+    #pragma unroll
+    for (int n = 8; n < 16; ++n) { __builtin_amdgcn_sched_barrier(0); mm(n, 1); __builtin_amdgcn_sched_barrier(0); dma(n - 8, curOff); }
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(0xC07F);   /* lgkmcnt(0): set 0 was requested eight MFMAs ago; stating it here keeps waits out of the first K step */
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   /* no direct load may still be writing LDS when the workgroup ends */
+
+  const bool diagTile = (ta == tb);
+  #pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    #pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      const int y = y0 + wy * WAVE_TILE + b * 32 + (lane & 31);
+      #pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int x = x0 + wx * WAVE_TILE + a * 32 + acc_row(r, lane);
+        if (x < args.N && y < args.N && (!diagTile || y <= x)) {
+          const int64_t e = hyk::tri_index(y, x); const int32_t w = acc[a][b][r];
+          if constexpr (EPI == EPI_MOD) {
+            uint32_t* dst = reinterpret_cast<uint32_t*>(args.acc);
+            const uint32_t v = hyk::reduce_i32(w, grp.m, grp.d, grp.c32);
+            if (grp.mulRe) { atomicAdd(&dst[(int64_t)grp.planeRe * args.planeStride + e], grp.mulRe == 1u ? v : hyk::reduce_u32(v * grp.mulRe, grp.m, grp.d)); }
+            if (grp.mulIm) { atomicAdd(&dst[(int64_t)grp.planeIm * args.planeStride + e], grp.mulIm == 1u ? v : hyk::reduce_u32(v * grp.mulIm, grp.m, grp.d)); }
+          } else {
+            unsigned long long* dst = reinterpret_cast<unsigned long long*>(args.acc);
+            const unsigned long long pos = (unsigned long long)(long long)w, negv = (unsigned long long)(-(long long)w);
+            if (grp.mulRe) { atomicAdd(&dst[(int64_t)grp.planeRe * args.planeStride + e], grp.mulRe == 1u ? pos : negv); }
+            if (grp.mulIm) { atomicAdd(&dst[(int64_t)grp.planeIm * args.planeStride + e], grp.mulIm == 1u ? pos : negv); }
+          }
+        }
+      }
+    }
+  }
+}
+
 /* ------------------------------------------------------------------ CRT reconstruction */
 struct ReconTable {
   int32_t order;
@@ -300,7 +460,7 @@ __global__ void fill_zero_kernel(uint4* __restrict__ p, int64_t n16) {
 /* ------------------------------------------------------------------ host-side planning */
 struct Launch { GramArgs args; int epi; };
 
-int g_bk = 64;  /* K slab per LDS stage: 64 or 128 (set through hykGramSetSlab for tuning) */
+int g_bk = 0;   /* 0: direct-to-LDS kernel (default); 64 / 128: register-staged kernel with that K slab (hykGramSetSlab) */
 
 /* optional per-launch timing of the contraction kernel with HIP events on its own stream */
 struct Timed { hipEvent_t start, stop; };
@@ -318,10 +478,22 @@ template <int BK, int EPI> hipError_t launch_one(hipStream_t stream, const GramA
   return hipGetLastError();
 }
 
+template <int EPI> hipError_t launch_dma(hipStream_t stream, const GramArgs& a) {
+  const int ldsBytes = DMA_STAGES * DMA_STAGE_BYTES;
+  static bool attr = false;
+  if (!attr) { hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gram_dma_kernel<EPI>), hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes); if (e != hipSuccess) { return e; } attr = true; }
+  const int blocks = a.itemsPerXcd * XCDS;
+  Timed t{ nullptr, nullptr };
+  if (g_profile) { if (hipEventCreate(&t.start) != hipSuccess || hipEventCreate(&t.stop) != hipSuccess) { return hipErrorUnknown; } (void)hipEventRecord(t.start, stream); }
+  gram_dma_kernel<EPI><<<blocks, G_THREADS, ldsBytes, stream>>>(a);
+  if (g_profile) { (void)hipEventRecord(t.stop, stream); g_timed.push_back(t); }
+  return hipGetLastError();
+}
+
 hipError_t launch_gram(hipStream_t stream, GramArgs& a, int epi, int maxProducts) {
   /* K split: enough items to fill the chip a few times over, never more than maxProducts int8 products per int32 */
   int maxPairs = 1; for (int g = 0; g < a.groupCount; ++g) { maxPairs = a.groups[g].pairCount > maxPairs ? a.groups[g].pairCount : maxPairs; }
-  const int bk = g_bk; int kCap = (maxProducts / maxPairs) / bk * bk; if (kCap < bk) { return hipErrorInvalidValue; }
+  const int bk = g_bk == 0 ? DMA_BK : g_bk; int kCap = (maxProducts / maxPairs) / bk * bk; if (kCap < bk) { return hipErrorInvalidValue; }
   const int64_t base = (int64_t)a.groupCount * a.tileCount; int splits = 1;
   const int wanted = 1024;  /* about four waves of 256 workgroups */
   if (base < wanted) { splits = (int)((wanted + base - 1) / base); }
@@ -332,6 +504,7 @@ hipError_t launch_gram(hipStream_t stream, GramArgs& a, int epi, int maxProducts
   a.totalItems = (int)total; a.itemsPerXcd = (int)((total + XCDS - 1) / XCDS);
   if (total * a.tileCount >= (1ll << 32) || total * a.kSplits >= (1ll << 32)) { return hipErrorInvalidValue; }
   a.tileMagic = a.tileCount > 1 ? (uint32_t)((1ull << 32) / (uint32_t)a.tileCount) + 1u : 0u; a.splitMagic = a.kSplits > 1 ? (uint32_t)((1ull << 32) / (uint32_t)a.kSplits) + 1u : 0u;
+  if (g_bk == 0) { return epi == EPI_MOD ? launch_dma<EPI_MOD>(stream, a) : launch_dma<EPI_I64>(stream, a); }
   if (bk == 128) { return epi == EPI_MOD ? launch_one<128, EPI_MOD>(stream, a) : launch_one<128, EPI_I64>(stream, a); }
   return epi == EPI_MOD ? launch_one<64, EPI_MOD>(stream, a) : launch_one<64, EPI_I64>(stream, a);
 }
@@ -372,7 +545,7 @@ extern "C" int hykGramProfileRead(double* totalMs, int32_t* launches) {
   if (totalMs) { *totalMs = sum; } if (launches) { *launches = (int32_t)g_timed.size(); } return 0;
 }
 
-extern "C" int hykGramSetSlab(int32_t bk) { if (bk != 64 && bk != 128) { return -1; } g_bk = bk; return 0; }
+extern "C" int hykGramSetSlab(int32_t bk) { if (bk != 0 && bk != 64 && bk != 128) { return -1; } g_bk = bk; return 0; }
 
 extern "C" size_t hykGramWorkspaceBytes(int32_t kind, int32_t Complex, int32_t N, int32_t orderA) {
   if (N <= 0 || orderA <= 0) { return 0; }

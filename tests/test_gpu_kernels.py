@@ -141,15 +141,17 @@ def test_gram_extreme_values_and_long_k(gl, oracle):
     assert np.array_equal(gl.gram("crt", 0, N, 2, panels, 2), want)
 
 
-def test_gram_slab_128(gl, oracle):
+@pytest.mark.parametrize("slab", [64, 128])
+def test_gram_register_staged_variants(gl, oracle, slab):
+    """The register-staged contraction kernels (K slab 64 / 128) give the same bits as the default direct-to-LDS one."""
     rng = np.random.default_rng(36)
     panels = random_panels(rng, 3, 270, 640, 600, -125, 126)
     want = oracle.i8herk("crt", 0, 270, 3, panels, 0, 2)
     try:
-        assert gl.L.hykGramSetSlab(128) == 0
+        assert gl.L.hykGramSetSlab(slab) == 0
         got = gl.gram("crt", 0, 270, 3, panels, 2)
     finally:
-        gl.L.hykGramSetSlab(64)
+        gl.L.hykGramSetSlab(0)
     assert np.array_equal(got, want)
 
 
