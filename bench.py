@@ -21,6 +21,10 @@ sys.path.insert(0, ROOT)
 
 INT8_PEAK_TOPS = 5000.0   # MI355X dense INT8 MFMA peak, 5.0 POP/s
 
+# HBM bytes per launch of the contraction kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script
+# (profiles/gram_dma_kernel_target_hbm_traffic.md), each scaled by what the counter reads for copy_kernel's known 1 GiB.
+MEASURED_TRAFFIC = {("target", 0): 8.58e9 + 0.44e9}
+
 WORKLOADS = {
     # name: (type, opA, M, N, K, eps, algorithm, description)
     "target": (0, "N", 131072, 2048, 1024, 1e-12, b"A", "real FP64 M=131072 N=2048 eps=1e-12 (CRT real, 14 moduli)"),
@@ -90,7 +94,10 @@ def main():
     ap.add_argument("--workload", default="target", choices=sorted(WORKLOADS))
     ap.add_argument("--no-fit", action="store_true", help="skip the end-to-end hyacinTsvdFit timing")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--cpu-rows", type=int, default=4096)
+    ap.add_argument("--no-ceiling", action="store_true", help="skip the register-only MFMA ceiling measurement")
+    ap.add_argument("--cpu-rows", type=int, default=65536, help="rows of the workload the CPU baseline is timed on (about 15 s of host work)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="before the timed region, run three plain 1 GiB -> 1 GiB device copies (copy_kernel): the known-size reference for HBM traffic counters")
     ap.add_argument("--slab", type=int, default=-1, help="contraction kernel variant: 0 direct-to-LDS (default), 64 / 128 register-staged with that K slab")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -120,6 +127,14 @@ def main():
         L.hyacinXquantizeScaleBatch(C.byref(h), batches, seg, lastM, N, at, pA, lda, u, pV)
         L.hyacinXherkBatch(C.byref(h), batches, seg, lastM, N, at, pA, lda, u, pV, 0, lP, pC)
 
+    if a.copy_calibration:
+        src = torch.ones(2 ** 27, dtype=torch.float64, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):   # 2^20 x 128 FP64: reads 1 GiB, writes 1 GiB
+            assert L.hykMatcopy(stream, b"A", 2 ** 20, 128, 0, C.c_void_p(src.data_ptr()), 2 ** 20, 0, C.c_void_p(dst.data_ptr()), 2 ** 20) == 0
+        torch.cuda.synchronize()
+        del src, dst
+
     for _ in range(a.warmup):
         step()
     torch.cuda.synchronize()
@@ -141,6 +156,13 @@ def main():
     launches_per_step = max(1, kn.value // a.steps)
     t_kernel = kms.value / 1e3 / a.steps            # contraction kernel time per step
     achieved = ops / t_kernel / 1e12 if t_kernel > 0 else 0.0
+
+    ceiling = None
+    if not a.no_ceiling:   # what a register-only MFMA loop sustains on this device with random operands (power-limited clock)
+        tops, ghz = C.c_double(), C.c_double()
+        if L.hykMfmaCeiling(stream, h.DeviceSMs, 20000, 1, C.byref(tops), C.byref(ghz)) == 0:
+            ceiling = {"value": tops.value, "unit": "TFLOP/s", "clock_ghz": ghz.value,
+                       "what": "register-only v_mfma_i32_32x32x32_i8 loop, random int8 operands, one workgroup of 4 waves per CU"}
 
     fit_ms = None
     if not a.no_fit:
@@ -164,9 +186,11 @@ def main():
                    "quant_bits": u, "gram_limbs": lP, "row_slices": batches},
         "pct_int8_mfma_peak": 100.0 * achieved / INT8_PEAK_TOPS,
         "tsvd_fit_ms": fit_ms,
-        "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s", "frac": achieved / INT8_PEAK_TOPS, "traffic": None,
-                     "kernel": "gram_kernel", "ops": "int8 multiply-adds x2, upper triangle only", "launches_per_step": launches_per_step,
-                     "avg_launch_ms": kms.value / max(1, kn.value), "algorithmic_ops_per_step": ops},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s", "frac": achieved / INT8_PEAK_TOPS,
+                     "traffic": MEASURED_TRAFFIC.get((a.workload, max(a.slab, 0))),
+                     "kernel": "gram_dma_kernel" if a.slab <= 0 else "gram_kernel<%d>" % a.slab, "ops": "int8 multiply-adds x2, upper triangle only", "launches_per_step": launches_per_step,
+                     "avg_launch_ms": kms.value / max(1, kn.value), "algorithmic_ops_per_step": ops,
+                     "sustained_mfma_ceiling": ceiling},
     }
     if not a.no_cpu:
         rows = min(a.cpu_rows, M)

@@ -31,7 +31,7 @@ API_SYMBOLS = [
 KERNEL_SYMBOLS = [
     "hykColumnExponents", "hykSliceRange", "hykQuantizeLimbs", "hykQuantizeCrt", "hykZeroRows",
     "hykGramWorkspaceBytes", "hykGramWorkspaceClear", "hykGramCrt", "hykGramLimbs", "hykGramSetSlab",
-    "hykGramProfile", "hykGramProfileRead", "hykGramRange", "hykDequantize", "hykPotrfpWorkspaceBytes", "hykPotrfp", "hykFactorToB", "hykJacobiSweep",
+    "hykGramProfile", "hykGramProfileRead", "hykMfmaCeiling", "hykGramRange", "hykDequantize", "hykPotrfpWorkspaceBytes", "hykPotrfp", "hykFactorToB", "hykJacobiSweep",
     "hykColumnNorms", "hykBasisOut", "hykValuesOut", "hykInterpSolve", "hykInterpOut", "hykMatcopy",
     "hykSumSquares", "hykMatmulCf16", "hykGemm", "hykOrthonormalize",
 ]
@@ -89,6 +89,7 @@ def lib():
         L.hykGramSetSlab.argtypes = [i32]
         L.hykGramProfile.argtypes = [i32]
         L.hykGramProfileRead.argtypes = [C.POINTER(dbl), C.POINTER(i32)]
+        L.hykMfmaCeiling.argtypes = [vp, i32, i32, i32, C.POINTER(dbl), C.POINTER(dbl)]
         L.hykGramRange.argtypes = [vp, i32, i32, vp, vp, vp]
         L.hykDequantize.argtypes = [vp, i32, i32, vp, vp, i32, vp, i64]
         L.hykPotrfpWorkspaceBytes.argtypes = [i32, i32]; L.hykPotrfpWorkspaceBytes.restype = C.c_size_t

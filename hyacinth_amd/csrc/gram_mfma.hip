@@ -545,6 +545,73 @@ extern "C" int hykGramProfileRead(double* totalMs, int32_t* launches) {
   if (totalMs) { *totalMs = sum; } if (launches) { *launches = (int32_t)g_timed.size(); } return 0;
 }
 
+/* Register-only MFMA loop: what the matrix cores sustain on this device when nothing else competes for power.  Every lane
+ * holds eight int8 operand fragments (hashed lane / block indices when `random`, zeros otherwise) and issues the same
+ * 4x4 pattern of v_mfma_i32_32x32x32_i8 as the contraction kernel; block 0 reports its shader-clock and wall-clock spans. */
+__global__ __launch_bounds__(G_THREADS, 1) void mfma_ceiling_kernel(int iters, int random, int* sink, long long* clocks) {
+  v4i a[4], b[4];
+  #pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    #pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      uint32_t h = (uint32_t)(threadIdx.x * 8 + i) * 2654435761u + (uint32_t)(blockIdx.x * 4 + c) * 40503u; h ^= h >> 15; h *= 2246822519u; h ^= h >> 13;
+      a[i][c] = random ? (int)h : 0; b[i][c] = random ? (int)(h * 3266489917u + 0x9e3779b9u) : 0;
+    }
+  }
+  v16i acc[4][4];
+  #pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    #pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      #pragma unroll
+      for (int r = 0; r < 16; ++r) { acc[i][j][r] = 0; }
+    }
+  }
+  const long long c0 = clock64(), w0 = wall_clock64();
+  for (int it = 0; it < iters; ++it) {
+    #pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      #pragma unroll
+      for (int j = 0; j < 4; ++j) { acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[i], b[j], acc[i][j], 0, 0, 0); }
+    }
+  }
+  const long long c1 = clock64(), w1 = wall_clock64();
+  int sum = 0;
+  #pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    #pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      #pragma unroll
+      for (int r = 0; r < 16; ++r) { sum += acc[i][j][r]; }
+    }
+  }
+  sink[blockIdx.x * G_THREADS + threadIdx.x] = sum;
+  if (threadIdx.x == 0 && blockIdx.x == 0) { clocks[0] = c1 - c0; clocks[1] = w1 - w0; }
+}
+
+/* Measurement hook (no counterpart in the reference).  Runs the register-only MFMA loop on `blocks` workgroups (one per
+ * compute unit is the natural choice) and reports int8 tera-ops per second and the shader clock it ran at.  Allocates and
+ * frees its own small buffers and synchronises the stream. */
+extern "C" int hykMfmaCeiling(hipStream_t stream, int32_t blocks, int32_t iters, int32_t random, double* teraOps, double* clockGHz) {
+  if (blocks <= 0 || iters <= 0) { return -1; }
+  int* sink = nullptr; long long* clocks = nullptr; hipEvent_t e0 = nullptr, e1 = nullptr; int rc = -3;
+  if (hipMalloc(&sink, (size_t)blocks * G_THREADS * sizeof(int)) == hipSuccess && hipMalloc(&clocks, 2 * sizeof(long long)) == hipSuccess &&
+      hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess) {
+    mfma_ceiling_kernel<<<blocks, G_THREADS, 0, stream>>>(iters / 8 + 1, random, sink, clocks);   /* warm-up, lets the clock settle */
+    (void)hipEventRecord(e0, stream);
+    mfma_ceiling_kernel<<<blocks, G_THREADS, 0, stream>>>(iters, random, sink, clocks);
+    (void)hipEventRecord(e1, stream);
+    long long h[2] = { 0, 1 }; float ms = 0.f;
+    if (hipEventSynchronize(e1) == hipSuccess && hipEventElapsedTime(&ms, e0, e1) == hipSuccess && hipMemcpy(h, clocks, sizeof(h), hipMemcpyDeviceToHost) == hipSuccess && ms > 0.f) {
+      if (teraOps) { *teraOps = (double)blocks * 4. * (double)iters * 16. * 65536. / ((double)ms * 1e-3) / 1e12; }
+      if (clockGHz) { *clockGHz = h[1] > 0 ? (double)h[0] / (double)h[1] * 0.1 : 0.; }   /* wall clock counts at 100 MHz */
+      rc = 0;
+    }
+  }
+  if (e0) { (void)hipEventDestroy(e0); } if (e1) { (void)hipEventDestroy(e1); } if (sink) { (void)hipFree(sink); } if (clocks) { (void)hipFree(clocks); }
+  return rc;
+}
+
 extern "C" int hykGramSetSlab(int32_t bk) { if (bk != 0 && bk != 64 && bk != 128) { return -1; } g_bk = bk; return 0; }
 
 extern "C" size_t hykGramWorkspaceBytes(int32_t kind, int32_t Complex, int32_t N, int32_t orderA) {

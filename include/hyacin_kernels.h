@@ -54,8 +54,15 @@ int hykGramLimbs(hipStream_t stream, int32_t Complex, int32_t N, int32_t orderA,
 int hykGramProfile(int32_t enable);
 int hykGramProfileRead(double* totalMs, int32_t* launches);
 
-/* K slab staged in LDS per step of the Gram kernel: 64 or 128 bytes (tuning knob; default 64). */
+/* Variant of the contraction kernel (tuning knob): 0 = operand slabs loaded straight from global memory into a ring of
+ * LDS stages (default); 64 / 128 = staged through registers with that many K bytes per LDS stage. */
 int hykGramSetSlab(int32_t bk);
+
+/* Measurement hook (no counterpart in the reference): int8 tera-ops per second that a register-only loop of
+ * v_mfma_i32_32x32x32_i8 sustains on `blocks` workgroups of four wavefronts, with pseudo-random (random != 0) or all-zero
+ * operands, and the shader clock in GHz it ran at.  The device lowers its clock under the power draw of busy matrix
+ * cores, so this -- not the data-sheet peak -- is what a perfect contraction kernel could reach.  Synchronises the stream. */
+int hykMfmaCeiling(hipStream_t stream, int32_t blocks, int32_t iters, int32_t random, double* teraOps, double* clockGHz);
 
 /* Bit length of the dominant diagonal entry of the integer Gram.  Replaces gram_range_kernel, src/fp_i63tp_dequantize.cu:17-26. */
 int hykGramRange(hipStream_t stream, int32_t N, int32_t orderC, const uint64_t* C, const int32_t* vexp, int32_t* out);
@@ -87,7 +94,7 @@ int hykMatcopy(hipStream_t stream, char mode, int64_t M, int64_t N, int32_t srcT
 /* *out += sum of squares.  Replaces cublasDnrm2_64, src/lra.cpp:170,204. */
 int hykSumSquares(hipStream_t stream, int64_t M, int64_t N, const double* A, int64_t lda, double* out);
 
-/* Complex FP16 matrix product C = op(A) B on interleaved half pairs, FP32 accumulation on the MFMA units.
+/* Complex FP16 matrix product C = op(A) B on interleaved half pairs, FP32 accumulation (LDS-tiled vector-ALU kernel).
  * Replaces internal::matmul_cf16_{cn,tn,nn}, src/matmul_fp16_complex.cu:21-89. opA: 'N', 'T' or 'C'. */
 int hykMatmulCf16(hipStream_t stream, char opA, int32_t M, int32_t N, int32_t K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C, int64_t ldc);
 
@@ -96,8 +103,9 @@ int hykMatmulCf16(hipStream_t stream, char opA, int32_t M, int32_t N, int32_t K,
  * alpha/beta are real scalars. opA 'N' | 'T' | 'C', opB 'N' | 'T' | 'C'. */
 int hykGemm(hipStream_t stream, char opA, char opB, int32_t M, int32_t N, int32_t K, double alpha, int32_t type, const void* A, int64_t lda, const void* B, int64_t ldb, double beta, void* C, int64_t ldc);
 
-/* Householder QR, Q factor only: V (N x r, FP64 or complex FP64, interleaved) is overwritten by an orthonormal basis of
- * its column space.  Replaces cuSOLVER geqrf + orgqr/ungqr, src/lra.cpp:176-191. work: r * sizeof(element) + 64 bytes. */
+/* V (N x r, FP64 or complex FP64, interleaved) is overwritten by an orthonormal basis of its column space (one-sided
+ * Jacobi rotations, then column normalisation).  Replaces the Q factor of cuSOLVER geqrf + orgqr/ungqr,
+ * src/lra.cpp:176-191: the same subspace, a different basis of it.  work: r * sizeof(element) + 64 bytes. */
 int hykOrthonormalize(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* V, int64_t ldv, double* work);
 
 #ifdef __cplusplus
