@@ -21,11 +21,17 @@ namespace hyh {
 inline bool is_complex(int t) { return (t & 1) != 0; }
 inline int elem_bytes(int t) { static const int b[12] = { 8, 16, 4, 8, 2, 4, 16, 32, 12, 24, 16, 32 }; return (t >= 0 && t < 12) ? b[t] : 0; }
 
-/* stream-ordered scratch from the handle's pool (reference: cudaMallocFromPoolAsync / cudaFreeAsync throughout) */
+/* Stream-ordered scratch from the handle's pool (reference: cudaMallocFromPoolAsync / cudaFreeAsync throughout).
+ * When the handle owns its pool, blocks are kept and reused instead of being returned after every call: the runtime's
+ * pool calls cost up to a millisecond each for multi-gigabyte blocks, more than the kernels between them.  All work of a
+ * handle is ordered on its one stream, so a reused block is never touched by two calls at once.  hyacinDestroy frees them. */
+void* scratch_acquire(const hyacinHandle_t* h, size_t bytes, bool* kept);
+void scratch_release(const hyacinHandle_t* h, void* p, bool kept);
+void scratch_drop_all(const hyacinHandle_t* h);
 struct Scratch {
-  const hyacinHandle_t* h; void* p = nullptr;
-  Scratch(const hyacinHandle_t* h_, size_t bytes) : h(h_) { if (bytes) { HYH_CHECK(hipMallocFromPoolAsync(&p, bytes, h->mempool, h->hipStream)); } }
-  ~Scratch() { if (p) { HYH_CHECK(hipFreeAsync(p, h->hipStream)); } }
+  const hyacinHandle_t* h; void* p = nullptr; bool kept = false;
+  Scratch(const hyacinHandle_t* h_, size_t bytes) : h(h_) { if (bytes) { p = scratch_acquire(h, bytes, &kept); } }
+  ~Scratch() { if (p) { scratch_release(h, p, kept); } }
   Scratch(const Scratch&) = delete; Scratch& operator=(const Scratch&) = delete;
   template <typename T> T* as() const { return reinterpret_cast<T*>(p); }
 };

@@ -8,6 +8,8 @@
  */
 #include <cstring>
 #include <string>
+#include <map>
+#include <mutex>
 #include "common.hpp"
 
 namespace {
@@ -15,6 +17,10 @@ namespace {
 constexpr uint32_t OWNS_MEMPOOL = 0x4, OWNS_PINNED = 0x8, OWNS_TIMER = 0x10;   /* bit values of src/utils.cpp:45-49 */
 
 struct EventTimer { std::vector<std::pair<hyh::Segment, hipEvent_t>> events; hyh::Segment last = hyh::Segment::untimed; };
+
+/* blocks kept per handle-owned pool */
+struct Block { void* p; size_t bytes; bool busy; };
+std::mutex g_keptMutex; std::map<hipMemPool_t, std::vector<Block>> g_kept;
 
 bool env_get(const char* key, std::string& out) { const char* v = std::getenv(key); if (!v) { return false; } out = v; return true; }
 bool env_true(const std::string& s) { return s == "1" || s == "true" || s == "True"; }
@@ -53,8 +59,42 @@ extern "C" void hyacinCreate(hyacinHandle_t* handle) {
   if (verbose && handle->logger == nullptr) { handle->logger = stdout; }
 }
 
+void* hyh::scratch_acquire(const hyacinHandle_t* h, size_t bytes, bool* kept) {
+  void* p = nullptr; *kept = false;
+  if ((h->HandleOwnedResource & OWNS_MEMPOOL) && h->mempool) {
+    std::lock_guard<std::mutex> lock(g_keptMutex);
+    std::vector<Block>& blocks = g_kept[h->mempool]; Block* best = nullptr;
+    for (Block& b : blocks) { if (!b.busy && b.bytes >= bytes && b.bytes / 4 <= bytes && (!best || b.bytes < best->bytes)) { best = &b; } }
+    if (best) { best->busy = true; *kept = true; return best->p; }
+    if (blocks.size() >= 64) {   /* many different sizes have come by: return the idle ones to the pool */
+      std::vector<Block> live; for (Block& b : blocks) { if (b.busy) { live.push_back(b); } else { HYH_CHECK(hipFreeAsync(b.p, h->hipStream)); } } blocks.swap(live);
+    }
+    const size_t rounded = (bytes + 255) / 256 * 256;
+    HYH_CHECK(hipMallocFromPoolAsync(&p, rounded, h->mempool, h->hipStream));
+    if (p) { blocks.push_back(Block{ p, rounded, true }); *kept = true; }
+    return p;
+  }
+  HYH_CHECK(hipMallocFromPoolAsync(&p, bytes, h->mempool, h->hipStream));
+  return p;
+}
+
+void hyh::scratch_release(const hyacinHandle_t* h, void* p, bool kept) {
+  if (!kept) { HYH_CHECK(hipFreeAsync(p, h->hipStream)); return; }
+  std::lock_guard<std::mutex> lock(g_keptMutex);
+  auto it = g_kept.find(h->mempool); if (it == g_kept.end()) { return; }
+  for (Block& b : it->second) { if (b.p == p) { b.busy = false; return; } }
+}
+
+void hyh::scratch_drop_all(const hyacinHandle_t* h) {
+  std::lock_guard<std::mutex> lock(g_keptMutex);
+  auto it = g_kept.find(h->mempool); if (it == g_kept.end()) { return; }
+  for (Block& b : it->second) { HYH_CHECK(hipFreeAsync(b.p, h->hipStream)); }
+  g_kept.erase(it);
+}
+
 extern "C" void hyacinDestroy(hyacinHandle_t* handle) {
   if (!handle) { return; }
+  if ((handle->HandleOwnedResource & OWNS_MEMPOOL) && handle->mempool) { hyh::scratch_drop_all(handle); }
   HYH_CHECK(hipDeviceSynchronize());
   if ((handle->HandleOwnedResource & OWNS_MEMPOOL) && handle->mempool) { HYH_CHECK(hipMemPoolDestroy(handle->mempool)); }
   if ((handle->HandleOwnedResource & OWNS_PINNED) && handle->pinnedWorkspace) { HYH_CHECK(hipHostFree(handle->pinnedWorkspace)); }
