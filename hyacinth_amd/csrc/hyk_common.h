@@ -84,11 +84,7 @@ HYK_HD I96 round_scaled(Dec d, int32_t expon) {
 }
 
 /* ---------------------------------------------------------------- modular reduction */
-struct Mod { uint32_t m, d, c16, c32, c48, c64, c80; };  /* d = floor(2^32 / m); c_k = 2^k mod m */
-
 HYK_HD constexpr uint32_t pow2_mod(uint32_t k, uint32_t m) { uint32_t r = 1u % m; for (uint32_t i = 0; i < k; ++i) { r = (r * 2u) % m; } return r; }
-HYK_HD constexpr Mod make_mod(uint32_t m) { return Mod{ m, (uint32_t)(0x100000000ull / m), pow2_mod(16, m), pow2_mod(32, m), pow2_mod(48, m), pow2_mod(64, m), pow2_mod(80, m) }; }
-
 HYK_HD uint32_t umulhi32(uint32_t a, uint32_t b) {
 #if defined(__HIP_DEVICE_COMPILE__)
   return __umulhi(a, b);
@@ -104,18 +100,63 @@ HYK_HD uint32_t reduce_i32(int32_t v, uint32_t m, uint32_t d, uint32_t c32) {
   uint32_t r = reduce_u32((uint32_t)v, m, d); if (v < 0) { r = (r >= c32) ? (r - c32) : (r + m - c32); } return r;
 }
 
-/* canonical |q| mod m folded with the sign; WORDS = number of 16-bit words of |q| that can be non-zero (1..6) */
-template <int WORDS> HYK_HD uint32_t reduce_i96(I96 q, const Mod& k) {
-  uint32_t neg = q.hi >> 31; I96 a = neg ? i96_neg(q) : q;
-  uint32_t w0 = (uint32_t)a.lo, w1 = (uint32_t)(a.lo >> 32), w2 = a.hi;
-  uint32_t t = w0 & 0xffffu;
-  if (WORDS > 1) { t += k.c16 * (w0 >> 16); }
-  if (WORDS > 2) { t += k.c32 * (w1 & 0xffffu); }
-  if (WORDS > 3) { t += k.c48 * (w1 >> 16); }
-  if (WORDS > 4) { t += k.c64 * (w2 & 0xffffu); }
-  if (WORDS > 5) { t += k.c80 * (w2 >> 16); }
-  uint32_t r = reduce_u32(t, k.m, k.d);
-  return (neg && r) ? (k.m - r) : r;
+/* ---------------------------------------------------------------- residues through byte dot products
+ * For a modulus m <= 256 every power 2^(8 i) mod m fits a byte, so the residue of a multi-byte non-negative integer is
+ * the dot product of its bytes with those constants, reduced once more.  A signed q is first biased by 2^(32 DOTS - 1)
+ * (a flip of the top bit of its DOTS-dword two's complement), which makes it non-negative; the bias and the centring of
+ * the stored value are folded into one constant addend. */
+struct DotMod { uint32_t m; uint32_t cv[3]; float inv, halfInv; uint32_t bias[3]; };   /* bias[d - 1] = -2^(32 d - 1) mod m */
+
+HYK_HD constexpr uint32_t pack_pow2(uint32_t first, uint32_t m) {
+  return pow2_mod(first, m) | (pow2_mod(first + 8, m) << 8) | (pow2_mod(first + 16, m) << 16) | (pow2_mod(first + 24, m) << 24);
+}
+HYK_HD constexpr DotMod make_dotmod(uint32_t m) {
+  return DotMod{ m, { pack_pow2(0, m), pack_pow2(32, m), pack_pow2(64, m) }, 1.0f / (float)m, 0.5f / (float)m,
+                 { (m - pow2_mod(31, m)) % m, (m - pow2_mod(63, m)) % m, (m - pow2_mod(95, m)) % m } };
+}
+
+/* sum of the four byte products + c */
+HYK_HD uint32_t udot4(uint32_t a, uint32_t b, uint32_t c) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return __builtin_amdgcn_udot4(a, b, c, false);
+#else
+  for (int i = 0; i < 4; ++i) { c += ((a >> (8 * i)) & 0xffu) * ((b >> (8 * i)) & 0xffu); } return c;
+#endif
+}
+
+/* canonical t mod m for t < 2^20: the quotient comes from one float multiply-add; the half-unit offset keeps the product
+ * at least 1/(2m) away from an integer, far more than the rounding error for t < 2^22, so truncation gives floor(t / m) */
+HYK_HD uint32_t reduce_small(uint32_t t, const DotMod& k) {
+  const uint32_t q = (uint32_t)((float)t * k.inv + k.halfInv); return t - q * k.m;
+}
+
+/* canonical (q + addend) mod m of a signed q with |q| < 2^(32 DOTS - 1); addend < 2^10 */
+template <int DOTS> HYK_HD uint32_t residue_dot(I96 q, const DotMod& k, uint32_t addend) {
+  const uint32_t w0 = (uint32_t)q.lo, w1 = (uint32_t)(q.lo >> 32), w2 = q.hi;
+  uint32_t t = udot4(DOTS == 1 ? (w0 ^ 0x80000000u) : w0, k.cv[0], k.bias[DOTS - 1] + addend);
+  if (DOTS > 1) { t = udot4(DOTS == 2 ? (w1 ^ 0x80000000u) : w1, k.cv[1], t); }
+  if (DOTS > 2) { t = udot4(w2 ^ 0x80000000u, k.cv[2], t); }
+  return reduce_small(t, k);
+}
+
+/* The int8 the reference stores for a canonical residue r: r itself up to 127, r - m above.  For any t congruent to r,
+ * ((t + c) mod m) - c with c = max(m - 128, 0) is that value: it lies in [-c, m - 1 - c] = [128 - m, 127] (m > 128). */
+HYK_HD constexpr uint32_t stored_centre(uint32_t m) { return m > 128u ? m - 128u : 0u; }
+template <int DOTS> HYK_HD int32_t stored_residue_dot(I96 q, const DotMod& k) {
+  return (int32_t)residue_dot<DOTS>(q, k, stored_centre(k.m)) - (int32_t)stored_centre(k.m);
+}
+
+/* ---------------------------------------------------------------- residues in double precision
+ * For |a| < 2^51 the integer a is exact in a double and  a - m * rint((a - delta) / m)  is the representative of a mod m
+ * in [delta - (m-1)/2, delta + (m-1)/2]: the quotient is computed with an error below 2^-10 while (a - delta) / m stays at
+ * least 1/(2m) >= 2^-9 away from a rounding tie (m odd, or m = 256 with a half-integer delta), so rint never picks the
+ * wrong neighbour, and the final multiply-add is exact.  Three full-rate FP64 instructions per residue. */
+struct F64Mod { double inv, tieShift, negM; };   /* 1/m, -delta/m, -m */
+HYK_HD constexpr double stored_delta(uint32_t m) { return (m > 128u ? 128.0 - (double)m : 0.0) + ((double)m - 1.0) * 0.5; }  /* range [128 - m, 127] or [0, m - 1] */
+HYK_HD constexpr F64Mod make_f64mod(uint32_t m, double delta) { return F64Mod{ 1.0 / (double)m, -delta / (double)m, -(double)m }; }
+HYK_HD double residue_f64(double a, const F64Mod& k) {
+  const double quot = __builtin_rint(__builtin_fma(a, k.inv, k.tieShift));
+  return __builtin_fma(k.negM, quot, a);
 }
 
 /* residue stored in int8: values above 127 wrap by -m (reference: src/quantize_crt_real.cu:33) */

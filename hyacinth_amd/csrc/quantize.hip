@@ -29,13 +29,39 @@ namespace {
 constexpr int Q_THREADS = 256;
 constexpr int Q_ROWS = 4;
 
-/* loaders: element -> decomposed real / imaginary parts */
-struct ElemF64 { static constexpr int cplx = 0; using T = uint64_t; static __device__ __forceinline__ void load(const T* p, hyk::Dec& re, hyk::Dec& im) { re = hyk::decompose_f64(*p); im = hyk::Dec{ 0, 0, 0 }; } };
-struct ElemF32 { static constexpr int cplx = 0; using T = uint32_t; static __device__ __forceinline__ void load(const T* p, hyk::Dec& re, hyk::Dec& im) { re = hyk::decompose_f32(*p); im = hyk::Dec{ 0, 0, 0 }; } };
-struct ElemF16 { static constexpr int cplx = 0; using T = uint16_t; static __device__ __forceinline__ void load(const T* p, hyk::Dec& re, hyk::Dec& im) { re = hyk::decompose_f16(*p); im = hyk::Dec{ 0, 0, 0 }; } };
-struct ElemF64C { static constexpr int cplx = 1; using T = ulonglong2; static __device__ __forceinline__ void load(const T* p, hyk::Dec& re, hyk::Dec& im) { T v = *p; re = hyk::decompose_f64(v.x); im = hyk::decompose_f64(v.y); } };
-struct ElemF32C { static constexpr int cplx = 1; using T = uint2; static __device__ __forceinline__ void load(const T* p, hyk::Dec& re, hyk::Dec& im) { T v = *p; re = hyk::decompose_f32(v.x); im = hyk::decompose_f32(v.y); } };
-struct ElemF16C { static constexpr int cplx = 1; using T = uint32_t; static __device__ __forceinline__ void load(const T* p, hyk::Dec& re, hyk::Dec& im) { T v = *p; re = hyk::decompose_f16(v & 0xffffu); im = hyk::decompose_f16(v >> 16); } };
+__device__ __forceinline__ float half_bits(uint16_t b) { __half_raw r; r.x = b; return __half2float(__half(r)); }
+
+/* loaders: element -> decomposed real / imaginary parts (integer path) or doubles (FP64 residue path) */
+struct ElemF64 { static constexpr int cplx = 0; using T = uint64_t; static __device__ __forceinline__ void load(const T* p, hyk::Dec& re, hyk::Dec& im) { re = hyk::decompose_f64(*p); im = hyk::Dec{ 0, 0, 0 }; }
+  static __device__ __forceinline__ void load_f64(const T* p, double& re, double& im) { re = __longlong_as_double((long long)*p); im = 0.; } };
+struct ElemF32 { static constexpr int cplx = 0; using T = uint32_t; static __device__ __forceinline__ void load(const T* p, hyk::Dec& re, hyk::Dec& im) { re = hyk::decompose_f32(*p); im = hyk::Dec{ 0, 0, 0 }; }
+  static __device__ __forceinline__ void load_f64(const T* p, double& re, double& im) { re = (double)__uint_as_float(*p); im = 0.; } };
+struct ElemF16 { static constexpr int cplx = 0; using T = uint16_t; static __device__ __forceinline__ void load(const T* p, hyk::Dec& re, hyk::Dec& im) { re = hyk::decompose_f16(*p); im = hyk::Dec{ 0, 0, 0 }; }
+  static __device__ __forceinline__ void load_f64(const T* p, double& re, double& im) { re = (double)half_bits(*p); im = 0.; } };
+struct ElemF64C { static constexpr int cplx = 1; using T = ulonglong2; static __device__ __forceinline__ void load(const T* p, hyk::Dec& re, hyk::Dec& im) { T v = *p; re = hyk::decompose_f64(v.x); im = hyk::decompose_f64(v.y); }
+  static __device__ __forceinline__ void load_f64(const T* p, double& re, double& im) { T v = *p; re = __longlong_as_double((long long)v.x); im = __longlong_as_double((long long)v.y); } };
+struct ElemF32C { static constexpr int cplx = 1; using T = uint2; static __device__ __forceinline__ void load(const T* p, hyk::Dec& re, hyk::Dec& im) { T v = *p; re = hyk::decompose_f32(v.x); im = hyk::decompose_f32(v.y); }
+  static __device__ __forceinline__ void load_f64(const T* p, double& re, double& im) { T v = *p; re = (double)__uint_as_float(v.x); im = (double)__uint_as_float(v.y); } };
+struct ElemF16C { static constexpr int cplx = 1; using T = uint32_t; static __device__ __forceinline__ void load(const T* p, hyk::Dec& re, hyk::Dec& im) { T v = *p; re = hyk::decompose_f16(v & 0xffffu); im = hyk::decompose_f16(v >> 16); }
+  static __device__ __forceinline__ void load_f64(const T* p, double& re, double& im) { T v = *p; re = (double)half_bits((uint16_t)(v & 0xffffu)); im = (double)half_bits((uint16_t)(v >> 16)); } };
+
+/* The Q_ROWS consecutive elements of a thread: full, 16-byte aligned groups come in as 16-byte non-temporal vector loads
+ * issued back to back (A is read exactly once); ragged or unaligned groups element by element; missing rows read as zero. */
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+template <typename T>
+__device__ __forceinline__ void fetch_rows(const T* __restrict__ src, int valid, T (&tmp)[Q_ROWS]) {
+  constexpr int BYTES = (int)sizeof(T) * Q_ROWS;
+  if (valid == Q_ROWS && ((uintptr_t)src & (BYTES >= 16 ? 15u : 7u)) == 0) {
+    if constexpr (BYTES >= 16) {
+      #pragma unroll
+      for (int i = 0; i < BYTES / 16; ++i) { reinterpret_cast<u32x4*>(tmp)[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(src) + i); }
+    } else { *reinterpret_cast<u32x2*>(tmp) = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(src)); }
+  } else {
+    #pragma unroll
+    for (int r = 0; r < Q_ROWS; ++r) { tmp[r] = T{}; if (r < valid) { tmp[r] = src[r]; } }
+  }
+}
 
 __device__ __forceinline__ void store_panel(int8_t* dst, uint32_t packed, int valid, bool aligned) {
   if (aligned && valid == Q_ROWS) { *reinterpret_cast<uint32_t*>(dst) = packed; }
@@ -51,10 +77,10 @@ __global__ __launch_bounds__(Q_THREADS) void quantize_limbs_kernel(int32_t M, in
   int8_t* out = B + (int64_t)j * ldb + i0; const bool aligned = ((uintptr_t)out & 3u) == 0;
   constexpr int GROUPS = E::cplx ? 3 : 1;
   if (expon == HYK_INT_MAX) { for (int p = 0; p < order * GROUPS; ++p) { store_panel(out + p * strideB, 0u, valid, aligned); } return; }
-  hyk::I96 q[GROUPS][Q_ROWS];
+  hyk::I96 q[GROUPS][Q_ROWS]; typename E::T raw[Q_ROWS]; fetch_rows(&A[(int64_t)j * lda + i0], valid, raw);
   #pragma unroll
   for (int r = 0; r < Q_ROWS; ++r) {
-    hyk::Dec re{ 0, 0, 0 }, im{ 0, 0, 0 }; if (r < valid) { E::load(&A[(int64_t)j * lda + i0 + r], re, im); }
+    hyk::Dec re{ 0, 0, 0 }, im{ 0, 0, 0 }; E::load(&raw[r], re, im);
     if constexpr (E::cplx) { hyk::I96 a = hyk::round_scaled(re, expon), b = hyk::round_scaled(im, expon); q[0][r] = hyk::i96_add(a, b); q[1][r] = a; q[2][r] = b; }
     else { q[0][r] = hyk::round_scaled(re, expon); }
   }
@@ -74,46 +100,48 @@ __global__ __launch_bounds__(Q_THREADS) void quantize_limbs_kernel(int32_t M, in
 }
 
 /* ------------------------------------------------------------------ CRT */
-template <int X> struct RealMod { static constexpr hyk::Mod k = hyk::make_mod(hyk_crt_real_mo[X]); };
-template <int X> struct CplxMod { static constexpr hyk::Mod k = hyk::make_mod(hyk_crt_cplx_mo[X]); static constexpr uint32_t im = hyk_crt_cplx_im[X]; };
+/* DOTS = dwords of the biased two's complement of q that the byte dot products cover: |q| < 2^(32 DOTS - 1) */
+template <int X> struct RealMod { static constexpr hyk::DotMod k = hyk::make_dotmod(hyk_crt_real_mo[X]); };
+template <int X> struct CplxMod { static constexpr hyk::DotMod k = hyk::make_dotmod(hyk_crt_cplx_mo[X]); static constexpr uint32_t im = hyk_crt_cplx_im[X]; };
 
-template <typename E, int WORDS, int X>
+template <typename E, int DOTS, int X>
 __device__ __forceinline__ void crt_real_step(int32_t order, const hyk::I96 (&q)[Q_ROWS], int8_t* out, int64_t strideB, int valid, bool aligned) {
   if constexpr (X < HYK_CRT_REAL_COUNT) {
     if (X < order) {
-      constexpr hyk::Mod k = RealMod<X>::k; uint32_t packed = 0;
+      constexpr hyk::DotMod k = RealMod<X>::k; uint32_t packed = 0;
       #pragma unroll
-      for (int r = 0; r < Q_ROWS; ++r) { packed |= ((uint32_t)(uint8_t)hyk::residue_to_i8(hyk::reduce_i96<WORDS>(q[r], k), k.m)) << (8 * r); }
+      for (int r = 0; r < Q_ROWS; ++r) { packed |= ((uint32_t)(uint8_t)hyk::stored_residue_dot<DOTS>(q[r], k)) << (8 * r); }
       store_panel(out + (int64_t)X * strideB, packed, valid, aligned);
-      crt_real_step<E, WORDS, X + 1>(order, q, out, strideB, valid, aligned);
+      crt_real_step<E, DOTS, X + 1>(order, q, out, strideB, valid, aligned);
     }
   }
 }
 
-template <typename E, int WORDS>
+template <typename E, int DOTS>
 __global__ __launch_bounds__(Q_THREADS) void quantize_crt_real_kernel(int32_t M, int32_t order, const typename E::T* __restrict__ A, int64_t lda, const int32_t* __restrict__ vexp, int8_t* __restrict__ B, int64_t ldb, int64_t strideB) {
   const int32_t j = blockIdx.y; const int64_t i0 = ((int64_t)blockIdx.x * Q_THREADS + threadIdx.x) * Q_ROWS;
   if (i0 >= M) { return; }
   const int valid = (M - i0) < Q_ROWS ? (int)(M - i0) : Q_ROWS; const int32_t expon = vexp[j];
   int8_t* out = B + (int64_t)j * ldb + i0; const bool aligned = ((uintptr_t)out & 3u) == 0;
   if (expon == HYK_INT_MAX) { for (int p = 0; p < order; ++p) { store_panel(out + p * strideB, 0u, valid, aligned); } return; }
-  hyk::I96 q[Q_ROWS];
+  hyk::I96 q[Q_ROWS]; typename E::T raw[Q_ROWS]; fetch_rows(&A[(int64_t)j * lda + i0], valid, raw);
   #pragma unroll
-  for (int r = 0; r < Q_ROWS; ++r) { hyk::Dec re{ 0, 0, 0 }, im{ 0, 0, 0 }; if (r < valid) { E::load(&A[(int64_t)j * lda + i0 + r], re, im); } q[r] = hyk::round_scaled(re, expon); }
-  crt_real_step<E, WORDS, 0>(order, q, out, strideB, valid, aligned);
+  for (int r = 0; r < Q_ROWS; ++r) { hyk::Dec re{ 0, 0, 0 }, im{ 0, 0, 0 }; E::load(&raw[r], re, im); q[r] = hyk::round_scaled(re, expon); }
+  crt_real_step<E, DOTS, 0>(order, q, out, strideB, valid, aligned);
 }
 
-template <typename E, int WORDS, int X>
+template <typename E, int DOTS, int X>
 __device__ __forceinline__ void crt_cplx_step(int32_t order, const hyk::I96 (&qr)[Q_ROWS], const hyk::I96 (&qi)[Q_ROWS], int8_t* out, int64_t strideB, int valid, bool aligned) {
   if constexpr (X < HYK_CRT_CPLX_COUNT) {
     if (X < order) {
-      constexpr hyk::Mod k = CplxMod<X>::k; constexpr uint32_t im = CplxMod<X>::im; uint32_t p0 = 0, p1 = 0, p2 = 0;
+      constexpr hyk::DotMod k = CplxMod<X>::k; constexpr uint32_t im = CplxMod<X>::im, centre = hyk::stored_centre(k.m); uint32_t p0 = 0, p1 = 0, p2 = 0;
       #pragma unroll
       for (int r = 0; r < Q_ROWS; ++r) {
-        uint32_t a = hyk::reduce_i96<WORDS>(qr[r], k), b = hyk::reduce_i96<WORDS>(qi[r], k);
+        const uint32_t a = hyk::residue_dot<DOTS>(qr[r], k, 0u), b = hyk::residue_dot<DOTS>(qi[r], k, 0u);   /* canonical */
         if constexpr (X < HYK_CRT_CPLX_SPLIT) {
-          uint32_t p = hyk::reduce_u32(a + (k.m - im) * b, k.m, k.d), q = hyk::reduce_u32(a + im * b, k.m, k.d);
-          p0 |= ((uint32_t)(uint8_t)hyk::residue_to_i8(p, k.m)) << (8 * r); p1 |= ((uint32_t)(uint8_t)hyk::residue_to_i8(q, k.m)) << (8 * r);
+          /* (re -+ iota im) mod m, stored as the reference does: ((t + c) mod m) - c, c = max(m - 128, 0) */
+          const int32_t p = (int32_t)hyk::reduce_small(a + (k.m - im) * b + centre, k) - (int32_t)centre, q = (int32_t)hyk::reduce_small(a + im * b + centre, k) - (int32_t)centre;
+          p0 |= ((uint32_t)(uint8_t)p) << (8 * r); p1 |= ((uint32_t)(uint8_t)q) << (8 * r);
         } else {
           uint32_t s = a + b; s = s >= k.m ? s - k.m : s;
           p0 |= ((uint32_t)(uint8_t)hyk::residue_to_i8(s, k.m)) << (8 * r); p1 |= ((uint32_t)(uint8_t)hyk::residue_to_i8(a, k.m)) << (8 * r); p2 |= ((uint32_t)(uint8_t)hyk::residue_to_i8(b, k.m)) << (8 * r);
@@ -125,12 +153,12 @@ __device__ __forceinline__ void crt_cplx_step(int32_t order, const hyk::I96 (&qr
         constexpr int base = 2 * HYK_CRT_CPLX_SPLIT + 3 * (X - HYK_CRT_CPLX_SPLIT);
         store_panel(out + (int64_t)base * strideB, p0, valid, aligned); store_panel(out + (int64_t)(base + 1) * strideB, p1, valid, aligned); store_panel(out + (int64_t)(base + 2) * strideB, p2, valid, aligned);
       }
-      crt_cplx_step<E, WORDS, X + 1>(order, qr, qi, out, strideB, valid, aligned);
+      crt_cplx_step<E, DOTS, X + 1>(order, qr, qi, out, strideB, valid, aligned);
     }
   }
 }
 
-template <typename E, int WORDS>
+template <typename E, int DOTS>
 __global__ __launch_bounds__(Q_THREADS) void quantize_crt_cplx_kernel(int32_t M, int32_t order, const typename E::T* __restrict__ A, int64_t lda, const int32_t* __restrict__ vexp, int8_t* __restrict__ B, int64_t ldb, int64_t strideB) {
   const int32_t j = blockIdx.y; const int64_t i0 = ((int64_t)blockIdx.x * Q_THREADS + threadIdx.x) * Q_ROWS;
   if (i0 >= M) { return; }
@@ -138,10 +166,90 @@ __global__ __launch_bounds__(Q_THREADS) void quantize_crt_cplx_kernel(int32_t M,
   int8_t* out = B + (int64_t)j * ldb + i0; const bool aligned = ((uintptr_t)out & 3u) == 0;
   const int panels = order <= HYK_CRT_CPLX_SPLIT ? 2 * order : 3 * order - HYK_CRT_CPLX_SPLIT;
   if (expon == HYK_INT_MAX) { for (int p = 0; p < panels; ++p) { store_panel(out + p * strideB, 0u, valid, aligned); } return; }
-  hyk::I96 qr[Q_ROWS], qi[Q_ROWS];
+  hyk::I96 qr[Q_ROWS], qi[Q_ROWS]; typename E::T raw[Q_ROWS]; fetch_rows(&A[(int64_t)j * lda + i0], valid, raw);
   #pragma unroll
-  for (int r = 0; r < Q_ROWS; ++r) { hyk::Dec re{ 0, 0, 0 }, im{ 0, 0, 0 }; if (r < valid) { E::load(&A[(int64_t)j * lda + i0 + r], re, im); } qr[r] = hyk::round_scaled(re, expon); qi[r] = hyk::round_scaled(im, expon); }
-  crt_cplx_step<E, WORDS, 0>(order, qr, qi, out, strideB, valid, aligned);
+  for (int r = 0; r < Q_ROWS; ++r) { hyk::Dec re{ 0, 0, 0 }, im{ 0, 0, 0 }; E::load(&raw[r], re, im); qr[r] = hyk::round_scaled(re, expon); qi[r] = hyk::round_scaled(im, expon); }
+  crt_cplx_step<E, DOTS, 0>(order, qr, qi, out, strideB, valid, aligned);
+}
+
+/* ------------------------------------------------------------------ CRT, quantized values below 2^51
+ * q = rint(x * 2^vexp) is then exact in a double (ldexp and rint are exact operations), and every residue costs three
+ * FP64 instructions (hyk::residue_f64) instead of byte dot products and an integer reduction. */
+template <int X> struct RealF64 { static constexpr hyk::F64Mod k = hyk::make_f64mod(hyk_crt_real_mo[X], hyk::stored_delta(hyk_crt_real_mo[X])); };
+template <int X> struct CplxF64 {
+  static constexpr hyk::F64Mod stored = hyk::make_f64mod(hyk_crt_cplx_mo[X], hyk::stored_delta(hyk_crt_cplx_mo[X]));
+  static constexpr hyk::F64Mod sym = hyk::make_f64mod(hyk_crt_cplx_mo[X], 0.0);   /* any small representative */
+  static constexpr double im = (double)hyk_crt_cplx_im[X];
+};
+__device__ __forceinline__ uint32_t byte_of(double r) { return (uint32_t)(int32_t)r & 0xffu; }
+
+template <int X>
+__device__ __forceinline__ void crt_real_f64_step(int32_t order, const double (&a)[Q_ROWS], int8_t* out, int64_t strideB, int valid, bool aligned) {
+  if constexpr (X < HYK_CRT_REAL_COUNT) {
+    if (X < order) {
+      constexpr hyk::F64Mod k = RealF64<X>::k; uint32_t packed = 0;
+      #pragma unroll
+      for (int r = 0; r < Q_ROWS; ++r) { packed |= byte_of(hyk::residue_f64(a[r], k)) << (8 * r); }
+      store_panel(out + (int64_t)X * strideB, packed, valid, aligned);
+      crt_real_f64_step<X + 1>(order, a, out, strideB, valid, aligned);
+    }
+  }
+}
+
+template <typename E>
+__global__ __launch_bounds__(Q_THREADS) void quantize_crt_real_f64_kernel(int32_t M, int32_t order, const typename E::T* __restrict__ A, int64_t lda, const int32_t* __restrict__ vexp, int8_t* __restrict__ B, int64_t ldb, int64_t strideB) {
+  const int32_t j = blockIdx.y; const int64_t i0 = ((int64_t)blockIdx.x * Q_THREADS + threadIdx.x) * Q_ROWS;
+  if (i0 >= M) { return; }
+  const int valid = (M - i0) < Q_ROWS ? (int)(M - i0) : Q_ROWS; const int32_t expon = vexp[j];
+  int8_t* out = B + (int64_t)j * ldb + i0; const bool aligned = ((uintptr_t)out & 3u) == 0;
+  if (expon == HYK_INT_MAX) { for (int p = 0; p < order; ++p) { store_panel(out + p * strideB, 0u, valid, aligned); } return; }
+  double a[Q_ROWS]; typename E::T raw[Q_ROWS]; fetch_rows(&A[(int64_t)j * lda + i0], valid, raw);
+  #pragma unroll
+  for (int r = 0; r < Q_ROWS; ++r) { double re = 0., im = 0.; E::load_f64(&raw[r], re, im); a[r] = __builtin_rint(__builtin_ldexp(re, expon)); }
+  crt_real_f64_step<0>(order, a, out, strideB, valid, aligned);
+}
+
+template <int X>
+__device__ __forceinline__ void crt_cplx_f64_step(int32_t order, const double (&ar)[Q_ROWS], const double (&ai)[Q_ROWS], int8_t* out, int64_t strideB, int valid, bool aligned) {
+  if constexpr (X < HYK_CRT_CPLX_COUNT) {
+    if (X < order) {
+      using K = CplxF64<X>; uint32_t p0 = 0, p1 = 0, p2 = 0;
+      #pragma unroll
+      for (int r = 0; r < Q_ROWS; ++r) {
+        if constexpr (X < HYK_CRT_CPLX_SPLIT) {
+          const double ra = hyk::residue_f64(ar[r], K::sym), rb = hyk::residue_f64(ai[r], K::sym);   /* |ra|, |rb| <= m / 2 */
+          p0 |= byte_of(hyk::residue_f64(__builtin_fma(-K::im, rb, ra), K::stored)) << (8 * r);
+          p1 |= byte_of(hyk::residue_f64(__builtin_fma(K::im, rb, ra), K::stored)) << (8 * r);
+        } else {
+          p0 |= byte_of(hyk::residue_f64(ar[r] + ai[r], K::stored)) << (8 * r); p1 |= byte_of(hyk::residue_f64(ar[r], K::stored)) << (8 * r); p2 |= byte_of(hyk::residue_f64(ai[r], K::stored)) << (8 * r);
+        }
+      }
+      if constexpr (X < HYK_CRT_CPLX_SPLIT) {
+        store_panel(out + (int64_t)(2 * X) * strideB, p0, valid, aligned); store_panel(out + (int64_t)(2 * X + 1) * strideB, p1, valid, aligned);
+      } else {
+        constexpr int base = 2 * HYK_CRT_CPLX_SPLIT + 3 * (X - HYK_CRT_CPLX_SPLIT);
+        store_panel(out + (int64_t)base * strideB, p0, valid, aligned); store_panel(out + (int64_t)(base + 1) * strideB, p1, valid, aligned); store_panel(out + (int64_t)(base + 2) * strideB, p2, valid, aligned);
+      }
+      crt_cplx_f64_step<X + 1>(order, ar, ai, out, strideB, valid, aligned);
+    }
+  }
+}
+
+template <typename E>
+__global__ __launch_bounds__(Q_THREADS) void quantize_crt_cplx_f64_kernel(int32_t M, int32_t order, const typename E::T* __restrict__ A, int64_t lda, const int32_t* __restrict__ vexp, int8_t* __restrict__ B, int64_t ldb, int64_t strideB) {
+  const int32_t j = blockIdx.y; const int64_t i0 = ((int64_t)blockIdx.x * Q_THREADS + threadIdx.x) * Q_ROWS;
+  if (i0 >= M) { return; }
+  const int valid = (M - i0) < Q_ROWS ? (int)(M - i0) : Q_ROWS; const int32_t expon = vexp[j];
+  int8_t* out = B + (int64_t)j * ldb + i0; const bool aligned = ((uintptr_t)out & 3u) == 0;
+  const int panels = 2 * (order < HYK_CRT_CPLX_SPLIT ? order : HYK_CRT_CPLX_SPLIT) + 3 * (order > HYK_CRT_CPLX_SPLIT ? order - HYK_CRT_CPLX_SPLIT : 0);
+  if (expon == HYK_INT_MAX) { for (int p = 0; p < panels; ++p) { store_panel(out + p * strideB, 0u, valid, aligned); } return; }
+  double ar[Q_ROWS], ai[Q_ROWS]; typename E::T raw[Q_ROWS]; fetch_rows(&A[(int64_t)j * lda + i0], valid, raw);
+  #pragma unroll
+  for (int r = 0; r < Q_ROWS; ++r) {
+    double re = 0., im = 0.; E::load_f64(&raw[r], re, im);
+    ar[r] = __builtin_rint(__builtin_ldexp(re, expon)); ai[r] = __builtin_rint(__builtin_ldexp(im, expon));
+  }
+  crt_cplx_f64_step<0>(order, ar, ai, out, strideB, valid, aligned);
 }
 
 /* rows [row0, row1) of `panels` panels set to zero: the Gram kernel contracts over whole 128-row blocks */
@@ -176,17 +284,20 @@ extern "C" int hykQuantizeCrt(hipStream_t stream, int32_t M, int32_t N, int32_t 
   if (M <= 0 || N <= 0) { return 0; }
   const int cplx = Atype & 1;
   if (orderA < 1 || orderA > (cplx ? HYK_CRT_CPLX_COUNT : HYK_CRT_REAL_COUNT) || N > 65535 || ldb < M) { return -1; }
-  const int64_t strideB = (int64_t)N * ldb; HYK_QGRID; const bool narrow = (0 < maxBits && maxBits <= 48);
+  const int64_t strideB = (int64_t)N * ldb; HYK_QGRID; const int dots = (0 < maxBits && maxBits <= 31) ? 1 : (0 < maxBits && maxBits <= 63) ? 2 : 3;
+  const bool viaF64 = (0 < maxBits && maxBits <= 51);   /* |q|, and |re + im| for complex input, below 2^51: exact in a double */
   #define HYK_LAUNCH_CRT(KERNEL, ELEM, TYPE) \
-    if (narrow) { KERNEL<ELEM, 3><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const TYPE*)A, lda, vexp, B, ldb, strideB); } \
-    else { KERNEL<ELEM, 6><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const TYPE*)A, lda, vexp, B, ldb, strideB); }
+    if (viaF64) { KERNEL##_f64_kernel<ELEM><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const TYPE*)A, lda, vexp, B, ldb, strideB); } \
+    else if (dots == 1) { KERNEL##_kernel<ELEM, 1><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const TYPE*)A, lda, vexp, B, ldb, strideB); } \
+    else if (dots == 2) { KERNEL##_kernel<ELEM, 2><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const TYPE*)A, lda, vexp, B, ldb, strideB); } \
+    else { KERNEL##_kernel<ELEM, 3><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const TYPE*)A, lda, vexp, B, ldb, strideB); }
   switch (Atype) {
-    case HYK_F64: HYK_LAUNCH_CRT(quantize_crt_real_kernel, ElemF64, uint64_t) break;
-    case HYK_F32: HYK_LAUNCH_CRT(quantize_crt_real_kernel, ElemF32, uint32_t) break;
-    case HYK_F16: HYK_LAUNCH_CRT(quantize_crt_real_kernel, ElemF16, uint16_t) break;
-    case HYK_F64C: HYK_LAUNCH_CRT(quantize_crt_cplx_kernel, ElemF64C, ulonglong2) break;
-    case HYK_F32C: HYK_LAUNCH_CRT(quantize_crt_cplx_kernel, ElemF32C, uint2) break;
-    case HYK_F16C: HYK_LAUNCH_CRT(quantize_crt_cplx_kernel, ElemF16C, uint32_t) break;
+    case HYK_F64: HYK_LAUNCH_CRT(quantize_crt_real, ElemF64, uint64_t) break;
+    case HYK_F32: HYK_LAUNCH_CRT(quantize_crt_real, ElemF32, uint32_t) break;
+    case HYK_F16: HYK_LAUNCH_CRT(quantize_crt_real, ElemF16, uint16_t) break;
+    case HYK_F64C: HYK_LAUNCH_CRT(quantize_crt_cplx, ElemF64C, ulonglong2) break;
+    case HYK_F32C: HYK_LAUNCH_CRT(quantize_crt_cplx, ElemF32C, uint2) break;
+    case HYK_F16C: HYK_LAUNCH_CRT(quantize_crt_cplx, ElemF16C, uint32_t) break;
     default: return -1;
   }
   #undef HYK_LAUNCH_CRT

@@ -28,15 +28,35 @@ void hm_digits(int type, const void* x, int64_t n, int32_t expon, int order, int
   }
 }
 
-void hm_residues(int cplxTable, int words, int type, const void* x, int64_t n, int32_t expon, int order, int8_t* out) {
+void hm_residues(int cplxTable, int dots, int type, const void* x, int64_t n, int32_t expon, int order, int8_t* out) {
   for (int64_t i = 0; i < n; ++i) {
     I96 q = round_scaled(dec_of(type, x, i, 0), expon);
     for (int m = 0; m < order; ++m) {
-      Mod k = make_mod(cplxTable ? hyk_crt_cplx_mo[m] : hyk_crt_real_mo[m]);
-      uint32_t r = words == 3 ? reduce_i96<3>(q, k) : reduce_i96<6>(q, k);
-      out[i * order + m] = residue_to_i8(r, k.m);
+      DotMod k = make_dotmod(cplxTable ? hyk_crt_cplx_mo[m] : hyk_crt_real_mo[m]);
+      int32_t r = dots == 1 ? stored_residue_dot<1>(q, k) : dots == 2 ? stored_residue_dot<2>(q, k) : stored_residue_dot<3>(q, k);
+      out[i * order + m] = (int8_t)r;
     }
   }
+}
+
+/* stored residue and canonical residue of the 96-bit two's complement {lo, hi} for one modulus */
+void hm_residue_raw(uint64_t lo, uint32_t hi, int dots, uint32_t m, int32_t* stored, uint32_t* canonical) {
+  I96 q; q.lo = lo; q.hi = hi; DotMod k = make_dotmod(m);
+  *stored = dots == 1 ? stored_residue_dot<1>(q, k) : dots == 2 ? stored_residue_dot<2>(q, k) : stored_residue_dot<3>(q, k);
+  *canonical = dots == 1 ? residue_dot<1>(q, k, 0u) : dots == 2 ? residue_dot<2>(q, k, 0u) : residue_dot<3>(q, k, 0u);
+}
+
+/* FP64 residue path: out[i] = representative of a_i mod m in the stored range (mode 0) or the symmetric one (mode 1) */
+void hm_residue_f64(const double* a, int64_t n, uint32_t m, int mode, double* out) {
+  F64Mod k = make_f64mod(m, mode ? 0.0 : stored_delta(m));
+  for (int64_t i = 0; i < n; ++i) { out[i] = residue_f64(a[i], k); }
+}
+
+/* number of t in [0, limit) with reduce_small(t) != t mod m */
+int64_t hm_reduce_small_errors(uint32_t m, uint32_t limit) {
+  DotMod k = make_dotmod(m); int64_t bad = 0;
+  for (uint32_t t = 0; t < limit; ++t) { bad += (reduce_small(t, k) != t % m); }
+  return bad;
 }
 
 int32_t hm_frexp(int type, const void* x) {

@@ -64,17 +64,61 @@ def test_digits_and_residues(hm, tcode, dtype):
             hm.hm_digits(tcode, _p(xs), C.c_int64(len(xs)), C.c_int32(expon), order, _p(out))
             assert out.reshape(len(xs), order).tolist() == [cf.balanced_digits(v, order) for v in q]
         for table, moduli in ((0, cf.REAL_MODULI), (1, cf.CPLX_MODULI)):
-            for words in (3, 6):
+            for dots in (2, 3):
                 out = np.zeros(len(xs) * len(moduli), np.int8)
-                hm.hm_residues(table, words, tcode, _p(xs), C.c_int64(len(xs)), C.c_int32(expon), len(moduli), _p(out))
+                hm.hm_residues(table, dots, tcode, _p(xs), C.c_int64(len(xs)), C.c_int32(expon), len(moduli), _p(out))
                 assert out.reshape(len(xs), len(moduli)).tolist() == [[cf.signed_residue(v, m) for m in moduli] for v in q]
-    # wide values need all six 16-bit words
+    # wide values need all three dwords
     big = np.array([1.0, -1.0, 0.75, -0.3, 1 - 2.0**-52], dtype=np.float64).astype(dtype)
     for expon in (60, 75, 81):
         q = [cf.rne_scaled(float(v), expon) for v in big]
         out = np.zeros(len(big) * 24, np.int8)
-        hm.hm_residues(0, 6, tcode, _p(big), C.c_int64(len(big)), C.c_int32(expon), 24, _p(out))
+        hm.hm_residues(0, 3, tcode, _p(big), C.c_int64(len(big)), C.c_int32(expon), 24, _p(out))
         assert out.reshape(len(big), 24).tolist() == [[cf.signed_residue(v, m) for m in cf.REAL_MODULI] for v in q]
+
+
+def test_dot_residues_at_the_range_limits(hm):
+    """q at and next to +-(2^(32 dots - 1) - 1), the largest magnitudes a dot count may be used for, and small values."""
+    for dots in (1, 2, 3):
+        top = 2 ** (32 * dots - 1)
+        values = [0, 1, -1, 127, 128, -128, -129, 255, 256, -255, -256, top - 1, -(top - 1), -top, top // 2, -(top // 2) - 1, top - 12345, -(top - 54321)]
+        for m in sorted(set(cf.REAL_MODULI) | set(cf.CPLX_MODULI)):
+            for v in values:
+                w = v & (2 ** 96 - 1)
+                st, ca = C.c_int32(), C.c_uint32()
+                hm.hm_residue_raw(C.c_uint64(w & (2 ** 64 - 1)), C.c_uint32(w >> 64), dots, m, C.byref(st), C.byref(ca))
+                assert ca.value == v % m, (dots, m, v)
+                assert st.value == cf.signed_residue(v, m) or (m == 256 and (st.value - cf.signed_residue(v, m)) % 256 == 0), (dots, m, v)
+                assert min(0, 128 - m) <= st.value <= 127
+
+
+def test_f64_residues_below_2_pow_51(hm):
+    """Three-instruction FP64 residue: exact for every |a| < 2^51, in the reference's stored range, also next to the ties."""
+    rng = np.random.default_rng(29)
+    top = 2 ** 51
+    vals = [0, 1, -1, 127, 128, -128, -129, top - 1, -(top - 1), top - 2, -(top - 2)]
+    vals += [int(v) for v in rng.integers(-top + 1, top, 4000)] + [int(v) for v in rng.integers(-70000, 70000, 4000)]
+    for m in sorted(set(cf.REAL_MODULI) | set(cf.CPLX_MODULI)):
+        near = [k * m + h + d for k in (-(top // m) + 1, -3, 0, 5, top // m - 2) for h in (m // 2, -(m // 2), 127, 128 - m) for d in (-1, 0, 1)]
+        xs = [v for v in vals + near if abs(v) < top]
+        a = np.array(xs, dtype=np.float64)
+        assert [int(v) for v in a] == xs
+        out = np.zeros(len(xs))
+        hm.hm_residue_f64(_p(a), C.c_int64(len(xs)), C.c_uint32(m), 0, _p(out))
+        want = [cf.signed_residue(v, m) for v in xs]
+        got = [int(v) for v in out]
+        if m == 256:
+            assert all((g - w) % 256 == 0 and -128 <= g <= 127 for g, w in zip(got, want))
+        else:
+            assert got == want, m
+        hm.hm_residue_f64(_p(a), C.c_int64(len(xs)), C.c_uint32(m), 1, _p(out))
+        assert all((int(g) - v) % m == 0 and abs(g) <= m / 2 for g, v in zip(out, xs)), m
+
+
+def test_reduce_small_is_exact_below_2_pow_20(hm):
+    hm.hm_reduce_small_errors.restype = C.c_int64
+    for m in sorted(set(cf.REAL_MODULI) | set(cf.CPLX_MODULI)):
+        assert hm.hm_reduce_small_errors(C.c_uint32(m), C.c_uint32(1 << 20)) == 0, m
 
 
 def test_frexp_exponents(hm):
