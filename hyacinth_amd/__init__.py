@@ -16,7 +16,7 @@ except Exception:  # pragma: no cover
     torch = None
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libhyacin.so")
+LIB_PATH = os.environ.get("HYACIN_LIBRARY") or os.path.join(HERE, "libhyacin.so")   # override: another build of the same library
 
 F64, F64C, F32, F32C, F16, F16C, DD, DDC, TF, TFC, QF, QFC = range(12)
 GRAM_LIMBS, GRAM_CRT = 0, 1

@@ -257,6 +257,7 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_kernel(const GramArgs args)
  * read wait for all direct loads in flight.  Their completion is tracked by hand with the vector-memory counter: every
  * slab step issues exactly 8 loads per lane (past the end of the K range it re-requests the last slab into a stage
  * nobody reads again), so "slab j + 1 has landed" is always "at most 16 loads outstanding". */
+template <int V> using IC = std::integral_constant<int, V>;
 constexpr int DMA_BK = 64, DMA_STAGES = 4, DMA_TILE_BYTES = TILE * DMA_BK, DMA_STAGE_BYTES = 2 * DMA_TILE_BYTES;
 
 __device__ __forceinline__ void dma16(uint32_t ldsAddr, const int8_t* src) {
@@ -332,50 +333,62 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_dma_kernel(const GramArgs a
   };
   auto mm = [&](int n, int set) { const int a = n >> 2, b = n & 3; acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[set][a], fl[set][b], acc[a][b], 0, 0, 0); };
 
-  /* prologue: four slabs on their way, the first one landed and published, its first fragments requested */
+  /* A run of MFMAs with fragment reads paired to the first of them, closed for the scheduler so that the direct loads
+   * issued between runs stay where they are written. */
+  auto run = [&](auto mmFirst_, auto mmCount_, auto mmSet_, auto rdFirst_, auto rdCount_, auto rdSet_, auto rdKk_, uint32_t rdOff) {
+    constexpr int mmFirst = decltype(mmFirst_)::value, mmCount = decltype(mmCount_)::value, mmSet = decltype(mmSet_)::value;
+    constexpr int rdFirst = decltype(rdFirst_)::value, rdCount = decltype(rdCount_)::value, rdSet = decltype(rdSet_)::value, rdKk = decltype(rdKk_)::value;
+    #pragma unroll
+    for (int i = 0; i < rdCount; ++i) { rd(rdFirst + i, rdSet, rdKk, rdOff); }
+    #pragma unroll
+    for (int n = 0; n < mmCount; ++n) { mm(mmFirst + n, mmSet); }
+    #pragma unroll
+    for (int i = 0; i < rdCount; ++i) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); }
+    if constexpr (mmCount > rdCount) { __builtin_amdgcn_sched_group_barrier(0x008, mmCount - rdCount, 0); }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  auto load = [&](int i, uint32_t stageOff) { dma(i, stageOff); __builtin_amdgcn_sched_barrier(0); };
+
+  /* prologue: slabs 0..2 and the lane-operand half of slab 3 on their way, slab 0 landed and published, its first fragments requested */
   #pragma unroll
   for (int st = 0; st < DMA_STAGES; ++st) {
     if (st) { peek(); advance(); }
     #pragma unroll
-    for (int i = 0; i < 8; ++i) { dma(i, (uint32_t)st * DMA_STAGE_BYTES); }
+    for (int i = 0; i < (st == DMA_STAGES - 1 ? 4 : 8); ++i) { dma(i, (uint32_t)st * DMA_STAGE_BYTES); }
   }
-  asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+  asm volatile("s_waitcnt vmcnt(20)" ::: "memory");
   __syncthreads();
   #pragma unroll
   for (int i = 0; i < 8; ++i) { rd(i, 0, 0, 0u); }
   __builtin_amdgcn_s_waitcnt(0xC07F);
+  __builtin_amdgcn_sched_barrier(0);
 
+  /* Steady state, slab `it` in stage it % 4.  The eight loads of a slab are spread over a whole slab time (a burst of them
+   * stalls instruction issue behind the address unit): the A-operand half of slab it + 3 goes out under the first K step
+   * into the stage freed one slab ago, the lane-operand half of slab it + 4 under the second K step into stage `cur`. */
   for (int it = 0; it < iters; ++it) {
-    const uint32_t curOff = (uint32_t)(it & (DMA_STAGES - 1)) * DMA_STAGE_BYTES, nxtOff = (uint32_t)((it + 1) & (DMA_STAGES - 1)) * DMA_STAGE_BYTES;
-    /* first K step: MFMAs on set 0; the fragments of the second K step go into set 1 under the first eight of them, four
-     * more cover the latency of the last read before the barrier */
-    #pragma unroll
-    for (int i = 0; i < 8; ++i) { rd(i, 1, 1, curOff); }
+    const uint32_t curOff = (uint32_t)(it & (DMA_STAGES - 1)) * DMA_STAGE_BYTES, nxtOff = (uint32_t)((it + 1) & (DMA_STAGES - 1)) * DMA_STAGE_BYTES,
+                   prvOff = (uint32_t)((it + DMA_STAGES - 1) & (DMA_STAGES - 1)) * DMA_STAGE_BYTES;
+    /* first K step: MFMAs on set 0, fragments of the second K step into set 1 */
     peek();
-    #pragma unroll
-    for (int n = 0; n < 12; ++n) { mm(n, 0); }
-    #pragma unroll
-    for (int i = 0; i < 8; ++i) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); }
-    __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
-    __builtin_amdgcn_sched_barrier(0);
+    run(IC<0>{}, IC<3>{}, IC<0>{}, IC<0>{}, IC<3>{}, IC<1>{}, IC<1>{}, curOff); load(4, prvOff);
+    run(IC<3>{}, IC<3>{}, IC<0>{}, IC<3>{}, IC<3>{}, IC<1>{}, IC<1>{}, curOff); load(5, prvOff);
+    run(IC<6>{}, IC<3>{}, IC<0>{}, IC<6>{}, IC<2>{}, IC<1>{}, IC<1>{}, curOff); load(6, prvOff);
+    run(IC<9>{}, IC<2>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<1>{}, IC<1>{}, curOff); load(7, prvOff);
+    run(IC<11>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<1>{}, IC<1>{}, curOff);
     /* slab it + 1 has landed (own loads) and every wave is done reading stage `cur`: publish */
     asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
     __syncthreads();
     __builtin_amdgcn_sched_barrier(0);
-    #pragma unroll
-    for (int n = 12; n < 16; ++n) { mm(n, 0); }
+    run(IC<12>{}, IC<4>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<1>{}, IC<1>{}, curOff);
     advance();
     __builtin_amdgcn_sched_barrier(0);
-    /* second K step: MFMAs on set 1; first fragments of the next slab into set 0, then stage `cur` is refilled with slab it + 4 */
-    #pragma unroll
-    for (int i = 0; i < 8; ++i) { rd(i, 0, 0, nxtOff); }
-    #pragma unroll
-    for (int n = 0; n < 8; ++n) { mm(n, 1); }
-    #pragma unroll
-    for (int i = 0; i < 8; ++i) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); }
-    #pragma unroll
-    for (int n = 8; n < 16; ++n) { __builtin_amdgcn_sched_barrier(0); mm(n, 1); __builtin_amdgcn_sched_barrier(0); dma(n - 8, curOff); }
-    __builtin_amdgcn_sched_barrier(0);
+    /* second K step: MFMAs on set 1, first fragments of the next slab into set 0 */
+    run(IC<0>{}, IC<4>{}, IC<1>{}, IC<0>{}, IC<4>{}, IC<0>{}, IC<0>{}, nxtOff); load(0, curOff);
+    run(IC<4>{}, IC<4>{}, IC<1>{}, IC<4>{}, IC<4>{}, IC<0>{}, IC<0>{}, nxtOff); load(1, curOff);
+    run(IC<8>{}, IC<4>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<0>{}, nxtOff); load(2, curOff);
+    run(IC<12>{}, IC<3>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<0>{}, nxtOff); load(3, curOff);
+    run(IC<15>{}, IC<1>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<0>{}, nxtOff);
     __builtin_amdgcn_s_waitcnt(0xC07F);   /* lgkmcnt(0): set 0 was requested eight MFMAs ago; stating it here keeps waits out of the first K step */
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   /* no direct load may still be writing LDS when the workgroup ends */
