@@ -66,6 +66,7 @@ struct GramArgs {
   const int8_t* panels; int64_t ldb, panelStride;
   void* acc; int64_t planeStride;
   int32_t N, nT, tileCount, kLen, kSplits, K, groupCount, totalItems, itemsPerXcd;
+  int32_t exclusive;                /* 1: this launch's items are the only writers of their accumulator entries */
   uint32_t tileMagic, splitMagic;   /* floor(2^32 / d) + 1: x / d == mulhi(x, magic) while x * d < 2^32 (checked on the host); 0 for d == 1 */
   GramGroup groups[MAX_GROUPS];
   uint32_t pairs[MAX_PAIRS];  /* lanePanel | aPanel << 16 */
@@ -73,6 +74,37 @@ struct GramArgs {
 
 /* element (i, j) of a 32x32 MFMA result held in accumulator register r of a lane */
 __device__ __forceinline__ int acc_row(int r, int lane) { return ((r >> 2) << 3) + ((lane >> 5) << 2) + (r & 3); }
+
+/* Epilogue shared by the contraction kernels (expanded in place: the accumulators must stay in registers): lane
+ * dimension j <-> y (contiguous in the packed triangle), register dimension i <-> x.  Items that are the only writers of
+ * their accumulator entries (one K split, planes not shared between groups: EXCL) store; all others add atomically. */
+#define HYK_GRAM_PUT(TYPE, PLANE, VALUE) { TYPE* p_ = &dst[(int64_t)(PLANE) * args.planeStride + e]; if constexpr (EXCL_) { *p_ = (VALUE); } else { atomicAdd(p_, (VALUE)); } }
+#define HYK_GRAM_EPILOGUE(EXCL) { \
+  constexpr bool EXCL_ = (EXCL); const bool diagTile = (ta == tb); \
+  _Pragma("unroll") for (int a = 0; a < 4; ++a) { \
+    _Pragma("unroll") for (int b = 0; b < 4; ++b) { \
+      __builtin_amdgcn_sched_barrier(0);   /* one 32x32 block at a time: keeps the accumulator copies out of scratch */ \
+      const int y = y0 + wy * WAVE_TILE + b * 32 + (lane & 31); \
+      _Pragma("unroll") for (int r = 0; r < 16; ++r) { \
+        const int x = x0 + wx * WAVE_TILE + a * 32 + acc_row(r, lane); \
+        if (x < args.N && y < args.N && (!diagTile || y <= x)) { \
+          const int64_t e = hyk::tri_index(y, x); const int32_t w = acc[a][b][r]; \
+          if constexpr (EPI == EPI_MOD) { \
+            uint32_t* dst = reinterpret_cast<uint32_t*>(args.acc); \
+            const uint32_t v = hyk::reduce_i32(w, grp.m, grp.d, grp.c32); \
+            if (grp.mulRe) HYK_GRAM_PUT(uint32_t, grp.planeRe, grp.mulRe == 1u ? v : hyk::reduce_u32(v * grp.mulRe, grp.m, grp.d)) \
+            if (grp.mulIm) HYK_GRAM_PUT(uint32_t, grp.planeIm, grp.mulIm == 1u ? v : hyk::reduce_u32(v * grp.mulIm, grp.m, grp.d)) \
+          } else { \
+            unsigned long long* dst = reinterpret_cast<unsigned long long*>(args.acc); \
+            const unsigned long long pos = (unsigned long long)(long long)w, negv = (unsigned long long)(-(long long)w); \
+            if (grp.mulRe) HYK_GRAM_PUT(unsigned long long, grp.planeRe, grp.mulRe == 1u ? pos : negv) \
+            if (grp.mulIm) HYK_GRAM_PUT(unsigned long long, grp.planeIm, grp.mulIm == 1u ? pos : negv) \
+          } \
+        } \
+      } \
+    } \
+  } \
+}
 
 template <int BK> struct Slab {
   static constexpr int PITCH = BK;                      /* bytes per tile row in LDS, unpadded; 16-byte slots are XOR-swizzled per row */
@@ -219,33 +251,7 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_kernel(const GramArgs args)
   for (; it + 1 < iters; it += 2) { slab(std::integral_constant<int, 0>{}); slab(std::integral_constant<int, 1>{}); }
   if (it < iters) { slab(std::integral_constant<int, 0>{}); }
 
-  /* epilogue: lane dimension j <-> y (contiguous in the packed triangle), register dimension i <-> x */
-  const bool diagTile = (ta == tb);
-  #pragma unroll
-  for (int a = 0; a < 4; ++a) {
-    #pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      const int y = y0 + wy * WAVE_TILE + b * 32 + (lane & 31);
-      #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int x = x0 + wx * WAVE_TILE + a * 32 + acc_row(r, lane);
-        if (x < args.N && y < args.N && (!diagTile || y <= x)) {
-          const int64_t e = hyk::tri_index(y, x); const int32_t w = acc[a][b][r];
-          if constexpr (EPI == EPI_MOD) {
-            uint32_t* dst = reinterpret_cast<uint32_t*>(args.acc);
-            const uint32_t v = hyk::reduce_i32(w, grp.m, grp.d, grp.c32);
-            if (grp.mulRe) { atomicAdd(&dst[(int64_t)grp.planeRe * args.planeStride + e], grp.mulRe == 1u ? v : hyk::reduce_u32(v * grp.mulRe, grp.m, grp.d)); }
-            if (grp.mulIm) { atomicAdd(&dst[(int64_t)grp.planeIm * args.planeStride + e], grp.mulIm == 1u ? v : hyk::reduce_u32(v * grp.mulIm, grp.m, grp.d)); }
-          } else {
-            unsigned long long* dst = reinterpret_cast<unsigned long long*>(args.acc);
-            const unsigned long long pos = (unsigned long long)(long long)w, negv = (unsigned long long)(-(long long)w);
-            if (grp.mulRe) { atomicAdd(&dst[(int64_t)grp.planeRe * args.planeStride + e], grp.mulRe == 1u ? pos : negv); }
-            if (grp.mulIm) { atomicAdd(&dst[(int64_t)grp.planeIm * args.planeStride + e], grp.mulIm == 1u ? pos : negv); }
-          }
-        }
-      }
-    }
-  }
+  HYK_GRAM_EPILOGUE(false)
 }
 
 /* ------------------------------------------------------------------ contraction with direct global -> LDS loads
@@ -264,7 +270,7 @@ __device__ __forceinline__ void dma16(uint32_t ldsAddr, const int8_t* src) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(ldsAddr), "v"(src) : "memory");
 }
 
-template <int EPI>
+template <int EPI, bool EXCL>
 __global__ __launch_bounds__(G_THREADS, 1) void gram_dma_kernel(const GramArgs args) {
   using S = Slab<DMA_BK>;
   constexpr int BK = DMA_BK;
@@ -393,32 +399,7 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_dma_kernel(const GramArgs a
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   /* no direct load may still be writing LDS when the workgroup ends */
 
-  const bool diagTile = (ta == tb);
-  #pragma unroll
-  for (int a = 0; a < 4; ++a) {
-    #pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      const int y = y0 + wy * WAVE_TILE + b * 32 + (lane & 31);
-      #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int x = x0 + wx * WAVE_TILE + a * 32 + acc_row(r, lane);
-        if (x < args.N && y < args.N && (!diagTile || y <= x)) {
-          const int64_t e = hyk::tri_index(y, x); const int32_t w = acc[a][b][r];
-          if constexpr (EPI == EPI_MOD) {
-            uint32_t* dst = reinterpret_cast<uint32_t*>(args.acc);
-            const uint32_t v = hyk::reduce_i32(w, grp.m, grp.d, grp.c32);
-            if (grp.mulRe) { atomicAdd(&dst[(int64_t)grp.planeRe * args.planeStride + e], grp.mulRe == 1u ? v : hyk::reduce_u32(v * grp.mulRe, grp.m, grp.d)); }
-            if (grp.mulIm) { atomicAdd(&dst[(int64_t)grp.planeIm * args.planeStride + e], grp.mulIm == 1u ? v : hyk::reduce_u32(v * grp.mulIm, grp.m, grp.d)); }
-          } else {
-            unsigned long long* dst = reinterpret_cast<unsigned long long*>(args.acc);
-            const unsigned long long pos = (unsigned long long)(long long)w, negv = (unsigned long long)(-(long long)w);
-            if (grp.mulRe) { atomicAdd(&dst[(int64_t)grp.planeRe * args.planeStride + e], grp.mulRe == 1u ? pos : negv); }
-            if (grp.mulIm) { atomicAdd(&dst[(int64_t)grp.planeIm * args.planeStride + e], grp.mulIm == 1u ? pos : negv); }
-          }
-        }
-      }
-    }
-  }
+  HYK_GRAM_EPILOGUE(EXCL)
 }
 
 /* ------------------------------------------------------------------ CRT reconstruction */
@@ -491,33 +472,36 @@ template <int BK, int EPI> hipError_t launch_one(hipStream_t stream, const GramA
   return hipGetLastError();
 }
 
-template <int EPI> hipError_t launch_dma(hipStream_t stream, const GramArgs& a) {
+template <int EPI, bool EXCL> hipError_t launch_dma(hipStream_t stream, const GramArgs& a) {
   const int ldsBytes = DMA_STAGES * DMA_STAGE_BYTES;
   static bool attr = false;
-  if (!attr) { hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gram_dma_kernel<EPI>), hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes); if (e != hipSuccess) { return e; } attr = true; }
+  if (!attr) { hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gram_dma_kernel<EPI, EXCL>), hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes); if (e != hipSuccess) { return e; } attr = true; }
   const int blocks = a.itemsPerXcd * XCDS;
   Timed t{ nullptr, nullptr };
   if (g_profile) { if (hipEventCreate(&t.start) != hipSuccess || hipEventCreate(&t.stop) != hipSuccess) { return hipErrorUnknown; } (void)hipEventRecord(t.start, stream); }
-  gram_dma_kernel<EPI><<<blocks, G_THREADS, ldsBytes, stream>>>(a);
+  gram_dma_kernel<EPI, EXCL><<<blocks, G_THREADS, ldsBytes, stream>>>(a);
   if (g_profile) { (void)hipEventRecord(t.stop, stream); g_timed.push_back(t); }
   return hipGetLastError();
 }
 
-hipError_t launch_gram(hipStream_t stream, GramArgs& a, int epi, int maxProducts) {
+hipError_t launch_gram(hipStream_t stream, GramArgs& a, int epi, int maxProducts, bool unshared) {
   /* K split: enough items to fill the chip a few times over, never more than maxProducts int8 products per int32 */
   int maxPairs = 1; for (int g = 0; g < a.groupCount; ++g) { maxPairs = a.groups[g].pairCount > maxPairs ? a.groups[g].pairCount : maxPairs; }
   const int bk = g_bk == 0 ? DMA_BK : g_bk; int kCap = (maxProducts / maxPairs) / bk * bk; if (kCap < bk) { return hipErrorInvalidValue; }
   const int64_t base = (int64_t)a.groupCount * a.tileCount; int splits = 1;
-  const int wanted = 1024;  /* about four waves of 256 workgroups */
+  const int wanted = 512;   /* two rounds of 256 workgroups: every further K split costs another epilogue (65536 atomics) per tile */
   if (base < wanted) { splits = (int)((wanted + base - 1) / base); }
   int kLen = ((a.K + splits - 1) / splits + bk - 1) / bk * bk; if (kLen < 2048) { kLen = 2048; } if (kLen > kCap) { kLen = kCap; }
   if (kLen > a.K) { kLen = a.K; }
-  a.kLen = kLen; a.kSplits = (a.K + kLen - 1) / kLen;
+  a.kLen = kLen; a.kSplits = (a.K + kLen - 1) / kLen; a.exclusive = (unshared && a.kSplits == 1 && g_bk == 0) ? 1 : 0;
   const int64_t total = base * a.kSplits; if (total > 0x7fffffff / 2) { return hipErrorInvalidValue; }
   a.totalItems = (int)total; a.itemsPerXcd = (int)((total + XCDS - 1) / XCDS);
   if (total * a.tileCount >= (1ll << 32) || total * a.kSplits >= (1ll << 32)) { return hipErrorInvalidValue; }
   a.tileMagic = a.tileCount > 1 ? (uint32_t)((1ull << 32) / (uint32_t)a.tileCount) + 1u : 0u; a.splitMagic = a.kSplits > 1 ? (uint32_t)((1ull << 32) / (uint32_t)a.kSplits) + 1u : 0u;
-  if (g_bk == 0) { return epi == EPI_MOD ? launch_dma<EPI_MOD>(stream, a) : launch_dma<EPI_I64>(stream, a); }
+  if (g_bk == 0) {
+    if (a.exclusive) { return epi == EPI_MOD ? launch_dma<EPI_MOD, true>(stream, a) : launch_dma<EPI_I64, true>(stream, a); }
+    return epi == EPI_MOD ? launch_dma<EPI_MOD, false>(stream, a) : launch_dma<EPI_I64, false>(stream, a);
+  }
   if (bk == 128) { return epi == EPI_MOD ? launch_one<128, EPI_MOD>(stream, a) : launch_one<128, EPI_I64>(stream, a); }
   return epi == EPI_MOD ? launch_one<64, EPI_MOD>(stream, a) : launch_one<64, EPI_I64>(stream, a);
 }
@@ -528,9 +512,10 @@ void base_args(GramArgs& a, const int8_t* panels, int64_t ldb, int32_t N, int32_
 }
 
 struct GroupBuilder {
-  GramArgs a; int pairs = 0; int epi; int maxProducts; hipStream_t stream; hipError_t err = hipSuccess;
-  GroupBuilder(hipStream_t s, int epi_, int maxProducts_, const int8_t* panels, int64_t ldb, int32_t N, int32_t K, void* acc) : epi(epi_), maxProducts(maxProducts_), stream(s) { base_args(a, panels, ldb, N, K, acc); }
-  void flush() { if (a.groupCount > 0 && err == hipSuccess) { err = launch_gram(stream, a, epi, maxProducts); } a.groupCount = 0; pairs = 0; }
+  GramArgs a; int pairs = 0; int epi; int maxProducts; bool unshared; hipStream_t stream; hipError_t err = hipSuccess;
+  /* unshared: no two groups write the same accumulator plane (true for the real paths) */
+  GroupBuilder(hipStream_t s, int epi_, int maxProducts_, bool unshared_, const int8_t* panels, int64_t ldb, int32_t N, int32_t K, void* acc) : epi(epi_), maxProducts(maxProducts_), unshared(unshared_), stream(s) { base_args(a, panels, ldb, N, K, acc); }
+  void flush() { if (a.groupCount > 0 && err == hipSuccess) { err = launch_gram(stream, a, epi, maxProducts, unshared); } a.groupCount = 0; pairs = 0; }
   /* begins a group; flushes first when the tables are full */
   GramGroup& begin(int npairs) {
     if (a.groupCount == MAX_GROUPS || pairs + npairs > MAX_PAIRS) { flush(); }
@@ -641,7 +626,7 @@ extern "C" int hykGramCrt(hipStream_t stream, int32_t Complex, int32_t N, int32_
   if (N <= 0) { return 0; }
   if (orderA < 1 || orderA > (Complex ? HYK_CRT_CPLX_COUNT : HYK_CRT_REAL_COUNT) || orderC < 1 || orderC > 3 || K <= 0 || (K & 127) || ldb < K || (ldb & 15) || ((uintptr_t)panels & 15)) { return -1; }
   /* 131072 products per int32: residues of every modulus but 256 are at most 125 in magnitude, and mod 256 a wrap is harmless */
-  GroupBuilder gb(stream, EPI_MOD, 131072, panels, ldb, N, K, workspace);
+  GroupBuilder gb(stream, EPI_MOD, 131072, Complex == 0, panels, ldb, N, K, workspace);
   ReconTable tab; tab.order = orderA;
   if (!Complex) {
     for (int x = 0; x < orderA; ++x) { GramGroup& g = gb.begin(1); set_mod(g, hyk_crt_real_mo[x]); g.mulRe = 1; g.planeRe = (uint16_t)x; gb.pair(g, x, x); }
@@ -677,7 +662,7 @@ extern "C" int hykGramLimbs(hipStream_t stream, int32_t Complex, int32_t N, int3
   if (orderA < 1 || orderA > 12 || orderC < 1 || orderC > 3 || K <= 0 || (K & 127) || ldb < K || (ldb & 15) || ((uintptr_t)panels & 15)) { return -1; }
   const int levels = 2 * orderA - 1;
   /* 131071 products of magnitude <= 2^14 fit an int32 */
-  GroupBuilder gb(stream, EPI_I64, 131071, panels, ldb, N, K, workspace);
+  GroupBuilder gb(stream, EPI_I64, 131071, Complex == 0, panels, ldb, N, K, workspace);
   /* heaviest levels first so the tail of the launch is made of short items */
   for (int cnt = orderA; cnt >= 1; --cnt) for (int s = 0; s < levels; ++s) {
     const int lo = s < orderA ? 0 : s - orderA + 1, hi = s < orderA ? s : orderA - 1; if (hi - lo + 1 != cnt) { continue; }
