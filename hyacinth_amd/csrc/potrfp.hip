@@ -32,7 +32,7 @@ namespace {
 namespace cg = cooperative_groups;
 using hyk::dd_t;
 
-constexpr int P_THREADS = 256;
+constexpr int P_THREADS = 1024;   /* 16 wavefronts per compute unit: the dot products are latency-bound loads of the factor */
 constexpr int P_WAVES = P_THREADS / 64;
 
 struct Partial { double bx, by, trace; int32_t idx, pad; };
@@ -73,15 +73,26 @@ __device__ __forceinline__ void better(bool dd, double& bx, double& by, int32_t&
   if (bi < 0 || gt || (eq && oi < bi)) { bx = ox; by = oy; bi = oi; }
 }
 
+/* workgroup arg-max / sum: shuffles inside each wavefront, one exchange through LDS between them (two barriers) */
+template <bool DD>
+__device__ __forceinline__ void wave_reduce(double& bx, double& by, int32_t& bi, double& tr) {
+  #pragma unroll
+  for (int m = 32; m > 0; m >>= 1) {
+    const double ox = __shfl_xor(bx, m, 64), oy = __shfl_xor(by, m, 64), ot = __shfl_xor(tr, m, 64); const int32_t oi = __shfl_xor(bi, m, 64);
+    better(DD, bx, by, bi, ox, oy, oi); tr += ot;
+  }
+}
 template <bool DD>
 __device__ __forceinline__ void block_reduce(double& bx, double& by, int32_t& bi, double& tr) {
-  __shared__ double sx[P_THREADS], sy[P_THREADS], st[P_THREADS]; __shared__ int32_t si[P_THREADS];
-  const int t = threadIdx.x; sx[t] = bx; sy[t] = by; si[t] = bi; st[t] = tr; __syncthreads();
-  for (int s = P_THREADS / 2; s > 0; s >>= 1) {
-    if (t < s) { double ax = sx[t], ay = sy[t]; int32_t ai = si[t]; better(DD, ax, ay, ai, sx[t + s], sy[t + s], si[t + s]); sx[t] = ax; sy[t] = ay; si[t] = ai; st[t] += st[t + s]; }
-    __syncthreads();
-  }
-  bx = sx[0]; by = sy[0]; bi = si[0]; tr = st[0]; __syncthreads();
+  __shared__ double sx[P_WAVES], sy[P_WAVES], st[P_WAVES]; __shared__ int32_t si[P_WAVES];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  wave_reduce<DD>(bx, by, bi, tr);
+  if (lane == 0) { sx[wave] = bx; sy[wave] = by; si[wave] = bi; st[wave] = tr; }
+  __syncthreads();
+  bx = by = tr = 0.; bi = -1;
+  if (lane < P_WAVES) { bx = sx[lane]; by = sy[lane]; bi = si[lane]; tr = st[lane]; }
+  wave_reduce<DD>(bx, by, bi, tr);     /* every wavefront reduces the same P_WAVES entries: no broadcast needed */
+  __syncthreads();
 }
 
 template <bool DD, bool CPLX>
@@ -122,6 +133,7 @@ __global__ __launch_bounds__(P_THREADS) void potrfp_kernel(const PotrfArgs a) {
       if (l == c || a.done[l]) { continue; }
       const double* rl = &a.Rt[(int64_t)l * a.ldr * WE];
       R sre = R::zero(), sim = R::zero();
+      #pragma unroll 4
       for (int t = lane; t < k; t += 64) {
         if constexpr (CPLX) {
           R ar = R::load(&rl[(int64_t)t * WE]), ai = R::load(&rl[(int64_t)t * WE + WR]), br = R::load(&rcol[(int64_t)t * WE]), bim = R::load(&rcol[(int64_t)t * WE + WR]);

@@ -75,6 +75,122 @@ __global__ __launch_bounds__(T_THREADS) void jacobi_round_kernel(int32_t N, int3
   if (threadIdx.x == 0) { atomicAdd(rotations, 1); }
 }
 
+/* ------------------------------------------------------------------ blocked one-sided Jacobi
+ * A round of the plain kernel above moves every column through memory once per pair it takes part in.  Here a workgroup
+ * takes a pair of column blocks (BC columns each), keeps its rows of all 2 BC columns in registers (thread t owns rows
+ * t, t + 256, ...) and rotates every cross pair (BC steps of BC disjoint pairs) before writing them back: BC times fewer
+ * passes over B per sweep.  In the first round of a sweep the 2 BC columns go through a full round-robin instead, which
+ * also covers the pairs inside each block.  Column norms are summed once per round and carried through the rotations
+ * (alpha' = alpha - t gamma, beta' = beta + t gamma); only the BC cross products of a step need a workgroup reduction. */
+template <int NV>
+__device__ __forceinline__ void block_sum_many(double (&v)[NV], double* red, int parity) {
+  #pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    #pragma unroll
+    for (int off = 32; off > 0; off >>= 1) { v[i] += __shfl_xor(v[i], off, 64); }
+  }
+  double* mine = red + parity * (T_THREADS / 64) * NV;
+  if ((threadIdx.x & 63) == 0) {
+    #pragma unroll
+    for (int i = 0; i < NV; ++i) { mine[(threadIdx.x >> 6) * NV + i] = v[i]; }
+  }
+  __syncthreads();
+  #pragma unroll
+  for (int i = 0; i < NV; ++i) { double s = 0.; for (int w = 0; w < T_THREADS / 64; ++w) { s += mine[w * NV + i]; } v[i] = s; }
+}
+
+template <bool CPLX, int ROWS, int BC, bool FULL>
+__global__ __launch_bounds__(T_THREADS) void jacobi_block_round_kernel(int32_t N, int32_t nb, int32_t r, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations) {
+  constexpr int W = CPLX ? 2 : 1, NC = 2 * BC, GV = BC * W;
+  __shared__ double red[2 * (T_THREADS / 64) * (NC > GV ? NC : GV)];
+  const int i = blockIdx.x; int P, Q;
+  if (i == 0) { P = nb - 1; Q = round; } else { P = (round + i) % (nb - 1); Q = (round - i + (nb - 1)) % (nb - 1); }
+  if (P > Q) { const int t = P; P = Q; Q = t; }
+  int col[NC]; bool live[NC];
+  #pragma unroll
+  for (int c = 0; c < NC; ++c) { col[c] = (c < BC ? P : Q) * BC + (c % BC); live[c] = col[c] < r; }
+  if (!live[0]) { return; }                       /* both blocks beyond the last column */
+  /* rows of this thread */
+  double x[NC][ROWS][W];
+  #pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    #pragma unroll
+    for (int m = 0; m < ROWS; ++m) {
+      const int k = threadIdx.x + m * T_THREADS;
+      #pragma unroll
+      for (int w = 0; w < W; ++w) { x[c][m][w] = (live[c] && k < N) ? B[((int64_t)col[c] * N + k) * W + w] : 0.; }
+    }
+  }
+  double norm[NC];
+  #pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    double s = 0.;
+    #pragma unroll
+    for (int m = 0; m < ROWS; ++m) {
+      #pragma unroll
+      for (int w = 0; w < W; ++w) { s += x[c][m][w] * x[c][m][w]; }
+    }
+    norm[c] = s;
+  }
+  block_sum_many<NC>(norm, red, 0);
+  int applied = 0;
+  /* FULL: first round of a sweep, all pairs of the 2 BC columns (round-robin); otherwise the BC x BC cross pairs */
+  constexpr int STEPS = FULL ? NC - 1 : BC;
+  #pragma unroll
+  for (int step = 0; step < STEPS; ++step) {
+    double g[GV];
+    #pragma unroll
+    for (int j = 0; j < BC; ++j) {
+      const int fa = (j == 0) ? NC - 1 : (step + j) % (NC - 1), fb = (j == 0) ? step : (step - j + (NC - 1)) % (NC - 1);
+      const int c0 = FULL ? (fa < fb ? fa : fb) : j, c1 = FULL ? (fa < fb ? fb : fa) : BC + (j + step) % BC;
+      double gr = 0., gi = 0.;
+      #pragma unroll
+      for (int m = 0; m < ROWS; ++m) {
+        if constexpr (CPLX) { gr += x[c0][m][0] * x[c1][m][0] + x[c0][m][1] * x[c1][m][1]; gi += x[c0][m][0] * x[c1][m][1] - x[c0][m][1] * x[c1][m][0]; }
+        else { gr += x[c0][m][0] * x[c1][m][0]; }
+      }
+      g[j * W] = gr; if constexpr (CPLX) { g[j * W + 1] = gi; }
+    }
+    block_sum_many<GV>(g, red, (step + 1) & 1);
+    #pragma unroll
+    for (int j = 0; j < BC; ++j) {
+      const int fa = (j == 0) ? NC - 1 : (step + j) % (NC - 1), fb = (j == 0) ? step : (step - j + (NC - 1)) % (NC - 1);
+      const int c0 = FULL ? (fa < fb ? fa : fb) : j, c1 = FULL ? (fa < fb ? fb : fa) : BC + (j + step) % BC;
+      const double gre = g[j * W], gim = CPLX ? g[j * W + (CPLX ? 1 : 0)] : 0.;
+      const double alpha = norm[c0], beta = norm[c1], g2 = gre * gre + gim * gim;
+      if (live[c0] && live[c1] && g2 > tol * tol * alpha * beta && g2 > 0.) {
+        const double gabs = sqrt(g2), zeta = (beta - alpha) / (2. * gabs);
+        const double t = (zeta >= 0. ? 1. : -1.) / (fabs(zeta) + sqrt(1. + zeta * zeta)), cs = 1. / sqrt(1. + t * t), sn = cs * t;
+        const double er = gre / gabs, ei = gim / gabs;
+        #pragma unroll
+        for (int m = 0; m < ROWS; ++m) {
+          if constexpr (CPLX) {
+            const double pr = x[c0][m][0], pi = x[c0][m][1], q0 = x[c1][m][0], q1 = x[c1][m][1];
+            const double qr = q0 * er + q1 * ei, qi = q1 * er - q0 * ei;
+            x[c0][m][0] = cs * pr - sn * qr; x[c0][m][1] = cs * pi - sn * qi; x[c1][m][0] = sn * pr + cs * qr; x[c1][m][1] = sn * pi + cs * qi;
+          } else {
+            const double pv = x[c0][m][0], qv = x[c1][m][0] * er;
+            x[c0][m][0] = cs * pv - sn * qv; x[c1][m][0] = sn * pv + cs * qv;
+          }
+        }
+        norm[c0] = alpha - t * gabs; norm[c1] = beta + t * gabs; ++applied;
+      }
+    }
+  }
+  #pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    #pragma unroll
+    for (int m = 0; m < ROWS; ++m) {
+      const int k = threadIdx.x + m * T_THREADS;
+      if (live[c] && k < N) {
+        #pragma unroll
+        for (int w = 0; w < W; ++w) { B[((int64_t)col[c] * N + k) * W + w] = x[c][m][w]; }
+      }
+    }
+  }
+  if (threadIdx.x == 0 && applied) { atomicAdd(rotations, applied); }
+}
+
 template <bool CPLX>
 __global__ __launch_bounds__(T_THREADS) void column_norm_kernel(int32_t N, const double* __restrict__ B, double* __restrict__ sigma) {
   __shared__ double scratch[T_THREADS / 64]; constexpr int W = CPLX ? 2 : 1;
@@ -148,9 +264,28 @@ extern "C" int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t
   return 0;
 }
 
-/* one sweep = n-1 rounds over the r columns of B (N x r, FP64, complex interleaved); rotations counts the rotations applied */
+/* one sweep = every pair of the r columns of B (N x r, FP64, complex interleaved) once; rotations counts the rotations applied */
+template <bool CPLX, int ROWS, int BC>
+static int blocked_sweep(hipStream_t stream, int32_t N, int32_t r, double* B, double tol, int32_t* rotations) {
+  const int blocks = (r + BC - 1) / BC, nb = (blocks + 1) & ~1;
+  jacobi_block_round_kernel<CPLX, ROWS, BC, true><<<nb / 2, T_THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations);
+  for (int round = 1; round < nb - 1; ++round) { jacobi_block_round_kernel<CPLX, ROWS, BC, false><<<nb / 2, T_THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations); }
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
 extern "C" int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations) {
   if (N <= 0 || r <= 1) { return 0; }
+  /* blocked kernel when the rows of two column blocks fit the registers of a workgroup */
+  if (!Complex && r >= 16) {
+    if (N <= 4 * T_THREADS) { return blocked_sweep<false, 4, 4>(stream, N, r, B, tol, rotations); }
+    if (N <= 8 * T_THREADS) { return blocked_sweep<false, 8, 4>(stream, N, r, B, tol, rotations); }
+    if (N <= 16 * T_THREADS) { return blocked_sweep<false, 16, 4>(stream, N, r, B, tol, rotations); }
+  }
+  if (Complex && r >= 16) {
+    if (N <= 4 * T_THREADS) { return blocked_sweep<true, 4, 4>(stream, N, r, B, tol, rotations); }
+    if (N <= 8 * T_THREADS) { return blocked_sweep<true, 8, 4>(stream, N, r, B, tol, rotations); }
+    if (N <= 16 * T_THREADS) { return blocked_sweep<true, 16, 2>(stream, N, r, B, tol, rotations); }
+  }
   const int n = (r + 1) & ~1;
   for (int round = 0; round < n - 1; ++round) {
     if (Complex) { jacobi_round_kernel<true><<<n / 2, T_THREADS, 0, stream>>>(N, n, r, round, B, tol, rotations); } else { jacobi_round_kernel<false><<<n / 2, T_THREADS, 0, stream>>>(N, n, r, round, B, tol, rotations); }
