@@ -22,14 +22,12 @@
  * Cooperative launch: at most one workgroup per compute unit, all resident.
  */
 #include <hip/hip_runtime.h>
-#include <hip/hip_cooperative_groups.h>
 #include "hyk_common.h"
 #include "hyk_dd.h"
 #include "hyacin_kernels.h"
 
 namespace {
 
-namespace cg = cooperative_groups;
 using hyk::dd_t;
 
 constexpr int P_THREADS = 1024;   /* 16 wavefronts per compute unit: the dot products are latency-bound loads of the factor */
@@ -40,7 +38,7 @@ struct Partial { double bx, by, trace; int32_t idx, pad; };
 struct PotrfArgs {
   int32_t N, K, ldr; double eps2;
   const double* G; int64_t ldg;
-  double* Rt; double* D; int32_t* done; int32_t* jpiv; int32_t* pos; Partial* partials; int32_t* rankOut;
+  double* Rt; double* D; int32_t* done; int32_t* jpiv; int32_t* pos; Partial* partials; int32_t* rankOut; uint32_t* arrivals;
 };
 
 /* scalar types: value = re (+ i im), each part a dd_t (lo part unused in FP64 mode) */
@@ -95,9 +93,24 @@ __device__ __forceinline__ void block_reduce(double& bx, double& by, int32_t& bi
   __syncthreads();
 }
 
+/* Grid barrier for the co-resident workgroups of the cooperative launch: one arrival counter that only grows, so no
+ * reset phase; barrier number `epoch` (1, 2, ...) is passed once the counter has reached epoch * workgroups.  The fences
+ * publish this workgroup's global writes before the arrival and drop stale cache lines after the release. */
+__device__ __forceinline__ void grid_barrier(uint32_t* arrivals, uint32_t workgroups, uint32_t epoch) {
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    __threadfence();
+    atomicAdd(arrivals, 1u);
+    const uint32_t target = epoch * workgroups;
+    while (__hip_atomic_load(arrivals, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < target) { __builtin_amdgcn_s_sleep(1); }
+    __threadfence();
+  }
+  __syncthreads();
+}
+
 template <bool DD, bool CPLX>
 __global__ __launch_bounds__(P_THREADS) void potrfp_kernel(const PotrfArgs a) {
-  cg::grid_group grid = cg::this_grid();
+  uint32_t epoch = 0;
   using R = Real<DD>; constexpr int WR = Width<DD, CPLX>::real, WE = Width<DD, CPLX>::elem;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwg = gridDim.x, wg = blockIdx.x;
   const int gthread = wg * P_THREADS + tid, nthreads = nwg * P_THREADS, gwave = wg * P_WAVES + wave, nwaves = nwg * P_WAVES;
@@ -112,7 +125,7 @@ __global__ __launch_bounds__(P_THREADS) void potrfp_kernel(const PotrfArgs a) {
   }
   block_reduce<DD>(bx, by, bi, tr);
   if (tid == 0) { a.partials[wg] = Partial{ bx, by, tr, bi, 0 }; }
-  grid.sync();
+  grid_barrier(a.arrivals, (uint32_t)nwg, ++epoch);
   bx = by = tr = 0.; bi = -1;
   if (tid < nwg) { Partial p = a.partials[tid]; bx = p.bx; by = p.by; bi = p.idx; tr = p.trace; }
   block_reduce<DD>(bx, by, bi, tr);
@@ -132,8 +145,11 @@ __global__ __launch_bounds__(P_THREADS) void potrfp_kernel(const PotrfArgs a) {
     for (int l = gwave; l < N; l += nwaves) {
       if (l == c || a.done[l]) { continue; }
       const double* rl = &a.Rt[(int64_t)l * a.ldr * WE];
+      /* G[l, c] and d_l are needed only after the dot product: request them first so their latency hides under it */
+      const double* g = &a.G[((int64_t)l + (int64_t)c * a.ldg) * WE];
+      const R gre0 = R::load(g), d0 = R::load(&a.D[(int64_t)l * WR]); R gim0 = R::zero(); if constexpr (CPLX) { gim0 = R::load(g + WR); }
       R sre = R::zero(), sim = R::zero();
-      #pragma unroll 4
+      #pragma unroll 8
       for (int t = lane; t < k; t += 64) {
         if constexpr (CPLX) {
           R ar = R::load(&rl[(int64_t)t * WE]), ai = R::load(&rl[(int64_t)t * WE + WR]), br = R::load(&rcol[(int64_t)t * WE]), bim = R::load(&rcol[(int64_t)t * WE + WR]);
@@ -143,10 +159,9 @@ __global__ __launch_bounds__(P_THREADS) void potrfp_kernel(const PotrfArgs a) {
       }
       for (int m = 32; m > 0; m >>= 1) { sre = sre + sre.shfl_xor(m); if constexpr (CPLX) { sim = sim + sim.shfl_xor(m); } }
       if (lane == 0) {
-        const double* g = &a.G[((int64_t)l + (int64_t)c * a.ldg) * WE];
-        sre = sre + R::load(g); R rr = rho * sre; double* out = &a.Rt[((int64_t)l * a.ldr + k) * WE]; rr.store(out);
-        R d = R::load(&a.D[(int64_t)l * WR]);
-        if constexpr (CPLX) { sim = sim + R::load(g + WR); R ri = (rho * sim).neg(); ri.store(out + WR); d = d - (rr * rr + ri * ri); } else { d = d - rr * rr; }
+        sre = sre + gre0; R rr = rho * sre; double* out = &a.Rt[((int64_t)l * a.ldr + k) * WE]; rr.store(out);
+        R d = d0;
+        if constexpr (CPLX) { sim = sim + gim0; R ri = (rho * sim).neg(); ri.store(out + WR); d = d - (rr * rr + ri * ri); } else { d = d - rr * rr; }
         d.store(&a.D[(int64_t)l * WR]); tr += d.v.x;
         if (d.v.x > 0.) { better(DD, bx, by, bi, d.v.x, d.v.y, l); }
       }
@@ -155,7 +170,7 @@ __global__ __launch_bounds__(P_THREADS) void potrfp_kernel(const PotrfArgs a) {
     ++k;
     Partial* part = &a.partials[(k & 1) * nwg];
     if (tid == 0) { part[wg] = Partial{ bx, by, tr, bi, 0 }; }
-    grid.sync();
+    grid_barrier(a.arrivals, (uint32_t)nwg, ++epoch);
     bx = by = tr = 0.; bi = -1;
     if (tid < nwg) { Partial p = part[tid]; bx = p.bx; by = p.by; bi = p.idx; tr = p.trace; }
     block_reduce<DD>(bx, by, bi, tr);
@@ -173,6 +188,8 @@ __global__ __launch_bounds__(P_THREADS) void potrfp_kernel(const PotrfArgs a) {
   if (wg == 0 && tid == 0) { *a.rankOut = rank; }
 }
 
+__global__ void clear_word_kernel(uint32_t* p) { *p = 0u; }
+
 /* one-time per kernel: how many workgroups may be co-resident */
 template <bool DD, bool CPLX> int launch(hipStream_t stream, PotrfArgs& args, int cus) {
   int perCu = 0; if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, potrfp_kernel<DD, CPLX>, P_THREADS, 0) != hipSuccess || perCu < 1) { return -3; }
@@ -188,7 +205,7 @@ extern "C" size_t hykPotrfpWorkspaceBytes(int32_t N, int32_t Gtype) {
   if (N <= 0) { return 0; }
   const size_t wr = ((Gtype & ~1) == HYK_DD) ? 2 : 1;
   /* D | done | pos | partials(2 x 256) */
-  return (size_t)N * wr * 8 + (size_t)N * 4 * 2 + 2 * 256 * sizeof(Partial) + 256;
+  return (size_t)N * wr * 8 + (size_t)N * 4 * 2 + 2 * 256 * sizeof(Partial) + 256 + 256;
 }
 
 extern "C" int hykPotrfp(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, int32_t N, int32_t Gtype, const void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, void* workspace, int32_t* rankOut) {
@@ -199,7 +216,9 @@ extern "C" int hykPotrfp(hipStream_t stream, int32_t computeUnits, double eps, i
   if (!dd && (Gtype & ~1) != HYK_F64) { return -1; }
   PotrfArgs a; a.N = N; a.K = K; a.ldr = ldr; a.eps2 = eps * eps; a.G = (const double*)G; a.ldg = ldg; a.Rt = (double*)Rt; a.jpiv = jpiv; a.rankOut = rankOut;
   char* w = (char*)workspace; a.D = (double*)w; w += (size_t)N * (dd ? 2 : 1) * 8; a.done = (int32_t*)w; w += (size_t)N * 4; a.pos = (int32_t*)w; w += (size_t)N * 4;
-  w = (char*)(((uintptr_t)w + 15) & ~(uintptr_t)15); a.partials = (Partial*)w;
+  w = (char*)(((uintptr_t)w + 15) & ~(uintptr_t)15); a.partials = (Partial*)w; w += 2 * 256 * sizeof(Partial);
+  w = (char*)(((uintptr_t)w + 63) & ~(uintptr_t)63); a.arrivals = (uint32_t*)w;
+  clear_word_kernel<<<1, 1, 0, stream>>>(a.arrivals);
   if (dd) { return cplx ? launch<true, true>(stream, a, computeUnits) : launch<true, false>(stream, a, computeUnits); }
   return cplx ? launch<false, true>(stream, a, computeUnits) : launch<false, false>(stream, a, computeUnits);
 }
