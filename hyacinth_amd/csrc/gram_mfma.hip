@@ -484,14 +484,27 @@ template <int EPI, bool EXCL> hipError_t launch_dma(hipStream_t stream, const Gr
   return hipGetLastError();
 }
 
+int compute_units() {
+  static int units = 0;
+  if (units == 0) { int dev = 0, n = 0; if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) { units = n; } else { units = 256; } }
+  return units;
+}
+
 hipError_t launch_gram(hipStream_t stream, GramArgs& a, int epi, int maxProducts, bool unshared) {
-  /* K split: enough items to fill the chip a few times over, never more than maxProducts int8 products per int32 */
   int maxPairs = 1; for (int g = 0; g < a.groupCount; ++g) { maxPairs = a.groups[g].pairCount > maxPairs ? a.groups[g].pairCount : maxPairs; }
   const int bk = g_bk == 0 ? DMA_BK : g_bk; int kCap = (maxProducts / maxPairs) / bk * bk; if (kCap < bk) { return hipErrorInvalidValue; }
-  const int64_t base = (int64_t)a.groupCount * a.tileCount; int splits = 1;
-  const int wanted = 512;   /* two rounds of 256 workgroups: every further K split costs another epilogue (65536 atomics) per tile */
-  if (base < wanted) { splits = (int)((wanted + base - 1) / base); }
-  int kLen = ((a.K + splits - 1) / splits + bk - 1) / bk * bk; if (kLen < 2048) { kLen = 2048; } if (kLen > kCap) { kLen = kCap; }
+  /* K split.  One workgroup runs per compute unit, so a launch takes rounds = ceil(items / units) item times; an item costs
+   * its slabs plus a fixed prologue / epilogue (65536 reductions and atomics) worth about 48 slab times.  Take the split
+   * count that minimises rounds x (slabs + 48); the cap keeps the int32 sums exact. */
+  const int64_t base = (int64_t)a.groupCount * a.tileCount; const int units = compute_units();
+  const int minSplits = (a.K + kCap - 1) / kCap; int splits = minSplits; double best = -1.;
+  for (int cand = minSplits; cand <= minSplits + 15; ++cand) {
+    const int len = ((a.K + cand - 1) / cand + bk - 1) / bk * bk; if (len < 16 * bk && cand > minSplits) { break; }
+    const int count = (a.K + len - 1) / len; const int64_t rounds = (base * count + units - 1) / units;
+    const double cost = (double)rounds * ((double)(len / bk) + 48.);
+    if (best < 0. || cost < best * 0.98) { best = cost; splits = cand; }   /* a further split has to win by 2 % */
+  }
+  int kLen = ((a.K + splits - 1) / splits + bk - 1) / bk * bk; if (kLen > kCap) { kLen = kCap; }
   if (kLen > a.K) { kLen = a.K; }
   a.kLen = kLen; a.kSplits = (a.K + kLen - 1) / kLen; a.exclusive = (unshared && a.kSplits == 1 && g_bk == 0) ? 1 : 0;
   const int64_t total = base * a.kSplits; if (total > 0x7fffffff / 2) { return hipErrorInvalidValue; }

@@ -181,17 +181,31 @@ template <int X> struct CplxF64 {
   static constexpr hyk::F64Mod sym = hyk::make_f64mod(hyk_crt_cplx_mo[X], 0.0);   /* any small representative */
   static constexpr double im = (double)hyk_crt_cplx_im[X];
 };
-__device__ __forceinline__ uint32_t byte_of(double r) { return (uint32_t)(int32_t)r & 0xffu; }
+/* Integer -> byte without a conversion instruction: adding 1.5 * 2^52 to an integer-valued double |r| < 2^51 leaves r, in
+ * two's complement, in the low bits of the sum's mantissa.  For the real path the constant is folded into the residue's
+ * second multiply-add (a + 1.5 * 2^52 is still exact for |a| < 2^51), so a residue byte costs three FP64 instructions. */
+constexpr double LOW_BITS = 6755399441055744.0;   /* 1.5 * 2^52 */
+__device__ __forceinline__ uint32_t low_word(double r) { return (uint32_t)__double2loint(r + LOW_BITS); }
+__device__ __forceinline__ uint32_t low_word_of_biased(double rPlusBias) { return (uint32_t)__double2loint(rPlusBias); }
+__device__ __forceinline__ double residue_f64_biased(double a, double aBiased, const hyk::F64Mod& k) {
+  return __builtin_fma(k.negM, __builtin_rint(__builtin_fma(a, k.inv, k.tieShift)), aBiased);
+}
+/* low bytes of four words -> one dword (row 0 in the lowest byte) */
+__device__ __forceinline__ uint32_t pack4(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t w3) {
+  const uint32_t lo = __builtin_amdgcn_perm(w1, w0, 0x0c0c0400u), hi = __builtin_amdgcn_perm(w3, w2, 0x0c0c0400u);
+  return __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+}
+static_assert(Q_ROWS == 4, "pack4 packs the four rows of a thread");
 
 template <int X>
-__device__ __forceinline__ void crt_real_f64_step(int32_t order, const double (&a)[Q_ROWS], int8_t* out, int64_t strideB, int valid, bool aligned) {
+__device__ __forceinline__ void crt_real_f64_step(int32_t order, const double (&a)[Q_ROWS], const double (&ab)[Q_ROWS], int8_t* out, int64_t strideB, int valid, bool aligned) {
   if constexpr (X < HYK_CRT_REAL_COUNT) {
     if (X < order) {
-      constexpr hyk::F64Mod k = RealF64<X>::k; uint32_t packed = 0;
+      constexpr hyk::F64Mod k = RealF64<X>::k; uint32_t w[Q_ROWS];
       #pragma unroll
-      for (int r = 0; r < Q_ROWS; ++r) { packed |= byte_of(hyk::residue_f64(a[r], k)) << (8 * r); }
-      store_panel(out + (int64_t)X * strideB, packed, valid, aligned);
-      crt_real_f64_step<X + 1>(order, a, out, strideB, valid, aligned);
+      for (int r = 0; r < Q_ROWS; ++r) { w[r] = low_word_of_biased(residue_f64_biased(a[r], ab[r], k)); }
+      store_panel(out + (int64_t)X * strideB, pack4(w[0], w[1], w[2], w[3]), valid, aligned);
+      crt_real_f64_step<X + 1>(order, a, ab, out, strideB, valid, aligned);
     }
   }
 }
@@ -203,27 +217,28 @@ __global__ __launch_bounds__(Q_THREADS) void quantize_crt_real_f64_kernel(int32_
   const int valid = (M - i0) < Q_ROWS ? (int)(M - i0) : Q_ROWS; const int32_t expon = vexp[j];
   int8_t* out = B + (int64_t)j * ldb + i0; const bool aligned = ((uintptr_t)out & 3u) == 0;
   if (expon == HYK_INT_MAX) { for (int p = 0; p < order; ++p) { store_panel(out + p * strideB, 0u, valid, aligned); } return; }
-  double a[Q_ROWS]; typename E::T raw[Q_ROWS]; fetch_rows(&A[(int64_t)j * lda + i0], valid, raw);
+  double a[Q_ROWS], ab[Q_ROWS]; typename E::T raw[Q_ROWS]; fetch_rows(&A[(int64_t)j * lda + i0], valid, raw);
   #pragma unroll
-  for (int r = 0; r < Q_ROWS; ++r) { double re = 0., im = 0.; E::load_f64(&raw[r], re, im); a[r] = __builtin_rint(__builtin_ldexp(re, expon)); }
-  crt_real_f64_step<0>(order, a, out, strideB, valid, aligned);
+  for (int r = 0; r < Q_ROWS; ++r) { double re = 0., im = 0.; E::load_f64(&raw[r], re, im); a[r] = __builtin_rint(__builtin_ldexp(re, expon)); ab[r] = a[r] + LOW_BITS; }
+  crt_real_f64_step<0>(order, a, ab, out, strideB, valid, aligned);
 }
 
 template <int X>
 __device__ __forceinline__ void crt_cplx_f64_step(int32_t order, const double (&ar)[Q_ROWS], const double (&ai)[Q_ROWS], int8_t* out, int64_t strideB, int valid, bool aligned) {
   if constexpr (X < HYK_CRT_CPLX_COUNT) {
     if (X < order) {
-      using K = CplxF64<X>; uint32_t p0 = 0, p1 = 0, p2 = 0;
+      using K = CplxF64<X>; uint32_t w0[Q_ROWS], w1[Q_ROWS], w2[Q_ROWS];
       #pragma unroll
       for (int r = 0; r < Q_ROWS; ++r) {
         if constexpr (X < HYK_CRT_CPLX_SPLIT) {
           const double ra = hyk::residue_f64(ar[r], K::sym), rb = hyk::residue_f64(ai[r], K::sym);   /* |ra|, |rb| <= m / 2 */
-          p0 |= byte_of(hyk::residue_f64(__builtin_fma(-K::im, rb, ra), K::stored)) << (8 * r);
-          p1 |= byte_of(hyk::residue_f64(__builtin_fma(K::im, rb, ra), K::stored)) << (8 * r);
+          w0[r] = low_word(hyk::residue_f64(__builtin_fma(-K::im, rb, ra), K::stored));
+          w1[r] = low_word(hyk::residue_f64(__builtin_fma(K::im, rb, ra), K::stored)); w2[r] = 0u;
         } else {
-          p0 |= byte_of(hyk::residue_f64(ar[r] + ai[r], K::stored)) << (8 * r); p1 |= byte_of(hyk::residue_f64(ar[r], K::stored)) << (8 * r); p2 |= byte_of(hyk::residue_f64(ai[r], K::stored)) << (8 * r);
+          w0[r] = low_word(hyk::residue_f64(ar[r] + ai[r], K::stored)); w1[r] = low_word(hyk::residue_f64(ar[r], K::stored)); w2[r] = low_word(hyk::residue_f64(ai[r], K::stored));
         }
       }
+      const uint32_t p0 = pack4(w0[0], w0[1], w0[2], w0[3]), p1 = pack4(w1[0], w1[1], w1[2], w1[3]), p2 = pack4(w2[0], w2[1], w2[2], w2[3]); (void)p2;
       if constexpr (X < HYK_CRT_CPLX_SPLIT) {
         store_panel(out + (int64_t)(2 * X) * strideB, p0, valid, aligned); store_panel(out + (int64_t)(2 * X + 1) * strideB, p1, valid, aligned);
       } else {
