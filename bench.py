@@ -98,7 +98,7 @@ def main():
     ap.add_argument("--cpu-rows", type=int, default=65536, help="rows of the workload the CPU baseline is timed on (about 15 s of host work)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="before the timed region, run three plain 1 GiB -> 1 GiB device copies (copy_kernel): the known-size reference for HBM traffic counters")
-    ap.add_argument("--slab", type=int, default=-1, help="contraction kernel variant: 0 direct-to-LDS (default), 64 / 128 register-staged with that K slab")
+    ap.add_argument("--slab", type=int, default=-1, help="contraction kernel variant: 0 direct-to-LDS ring, 128-byte rows (default); 2 direct-to-LDS, 64-byte rows; 64 / 128 register-staged")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU: the Gram path of this build has no multi-GPU leg (run with --gpus 1)", file=sys.stderr)
@@ -188,7 +188,7 @@ def main():
         "tsvd_fit_ms": fit_ms,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s", "frac": achieved / INT8_PEAK_TOPS,
                      "traffic": MEASURED_TRAFFIC.get((a.workload, max(a.slab, 0))),
-                     "kernel": "gram_dma_kernel" if a.slab <= 0 else "gram_kernel<%d>" % a.slab, "ops": "int8 multiply-adds x2, upper triangle only", "launches_per_step": launches_per_step,
+                     "kernel": "gram_ring_kernel" if a.slab <= 0 else ("gram_dma_kernel" if a.slab == 2 else "gram_kernel<%d>" % a.slab), "ops": "int8 multiply-adds x2, upper triangle only", "launches_per_step": launches_per_step,
                      "avg_launch_ms": kms.value / max(1, kn.value), "algorithmic_ops_per_step": ops,
                      "sustained_mfma_ceiling": ceiling},
     }

@@ -28,8 +28,13 @@
  *
  * Mapping to the chip.  One 256-thread workgroup (4 wavefronts, 2x2, each
  * 128x128 = 4x4 v_mfma_i32_32x32x32_i8 tiles, 256 accumulator registers per
- * lane) per item; operand tiles staged through LDS in double-buffered K slabs
- * with a padded row pitch that makes the 16-byte fragment reads conflict-free.
+ * lane) per item and per compute unit.  Three generations of the main loop
+ * live here, selectable for measurement (hykGramSetSlab): operand slabs staged
+ * global -> registers -> LDS (gram_kernel), direct global -> LDS loads into a
+ * ring of four 64-K-byte stages (gram_dma_kernel), and the default, direct
+ * loads of whole 128-byte lines into a ring of ten half-tile units that fills
+ * the 160 KB of LDS (gram_ring_kernel).  In all of them the 16-byte LDS slots
+ * are XOR-swizzled per row so that fragment reads are bank-conflict free.
  * Workgroups are dispatched round-robin over the 8 XCDs, so item =
  * (blockIdx % 8) * itemsPerXcd + blockIdx / 8 keeps the items that run
  * together on one XCD (one L2) on the same panels and K range.
@@ -402,6 +407,193 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_dma_kernel(const GramArgs a
   HYK_GRAM_EPILOGUE(EXCL)
 }
 
+/* ------------------------------------------------------------------ contraction with full-line direct loads
+ * Same work items and epilogue again; what changes is the shape of the global -> LDS traffic.  A direct load that fetches
+ * 64 K-bytes of a row touches half a 128-byte cache line, and the L2 / address path is bound by requests, not bytes:
+ * with every load instruction covering 8 rows x 128 bytes (whole lines) the same bytes cost about half as much.  K
+ * therefore advances in slabs of 128 bytes, and all of LDS (160 KB) is a ring of ten 16 KB units, a unit being half an
+ * operand tile (128 rows x 128 K-bytes, 16-byte slots XOR-swizzled per row on the global side).  A slab is four
+ * consecutive units: lane rows 0-127, lane rows 128-255, A rows 0-127, A rows 128-255.
+ *
+ * Schedule of slab j (four MFMA K steps, fragments one step ahead in two register sets):
+ *   step 0, 1   fill the two lane units of slab j + 2 (freed by slab j - 1), one load per four MFMAs;
+ *   step 2      no loads; at its end slab j + 1 has landed (at most the 8 loads just issued are outstanding) and every
+ *               wave has read the last fragments of slab j: barrier;
+ *   step 3      first fragments of slab j + 1, and the two A units of slab j + 2 go into units slab j just released.
+ * The loads that gate a barrier are always at least three K steps (1536 MFMA cycles) old. */
+constexpr int RING_K = 128, RING_UNIT_BYTES = 128 * RING_K, RING_UNITS = 10, RING_BYTES = RING_UNITS * RING_UNIT_BYTES;
+
+template <int EPI, bool EXCL>
+__global__ __launch_bounds__(G_THREADS, 1) void gram_ring_kernel(const GramArgs args) {
+  using S = Slab<RING_K>;
+  extern __shared__ __align__(16) int8_t lds[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), wy = wave & 1, wx = wave >> 1;
+
+  const int item = (int)(blockIdx.x % XCDS) * args.itemsPerXcd + (int)(blockIdx.x / XCDS);
+  if ((int)(blockIdx.x / XCDS) >= args.itemsPerXcd || item >= args.totalItems) { return; }
+  const int gk = args.tileMagic ? (int)(((uint64_t)(uint32_t)item * args.tileMagic) >> 32) : item, t = item - gk * args.tileCount;
+  const int g = args.splitMagic ? (int)(((uint64_t)(uint32_t)gk * args.splitMagic) >> 32) : gk, ks = gk - g * args.kSplits;
+  int tb = 0; while ((tb + 1) * (tb + 2) / 2 <= t) { ++tb; }
+  const int ta = t - tb * (tb + 1) / 2;
+  const GramGroup grp = args.groups[g];
+  const int k0 = ks * args.kLen, kEnd = (k0 + args.kLen) < args.K ? (k0 + args.kLen) : args.K, slabs = (kEnd - k0) / RING_K;
+  const int y0 = ta * TILE, x0 = tb * TILE;
+
+  /* load r (0..3) of a unit: lane tid fills slot tid % 8 of row tid / 8 + 32 r (tile row + 128 for the second half) */
+  int64_t srcLane[2][4], srcA[2][4];
+  {
+    const int rowBase = tid >> 3, kq = (tid & 7) ^ S::swz(rowBase);   /* the swizzle depends on the row modulo 32 only */
+    #pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      #pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int row = h * 128 + rowBase + 32 * r;
+        int cy = y0 + row; cy = cy < args.N ? cy : args.N - 1; int cx = x0 + row; cx = cx < args.N ? cx : args.N - 1;
+        srcLane[h][r] = (int64_t)cy * args.ldb + kq * 16; srcA[h][r] = (int64_t)cx * args.ldb + kq * 16;
+      }
+    }
+  }
+  const uint32_t ldsBase = (uint32_t)(size_t)(__attribute__((address_space(3))) int8_t*)lds;
+  const uint32_t dmaBase = __builtin_amdgcn_readfirstlane(ldsBase + (uint32_t)wave * 1024u);
+
+  v16i acc[4][4];
+  #pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    #pragma unroll
+    for (int b = 0; b < 4; ++b) {
+      #pragma unroll
+      for (int r = 0; r < 16; ++r) { acc[a][b][r] = 0; }
+    }
+  }
+
+  /* Two request streams run through the same sequence of (pair, slab) positions: the lane units and, half a slab behind,
+   * the A units.  Each keeps the position it requested last; all of it is wave-uniform scalar state. */
+  const int iters = slabs * grp.pairCount;
+  const uint32_t pp0 = args.pairs[grp.pairBegin];
+  int pairL = 0, slabL = 0, issuedL = 1, pairA = 0, slabA = 0, issuedA = 1; uint32_t nextL = pp0, nextA = pp0;
+  const int8_t* baseLane = args.panels + (int64_t)(pp0 & 0xffffu) * args.panelStride + k0;
+  const int8_t* baseA = args.panels + (int64_t)(pp0 >> 16) * args.panelStride + k0;
+  auto peekL = [&]() { const int q = pairL + 1 < (int)grp.pairCount ? pairL + 1 : (int)grp.pairCount - 1; nextL = args.pairs[grp.pairBegin + q]; };
+  auto peekA = [&]() { const int q = pairA + 1 < (int)grp.pairCount ? pairA + 1 : (int)grp.pairCount - 1; nextA = args.pairs[grp.pairBegin + q]; };
+  auto advanceL = [&]() {
+    const bool more = issuedL < iters, wrap = more && (slabL + 1 == slabs);
+    const int8_t* cand = args.panels + (int64_t)(nextL & 0xffffu) * args.panelStride + k0;
+    baseLane = wrap ? cand : baseLane + (more ? RING_K : 0); slabL = wrap ? 0 : slabL + (more ? 1 : 0); pairL += wrap ? 1 : 0; issuedL += more ? 1 : 0;
+  };
+  auto advanceA = [&]() {
+    const bool more = issuedA < iters, wrap = more && (slabA + 1 == slabs);
+    const int8_t* cand = args.panels + (int64_t)(nextA >> 16) * args.panelStride + k0;
+    baseA = wrap ? cand : baseA + (more ? RING_K : 0); slabA = wrap ? 0 : slabA + (more ? 1 : 0); pairA += wrap ? 1 : 0; issuedA += more ? 1 : 0;
+  };
+  /* ring position of the next unit to fill (byte offset, wraps at RING_BYTES) */
+  uint32_t fillOff = 0;
+  auto next_unit = [&]() { const uint32_t u = fillOff; fillOff += RING_UNIT_BYTES; fillOff = fillOff == (uint32_t)RING_BYTES ? 0u : fillOff; return u; };
+  auto fill_lane = [&](int h, int r, uint32_t unitOff) { dma16(dmaBase + unitOff + (uint32_t)r * 4096u, baseLane + srcLane[h][r]); };
+  auto fill_a = [&](int h, int r, uint32_t unitOff) { dma16(dmaBase + unitOff + (uint32_t)r * 4096u, baseA + srcA[h][r]); };
+
+  const int rowOff = (lane & 31) * RING_K, sw = S::swz(lane & 31), hi = lane >> 5;
+  int kOff[4];
+  #pragma unroll
+  for (int kk = 0; kk < 4; ++kk) { kOff[kk] = ((2 * kk + hi) ^ sw) << 4; }
+  v4i fl[2][4], fa[2][4];
+  /* fragment read i (0..3 lane operand, 4..7 A operand) of K step kk; laneUnit / aUnit: byte offsets of this wave's units */
+  auto rd = [&](int i, int set, int kk, uint32_t laneUnit, uint32_t aUnit) {
+    if (i < 4) { fl[set][i] = *reinterpret_cast<const v4i*>(lds + laneUnit + rowOff + i * 32 * RING_K + kOff[kk]); }
+    else { fa[set][i - 4] = *reinterpret_cast<const v4i*>(lds + aUnit + rowOff + (i - 4) * 32 * RING_K + kOff[kk]); }
+  };
+  auto mm = [&](int n, int set) { const int a = n >> 2, b = n & 3; acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[set][a], fl[set][b], acc[a][b], 0, 0, 0); };
+  /* a run of MFMAs with fragment reads paired to the first of them, closed for the scheduler */
+  auto run = [&](auto mmFirst_, auto mmCount_, auto mmSet_, auto rdFirst_, auto rdCount_, auto rdSet_, auto rdKk_, uint32_t laneUnit, uint32_t aUnit) {
+    constexpr int mmFirst = decltype(mmFirst_)::value, mmCount = decltype(mmCount_)::value, mmSet = decltype(mmSet_)::value;
+    constexpr int rdFirst = decltype(rdFirst_)::value, rdCount = decltype(rdCount_)::value, rdSet = decltype(rdSet_)::value, rdKk = decltype(rdKk_)::value;
+    #pragma unroll
+    for (int i = 0; i < rdCount; ++i) { rd(rdFirst + i, rdSet, rdKk, laneUnit, aUnit); }
+    #pragma unroll
+    for (int n = 0; n < mmCount; ++n) { mm(mmFirst + n, mmSet); }
+    #pragma unroll
+    for (int i = 0; i < rdCount; ++i) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); }
+    if constexpr (mmCount > rdCount) { __builtin_amdgcn_sched_group_barrier(0x008, mmCount - rdCount, 0); }
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  /* a whole K step whose loads are spread four MFMAs apart: reads under the first eight MFMAs */
+  auto unit_offset = [&](uint32_t slabOff, int unit) { uint32_t o = slabOff + (uint32_t)unit * RING_UNIT_BYTES; return o >= (uint32_t)RING_BYTES ? o - (uint32_t)RING_BYTES : o; };
+
+  /* prologue: slabs 0 and 1 requested in full (eight units); slab 0 landed and published; its first fragments requested */
+  #pragma unroll
+  for (int s0 = 0; s0 < 2; ++s0) {
+    if (s0) { peekL(); advanceL(); peekA(); advanceA(); }
+    #pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const uint32_t u = next_unit();
+      #pragma unroll
+      for (int r = 0; r < 4; ++r) { fill_lane(h, r, u); }
+    }
+    #pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const uint32_t u = next_unit();
+      #pragma unroll
+      for (int r = 0; r < 4; ++r) { fill_a(h, r, u); }
+    }
+  }
+  peekL(); advanceL();                     /* lane stream: next to request is slab 2; A stream stays on slab 1 until the first barrier */
+  asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+  __syncthreads();
+  uint32_t slabOff = 0;                    /* ring offset of the first unit of the slab being contracted */
+  {
+    const uint32_t lu = unit_offset(slabOff, wy), au = unit_offset(slabOff, 2 + wx);
+    #pragma unroll
+    for (int i = 0; i < 8; ++i) { rd(i, 0, 0, lu, au); }
+  }
+  __builtin_amdgcn_s_waitcnt(0xC07F);
+  __builtin_amdgcn_sched_barrier(0);
+
+  for (int it = 0; it < iters; ++it) {
+    const uint32_t lu = unit_offset(slabOff, wy), au = unit_offset(slabOff, 2 + wx);
+    uint32_t nextOff = slabOff + 4u * RING_UNIT_BYTES; nextOff = nextOff >= (uint32_t)RING_BYTES ? nextOff - (uint32_t)RING_BYTES : nextOff;
+    const uint32_t nlu = unit_offset(nextOff, wy), nau = unit_offset(nextOff, 2 + wx);
+    peekL(); peekA();
+    /* K step 0: MFMAs on set 0, fragments of step 1 into set 1, lane unit 0 of slab it + 2 */
+    { const uint32_t u = next_unit();
+      run(IC<0>{}, IC<4>{}, IC<0>{}, IC<0>{}, IC<4>{}, IC<1>{}, IC<1>{}, lu, au); fill_lane(0, 0, u); __builtin_amdgcn_sched_barrier(0);
+      run(IC<4>{}, IC<4>{}, IC<0>{}, IC<4>{}, IC<4>{}, IC<1>{}, IC<1>{}, lu, au); fill_lane(0, 1, u); __builtin_amdgcn_sched_barrier(0);
+      run(IC<8>{}, IC<4>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<1>{}, IC<1>{}, lu, au); fill_lane(0, 2, u); __builtin_amdgcn_sched_barrier(0);
+      run(IC<12>{}, IC<4>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<1>{}, IC<1>{}, lu, au); fill_lane(0, 3, u); __builtin_amdgcn_sched_barrier(0); }
+    /* K step 1: MFMAs on set 1, fragments of step 2 into set 0, lane unit 1 of slab it + 2 */
+    { const uint32_t u = next_unit();
+      run(IC<0>{}, IC<4>{}, IC<1>{}, IC<0>{}, IC<4>{}, IC<0>{}, IC<2>{}, lu, au); fill_lane(1, 0, u); __builtin_amdgcn_sched_barrier(0);
+      run(IC<4>{}, IC<4>{}, IC<1>{}, IC<4>{}, IC<4>{}, IC<0>{}, IC<2>{}, lu, au); fill_lane(1, 1, u); __builtin_amdgcn_sched_barrier(0);
+      run(IC<8>{}, IC<4>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<2>{}, lu, au); fill_lane(1, 2, u); __builtin_amdgcn_sched_barrier(0);
+      run(IC<12>{}, IC<4>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<2>{}, lu, au); fill_lane(1, 3, u); __builtin_amdgcn_sched_barrier(0); }
+    /* K step 2: MFMAs on set 0, fragments of step 3 into set 1, no loads */
+    run(IC<0>{}, IC<4>{}, IC<0>{}, IC<0>{}, IC<4>{}, IC<1>{}, IC<3>{}, lu, au);
+    run(IC<4>{}, IC<8>{}, IC<0>{}, IC<4>{}, IC<4>{}, IC<1>{}, IC<3>{}, lu, au);
+    /* slab it + 1 has landed (own loads: only the eight lane loads above may be outstanding) and every wave has read
+     * its last fragments of slab it: publish, release */
+    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
+    run(IC<12>{}, IC<4>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<1>{}, IC<3>{}, lu, au);
+    advanceL(); advanceA();
+    __builtin_amdgcn_sched_barrier(0);
+    /* K step 3: MFMAs on set 1, first fragments of slab it + 1 into set 0, both A units of slab it + 2 */
+    { const uint32_t u0 = next_unit(), u1 = next_unit();
+      run(IC<0>{}, IC<2>{}, IC<1>{}, IC<0>{}, IC<2>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(0, 0, u0); __builtin_amdgcn_sched_barrier(0);
+      run(IC<2>{}, IC<2>{}, IC<1>{}, IC<2>{}, IC<2>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(0, 1, u0); __builtin_amdgcn_sched_barrier(0);
+      run(IC<4>{}, IC<2>{}, IC<1>{}, IC<4>{}, IC<2>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(0, 2, u0); __builtin_amdgcn_sched_barrier(0);
+      run(IC<6>{}, IC<2>{}, IC<1>{}, IC<6>{}, IC<2>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(0, 3, u0); __builtin_amdgcn_sched_barrier(0);
+      run(IC<8>{}, IC<2>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(1, 0, u1); __builtin_amdgcn_sched_barrier(0);
+      run(IC<10>{}, IC<2>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(1, 1, u1); __builtin_amdgcn_sched_barrier(0);
+      run(IC<12>{}, IC<2>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(1, 2, u1); __builtin_amdgcn_sched_barrier(0);
+      run(IC<14>{}, IC<2>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(1, 3, u1); __builtin_amdgcn_sched_barrier(0); }
+    __builtin_amdgcn_s_waitcnt(0xC07F);   /* lgkmcnt(0): the fragments of the next slab were requested eight MFMAs ago */
+    slabOff = nextOff;
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   /* no direct load may still be writing LDS when the workgroup ends */
+
+  constexpr int aBegin = 0, aEnd = 4;
+  HYK_GRAM_EPILOGUE(EXCL)
+}
+
 /* ------------------------------------------------------------------ CRT reconstruction */
 struct ReconTable {
   int32_t order;
@@ -454,7 +646,7 @@ __global__ void fill_zero_kernel(uint4* __restrict__ p, int64_t n16) {
 /* ------------------------------------------------------------------ host-side planning */
 struct Launch { GramArgs args; int epi; };
 
-int g_bk = 0;   /* 0: direct-to-LDS kernel (default); 64 / 128: register-staged kernel with that K slab (hykGramSetSlab) */
+int g_bk = 0;   /* 0: direct-to-LDS ring of 128-byte rows (default); 2: direct-to-LDS ring of 64-byte rows; 64 / 128: register-staged kernel with that K slab (hykGramSetSlab) */
 
 /* optional per-launch timing of the contraction kernel with HIP events on its own stream */
 struct Timed { hipEvent_t start, stop; };
@@ -484,6 +676,17 @@ template <int EPI, bool EXCL> hipError_t launch_dma(hipStream_t stream, const Gr
   return hipGetLastError();
 }
 
+template <int EPI, bool EXCL> hipError_t launch_ring(hipStream_t stream, const GramArgs& a) {
+  static bool attr = false;
+  if (!attr) { hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gram_ring_kernel<EPI, EXCL>), hipFuncAttributeMaxDynamicSharedMemorySize, RING_BYTES); if (e != hipSuccess) { return e; } attr = true; }
+  const int blocks = a.itemsPerXcd * XCDS;
+  Timed t{ nullptr, nullptr };
+  if (g_profile) { if (hipEventCreate(&t.start) != hipSuccess || hipEventCreate(&t.stop) != hipSuccess) { return hipErrorUnknown; } (void)hipEventRecord(t.start, stream); }
+  gram_ring_kernel<EPI, EXCL><<<blocks, G_THREADS, RING_BYTES, stream>>>(a);
+  if (g_profile) { (void)hipEventRecord(t.stop, stream); g_timed.push_back(t); }
+  return hipGetLastError();
+}
+
 int compute_units() {
   static int units = 0;
   if (units == 0) { int dev = 0, n = 0; if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) { units = n; } else { units = 256; } }
@@ -492,26 +695,30 @@ int compute_units() {
 
 hipError_t launch_gram(hipStream_t stream, GramArgs& a, int epi, int maxProducts, bool unshared) {
   int maxPairs = 1; for (int g = 0; g < a.groupCount; ++g) { maxPairs = a.groups[g].pairCount > maxPairs ? a.groups[g].pairCount : maxPairs; }
-  const int bk = g_bk == 0 ? DMA_BK : g_bk; int kCap = (maxProducts / maxPairs) / bk * bk; if (kCap < bk) { return hipErrorInvalidValue; }
+  const int bk = g_bk == 0 ? RING_K : (g_bk == 2 ? DMA_BK : g_bk); int kCap = (maxProducts / maxPairs) / bk * bk; if (kCap < bk) { return hipErrorInvalidValue; }
   /* K split.  One workgroup runs per compute unit, so a launch takes rounds = ceil(items / units) item times; an item costs
-   * its slabs plus a fixed prologue / epilogue (65536 reductions and atomics) worth about 48 slab times.  Take the split
-   * count that minimises rounds x (slabs + 48); the cap keeps the int32 sums exact. */
+   * its K range plus a fixed prologue / epilogue (65536 reductions and atomics) worth about 48 x 64 K-bytes of it.  Take
+   * the split count that minimises rounds x (K range + epilogue); the cap keeps the int32 sums exact. */
   const int64_t base = (int64_t)a.groupCount * a.tileCount; const int units = compute_units();
   const int minSplits = (a.K + kCap - 1) / kCap; int splits = minSplits; double best = -1.;
   for (int cand = minSplits; cand <= minSplits + 15; ++cand) {
     const int len = ((a.K + cand - 1) / cand + bk - 1) / bk * bk; if (len < 16 * bk && cand > minSplits) { break; }
     const int count = (a.K + len - 1) / len; const int64_t rounds = (base * count + units - 1) / units;
-    const double cost = (double)rounds * ((double)(len / bk) + 48.);
+    const double cost = (double)rounds * ((double)len / 64. + 48.);   /* in units of 64 K-bytes of contraction */
     if (best < 0. || cost < best * 0.98) { best = cost; splits = cand; }   /* a further split has to win by 2 % */
   }
   int kLen = ((a.K + splits - 1) / splits + bk - 1) / bk * bk; if (kLen > kCap) { kLen = kCap; }
   if (kLen > a.K) { kLen = a.K; }
-  a.kLen = kLen; a.kSplits = (a.K + kLen - 1) / kLen; a.exclusive = (unshared && a.kSplits == 1 && g_bk == 0) ? 1 : 0;
+  a.kLen = kLen; a.kSplits = (a.K + kLen - 1) / kLen; a.exclusive = (unshared && a.kSplits == 1 && (g_bk == 0 || g_bk == 2)) ? 1 : 0;
   const int64_t total = base * a.kSplits; if (total > 0x7fffffff / 2) { return hipErrorInvalidValue; }
   a.totalItems = (int)total; a.itemsPerXcd = (int)((total + XCDS - 1) / XCDS);
   if (total * a.tileCount >= (1ll << 32) || total * a.kSplits >= (1ll << 32)) { return hipErrorInvalidValue; }
   a.tileMagic = a.tileCount > 1 ? (uint32_t)((1ull << 32) / (uint32_t)a.tileCount) + 1u : 0u; a.splitMagic = a.kSplits > 1 ? (uint32_t)((1ull << 32) / (uint32_t)a.kSplits) + 1u : 0u;
   if (g_bk == 0) {
+    if (a.exclusive) { return epi == EPI_MOD ? launch_ring<EPI_MOD, true>(stream, a) : launch_ring<EPI_I64, true>(stream, a); }
+    return epi == EPI_MOD ? launch_ring<EPI_MOD, false>(stream, a) : launch_ring<EPI_I64, false>(stream, a);
+  }
+  if (g_bk == 2) {
     if (a.exclusive) { return epi == EPI_MOD ? launch_dma<EPI_MOD, true>(stream, a) : launch_dma<EPI_I64, true>(stream, a); }
     return epi == EPI_MOD ? launch_dma<EPI_MOD, false>(stream, a) : launch_dma<EPI_I64, false>(stream, a);
   }
@@ -623,7 +830,7 @@ extern "C" int hykMfmaCeiling(hipStream_t stream, int32_t blocks, int32_t iters,
   return rc;
 }
 
-extern "C" int hykGramSetSlab(int32_t bk) { if (bk != 0 && bk != 64 && bk != 128) { return -1; } g_bk = bk; return 0; }
+extern "C" int hykGramSetSlab(int32_t bk) { if (bk != 0 && bk != 2 && bk != 64 && bk != 128) { return -1; } g_bk = bk; return 0; }
 
 extern "C" size_t hykGramWorkspaceBytes(int32_t kind, int32_t Complex, int32_t N, int32_t orderA) {
   if (N <= 0 || orderA <= 0) { return 0; }

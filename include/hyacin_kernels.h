@@ -55,7 +55,8 @@ int hykGramProfile(int32_t enable);
 int hykGramProfileRead(double* totalMs, int32_t* launches);
 
 /* Variant of the contraction kernel (tuning knob): 0 = operand slabs loaded straight from global memory into a ring of
- * LDS stages (default); 64 / 128 = staged through registers with that many K bytes per LDS stage. */
+ * LDS units with 128-byte rows (default); 2 = the same with 64-byte rows and four stages; 64 / 128 = staged through
+ * registers with that many K bytes per LDS stage. */
 int hykGramSetSlab(int32_t bk);
 
 /* Measurement hook (no counterpart in the reference): int8 tera-ops per second that a register-only loop of

@@ -141,15 +141,16 @@ def test_gram_extreme_values_and_long_k(gl, oracle):
     assert np.array_equal(gl.gram("crt", 0, N, 2, panels, 2), want)
 
 
-@pytest.mark.parametrize("slab", [64, 128])
-def test_gram_register_staged_variants(gl, oracle, slab):
-    """The register-staged contraction kernels (K slab 64 / 128) give the same bits as the default direct-to-LDS one."""
+@pytest.mark.parametrize("slab", [0, 2, 64, 128])
+@pytest.mark.parametrize("cplx,order,K,rows", [(0, 3, 640, 600), (1, 2, 1536, 1500), (0, 2, 4224, 4200)])
+def test_gram_kernel_variants(gl, oracle, slab, cplx, order, K, rows):
+    """Every contraction kernel variant (direct-to-LDS rings with 64- and 128-byte rows, register-staged K slabs) gives the same bits."""
     rng = np.random.default_rng(36)
-    panels = random_panels(rng, 3, 270, 640, 600, -125, 126)
-    want = oracle.i8herk("crt", 0, 270, 3, panels, 0, 2)
+    panels = random_panels(rng, oracle.n_panels("crt", order, cplx), 270, K, rows, -125, 126)
+    want = oracle.i8herk("crt", cplx, 270, order, panels, 0, 2)
     try:
         assert gl.L.hykGramSetSlab(slab) == 0
-        got = gl.gram("crt", 0, 270, 3, panels, 2)
+        got = gl.gram("crt", cplx, 270, order, panels, 2)
     finally:
         gl.L.hykGramSetSlab(0)
     assert np.array_equal(got, want)
