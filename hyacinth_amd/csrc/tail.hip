@@ -177,6 +177,7 @@ __global__ __launch_bounds__(T_THREADS) void jacobi_block_round_kernel(int32_t N
       }
     }
   }
+  if (applied == 0) { return; }                  /* nothing rotated (same decision in every thread): the columns in memory are current */
   #pragma unroll
   for (int c = 0; c < NC; ++c) {
     #pragma unroll
@@ -188,7 +189,7 @@ __global__ __launch_bounds__(T_THREADS) void jacobi_block_round_kernel(int32_t N
       }
     }
   }
-  if (threadIdx.x == 0 && applied) { atomicAdd(rotations, applied); }
+  if (threadIdx.x == 0) { atomicAdd(rotations, applied); }
 }
 
 template <bool CPLX>
