@@ -73,6 +73,8 @@ struct GramArgs {
   int32_t N, nT, tileCount, kLen, kSplits, K, groupCount, totalItems, itemsPerXcd;
   int32_t exclusive;                /* 1: this launch's items are the only writers of their accumulator entries */
   uint32_t tileMagic, splitMagic;   /* floor(2^32 / d) + 1: x / d == mulhi(x, magic) while x * d < 2^32 (checked on the host); 0 for d == 1 */
+  /* set-aligned schedule (ring kernel): a set = the tileCount tiles of one (group, K split); slots = compute units per XCD */
+  int32_t slotShift, roundsPerXcd, setCount, mainRounds, leftover, perRound; uint32_t mainMagic, leftMagic;
   GramGroup groups[MAX_GROUPS];
   uint32_t pairs[MAX_PAIRS];  /* lanePanel | aPanel << 16 */
 };
@@ -429,10 +431,23 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_ring_kernel(const GramArgs 
   extern __shared__ __align__(16) int8_t lds[];
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), wy = wave & 1, wx = wave >> 1;
 
-  const int item = (int)(blockIdx.x % XCDS) * args.itemsPerXcd + (int)(blockIdx.x / XCDS);
-  if ((int)(blockIdx.x / XCDS) >= args.itemsPerXcd || item >= args.totalItems) { return; }
-  const int gk = args.tileMagic ? (int)(((uint64_t)(uint32_t)item * args.tileMagic) >> 32) : item, t = item - gk * args.tileCount;
-  const int g = args.splitMagic ? (int)(((uint64_t)(uint32_t)gk * args.splitMagic) >> 32) : gk, ks = gk - g * args.kSplits;
+  /* Set-aligned schedule.  The workgroups of an XCD start in the order of their index and, one per compute unit, run in
+   * rounds of `slots`.  All tiles of a set (one group, one K split) read the same panels, so a round should hold tiles
+   * of one set: a set takes mainRounds whole rounds, and the tileCount % slots tiles left over are packed perRound sets
+   * to a round behind all the whole ones.  Round rr of the launch is round rr / 8 of XCD rr % 8, which spreads the
+   * left-over rounds (they read the most panel bytes per tile) over the XCDs. */
+  const int xcd = (int)(blockIdx.x % XCDS), q = (int)(blockIdx.x / XCDS), slots = 1 << args.slotShift;
+  const int round = q >> args.slotShift, slot = q & (slots - 1), rr = round * XCDS + xcd;
+  auto divide = [](int v, uint32_t magic) { return magic ? (int)(((uint64_t)(uint32_t)v * magic) >> 32) : v; };
+  int set, t;
+  if (rr < args.setCount * args.mainRounds) { set = divide(rr, args.mainMagic); t = ((rr - set * args.mainRounds) << args.slotShift) + slot; }
+  else {
+    if (args.leftover == 0) { return; }
+    const int inRound = divide(slot, args.leftMagic); set = (rr - args.setCount * args.mainRounds) * args.perRound + inRound;
+    if (inRound >= args.perRound || set >= args.setCount) { return; }
+    t = (args.mainRounds << args.slotShift) + (slot - inRound * args.leftover);
+  }
+  const int g = divide(set, args.splitMagic), ks = set - g * args.kSplits;
   int tb = 0; while ((tb + 1) * (tb + 2) / 2 <= t) { ++tb; }
   const int ta = t - tb * (tb + 1) / 2;
   const GramGroup grp = args.groups[g];
@@ -679,7 +694,7 @@ template <int EPI, bool EXCL> hipError_t launch_dma(hipStream_t stream, const Gr
 template <int EPI, bool EXCL> hipError_t launch_ring(hipStream_t stream, const GramArgs& a) {
   static bool attr = false;
   if (!attr) { hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gram_ring_kernel<EPI, EXCL>), hipFuncAttributeMaxDynamicSharedMemorySize, RING_BYTES); if (e != hipSuccess) { return e; } attr = true; }
-  const int blocks = a.itemsPerXcd * XCDS;
+  const int blocks = XCDS * a.roundsPerXcd * (1 << a.slotShift);
   Timed t{ nullptr, nullptr };
   if (g_profile) { if (hipEventCreate(&t.start) != hipSuccess || hipEventCreate(&t.stop) != hipSuccess) { return hipErrorUnknown; } (void)hipEventRecord(t.start, stream); }
   gram_ring_kernel<EPI, EXCL><<<blocks, G_THREADS, RING_BYTES, stream>>>(a);
@@ -715,6 +730,13 @@ hipError_t launch_gram(hipStream_t stream, GramArgs& a, int epi, int maxProducts
   if (total * a.tileCount >= (1ll << 32) || total * a.kSplits >= (1ll << 32)) { return hipErrorInvalidValue; }
   a.tileMagic = a.tileCount > 1 ? (uint32_t)((1ull << 32) / (uint32_t)a.tileCount) + 1u : 0u; a.splitMagic = a.kSplits > 1 ? (uint32_t)((1ull << 32) / (uint32_t)a.kSplits) + 1u : 0u;
   if (g_bk == 0) {
+    /* set-aligned schedule; compute units per XCD rounded down to a power of two (32 on this device) */
+    int slots = units / XCDS; a.slotShift = 0; while ((2 << a.slotShift) <= slots) { ++a.slotShift; } slots = 1 << a.slotShift;
+    a.setCount = a.groupCount * a.kSplits; a.mainRounds = a.tileCount / slots; a.leftover = a.tileCount % slots; a.perRound = a.leftover ? slots / a.leftover : 0;
+    const int rounds = a.setCount * a.mainRounds + (a.leftover ? (a.setCount + a.perRound - 1) / a.perRound : 0);
+    a.roundsPerXcd = (rounds + XCDS - 1) / XCDS;
+    a.mainMagic = a.mainRounds > 1 ? (uint32_t)((1ull << 32) / (uint32_t)a.mainRounds) + 1u : 0u; a.leftMagic = a.leftover > 1 ? (uint32_t)((1ull << 32) / (uint32_t)a.leftover) + 1u : 0u;
+    if ((int64_t)rounds * a.mainRounds >= (1ll << 31) || (int64_t)a.setCount * a.kSplits >= (1ll << 31)) { return hipErrorInvalidValue; }
     if (a.exclusive) { return epi == EPI_MOD ? launch_ring<EPI_MOD, true>(stream, a) : launch_ring<EPI_I64, true>(stream, a); }
     return epi == EPI_MOD ? launch_ring<EPI_MOD, false>(stream, a) : launch_ring<EPI_I64, false>(stream, a);
   }

@@ -39,7 +39,11 @@ int32_t run_potrfp(const hyacinHandle_t* h, Factor& f, double eps, int32_t K, in
   int32_t* word = (int32_t*)h->pinnedWorkspace; *word = 0;
   HYH_KERNEL(hykPotrfp(h->hipStream, h->DeviceSMs, eps, K, N, f.type, f.G, f.ldg, f.Rt.p, f.ldr, jpiv, f.work.p, word));
   HYH_CHECK(hipStreamSynchronize(h->hipStream));
-  const int32_t rank = *word;
+  int32_t rank = *word;
+  if (rank < 0) {   /* the workgroups lost each other (a wait inside the kernel gave up): report no basis rather than a wrong one */
+    if (h->logger) { std::fprintf((FILE*)h->logger, "POTRFP-%s [N=%d] gave up waiting for a workgroup\n", type_tag(f.type), N); }
+    return 0;
+  }
   if (h->logger) { std::fprintf((FILE*)h->logger, "POTRFP-%s [eps=%.1le] [N=%d] [K=%d] [Cholesky-rank=%d]\n", type_tag(f.type), eps, N, K, rank); }
   return rank;
 }

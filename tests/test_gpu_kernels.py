@@ -4,7 +4,7 @@ import ctypes as C
 import numpy as np
 import pytest
 
-from util import ALL_KINDS, INT_MAX, rand_matrix
+from util import ALL_KINDS, INT_MAX, haar, rand_matrix
 
 pytestmark = pytest.mark.gpu
 
@@ -181,3 +181,107 @@ def test_dequantize(gl, oracle, cplx):
                 assert (np.abs(got[..., 1::2] - want[..., 1::2]) <= scale * 2.0**-100).all()
             else:
                 assert np.array_equal(got, want)
+
+
+def spd_raw(rng, N, r, cplx, gbase, floor=1e-9):
+    """Hermitian positive matrix with a separated spectrum (r leading values 10^(-i/3), the rest `floor`) in the raw
+    Gram layout [column][row][width]; a double-double matrix carries a non-zero low word."""
+    U = haar(rng, N, N, bool(cplx))
+    sig = np.concatenate([10.0 ** (-np.arange(r) / 3.0), floor * np.ones(N - r)])
+    Gm = (U * sig ** 2) @ U.conj().T
+    Gm = (Gm + Gm.conj().T) / 2
+    Gt = Gm.T
+    dd = gbase == 6
+    raw = np.zeros((N, N, (2 if dd else 1) * (2 if cplx else 1)))
+    step = 2 if dd else 1
+    raw[..., 0] = Gt.real
+    if cplx:
+        raw[..., step] = Gt.imag
+    if dd:
+        low = np.abs(Gt.real) * 2.0**-55 * rng.uniform(-1, 1, (N, N))
+        low = (low + low.T) / 2                 # keeps the matrix Hermitian
+        raw[..., 1] = low
+    return raw
+
+
+def spd_exact_dd(rng, N, r, cplx):
+    """B^H B of an r x N integer matrix whose row i is scaled by 2^-i, computed in Python integers and split exactly into
+    double-double words: a positive semi-definite matrix of rank r that is exact to the last bit of the low word, with
+    a spectrum spanning 2^(-2 r): what only double-double arithmetic can factor down to the last row."""
+    br = rng.integers(-2**15, 2**15, (r, N)).astype(object)
+    bi = rng.integers(-2**15, 2**15, (r, N)).astype(object) if cplx else None
+    gre = np.zeros((N, N), object)
+    gim = np.zeros((N, N), object)
+    for i in range(r):
+        w = 1 << (2 * (r - 1 - i))
+        gre += w * np.outer(br[i], br[i])
+        if cplx:
+            gre += w * np.outer(bi[i], bi[i])
+            gim += w * (np.outer(br[i], bi[i]) - np.outer(bi[i], br[i]))      # Im G[y, x] = sum re_y im_x - im_y re_x
+    raw = np.zeros((N, N, 4 if cplx else 2))
+    sh = -2 * (r - 1)
+    for y in range(N):
+        for x in range(N):
+            for part, g in ((0, gre), (2, gim)) if cplx else ((0, gre),):
+                v = int(g[y, x])
+                hi = float(v)
+                lo = float(v - int(hi))
+                raw[x, y, part] = np.ldexp(hi, sh)
+                raw[x, y, part + 1] = np.ldexp(lo, sh)
+    return raw
+
+
+# (N, leading values, K, eps for FP64, eps for double-double, floor, compute units offered)
+POTRFP_CASES = [(24, 9, 24, 1e-6, 1e-6, 1e-9, 256), (150, 40, 150, 1e-6, 1e-10, 1e-13, 256), (150, 15, 150, 0.0, 0.0, 1e-5, 3),
+                (150, 60, 17, 1e-12, 1e-12, 1e-15, 256), (700, 64, 700, 1e-6, 1e-9, 1e-12, 256)]
+
+
+@pytest.mark.parametrize("gbase", [0, 6])        # FP64, double-double
+@pytest.mark.parametrize("cplx", [0, 1])
+@pytest.mark.parametrize("N,r,K,eps64,epsdd,floor,units", POTRFP_CASES)
+def test_potrfp_kernel(gl, oracle, gbase, cplx, N, r, K, eps64, epsdd, floor, units):
+    """hykPotrfp against the oracle's pivoted Cholesky (src/hyacin_potrfp.cu:119-318): same rank, same pivots, factor rows equal
+    to rounding (the two sum in different orders, and row t carries the rounding of the Schur complement it came from, so
+    the bound grows with d_0 / d_t).  The cut-off sits well above the rounding level of the arithmetic and well above the
+    floor of the spectrum, so the rank is not decided by rounding.  `units` limits the workgroups, so that wavefronts
+    own several columns."""
+    from gpu_util import dev, zeros, ptr, stream, sync, host
+    rng = np.random.default_rng(41 + cplx + gbase)
+    gtype = gbase + cplx
+    eps = epsdd if gbase == 6 else eps64
+    exact = gbase == 6 and N <= 150 and eps > 0.
+    raw = spd_exact_dd(rng, N, min(r, 30), cplx) if exact else spd_raw(rng, N, r, cplx, gbase, floor)
+    work = raw.copy()
+    want_rank, want_piv = oracle.potrfp(work, gtype, eps, K)
+    if exact:
+        assert want_rank == min(min(r, 30), K)
+    width = raw.shape[2]
+    ldr = min(N, K + 1)
+    Rt = zeros(N * ldr * width * 8)
+    jp = zeros(N * 4)
+    rk = zeros(4)
+    ws = zeros(gl.L.hykPotrfpWorkspaceBytes(N, gtype))
+    assert gl.L.hykPotrfp(stream(), units, eps, K, N, gtype, ptr(dev(raw)), N, ptr(Rt), ldr, ptr(jp), ptr(ws), ptr(rk)) == 0
+    sync()
+    rank = int(host(rk, np.int32)[0])
+    piv = host(jp, np.int32)
+    assert rank == want_rank
+    assert sorted(piv.tolist()) == list(range(1, N + 1))
+    assert np.array_equal(piv[:rank], want_piv[:rank])
+    got = host(Rt, np.float64, (N, ldr, width))                    # [column l][row t]
+    ref = np.transpose(work, (1, 0, 2))                           # oracle: row t of R in row t of the column-permuted matrix
+    p = want_piv - 1
+    unit = 2.0**-100 if gbase == 6 else 2.0**-53
+    d0 = ref[0, 0, 0] ** 2
+    for t in range(rank):
+        a = got[p[t:], t, :]                                      # R[t, columns in pivot order from the diagonal on]
+        b = ref[t, t:, :]
+        if gbase == 6:
+            a = a[..., 0::2] + a[..., 1::2]
+            b = b[..., 0::2] + b[..., 1::2]
+        scale = np.abs(b).max()
+        bound = 1e3 * unit * d0 / ref[t, t, 0] ** 2
+        assert np.abs(a - b).max() <= bound * scale, (t, np.abs(a - b).max(), scale, bound)
+    # entries below the diagonal (in pivot order) stay zero
+    for t in range(1, rank):
+        assert not got[p[:t], t, :].any()
