@@ -103,7 +103,7 @@ constexpr int POLL_WAVES = MAX_WORKGROUPS / 64;
 struct Exchange { double x[P_WAVES], y[P_WAVES], t[P_WAVES], rx[POLL_WAVES], ry[POLL_WAVES], rt[POLL_WAVES]; int32_t i[P_WAVES], ri[POLL_WAVES]; int32_t failed; };
 
 /* Every wavefront holds one partial in its lane 0 (a wavefront works on one column at a time); afterwards the lanes
- * 0..15 of the first wavefront hold the workgroup's result.  One barrier; it also waits for this wavefront's stores. */
+ * 0..15 of the first wavefront hold the workgroup's result.  One barrier. */
 template <bool DD>
 __device__ __forceinline__ void reduce_leaders(Exchange& ex, double& bx, double& by, int32_t& bi, double& tr) {
   static_assert(P_WAVES == 16, "four butterfly steps");
@@ -184,6 +184,7 @@ __global__ __launch_bounds__(P_THREADS) void potrfp_kernel(const PotrfArgs a) {
     }
   }
   if (wg == 0) { for (int l = tid; l < N; l += P_THREADS) { a.jpiv[l] = l + 1; a.pos[l] = l; } }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   reduce_leaders<DD>(ex, bx, by, bi, tr);
   ++epoch;
   publish(&a.records[(epoch & 1) * MAX_WORKGROUPS + wg], bx, by, tr, bi, epoch);
@@ -229,7 +230,10 @@ __global__ __launch_bounds__(P_THREADS) void potrfp_kernel(const PotrfArgs a) {
         if (d.v.x > 0.) { better(DD, bx, by, bi, d.v.x, d.v.y, l); }
       }
     }
-    reduce_leaders<DD>(ex, bx, by, bi, tr);   /* its barrier waits for the stores above */
+    /* the factor entries have to be in memory before the record that lets other workgroups go on; a workgroup barrier
+     * does not wait for the stores of its wavefronts, so every wavefront waits for its own */
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    reduce_leaders<DD>(ex, bx, by, bi, tr);
     ++k; ++epoch;
     publish(&a.records[(epoch & 1) * MAX_WORKGROUPS + wg], bx, by, tr, bi, epoch);
     collect(ex, &a.records[(epoch & 1) * MAX_WORKGROUPS], nwg, epoch, bx, by, bi, tr);
