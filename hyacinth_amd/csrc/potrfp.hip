@@ -45,6 +45,7 @@ constexpr int P_WAVES = P_THREADS / 64;
  * words arrive in; no word has to wait for another. */
 struct Record { uint64_t w[8]; };
 constexpr int RECORD_WORDS = 7;
+constexpr int STAGE_BYTES = 48 * 1024;
 constexpr int MAX_WORKGROUPS = 256;
 constexpr int SPIN_LIMIT = 1 << 22;   /* polls of one record before the run is given up (seconds; a healthy wait is microseconds) */
 
@@ -172,6 +173,8 @@ __global__ __launch_bounds__(P_THREADS) void potrfp_kernel(const PotrfArgs a) {
   /* column gwave + i nwaves belongs to this wavefront for the whole run; bit i of finished: it has been a pivot */
   uint64_t finished = 0;
   __shared__ Exchange ex;
+  constexpr int STAGE = STAGE_BYTES / (WE * 8);   /* factor entries of the pivot column that fit the LDS stage */
+  __shared__ __attribute__((aligned(16))) double stage[STAGE_BYTES / 8];
   if (tid == 0) { ex.failed = 0; }
   __syncthreads();
 
@@ -201,8 +204,13 @@ __global__ __launch_bounds__(P_THREADS) void potrfp_kernel(const PotrfArgs a) {
       double* rc = &a.Rt[((int64_t)c * a.ldr + k) * WE]; sq.store(rc); if constexpr (CPLX) { R::zero().store(rc + WR); }
       const int p = a.pos[c], c0 = a.jpiv[k] - 1; a.jpiv[k] = c + 1; a.jpiv[p] = c0 + 1; a.pos[c] = k; a.pos[c0] = p;
     }
-    /* column c of R, shared by every dot product of this step: Rt[c][0..k), written by the wavefront that owns c */
+    /* column c of R, shared by every dot product of this step: Rt[c][0..k), written by the wavefront that owns c.  The
+     * workgroup fetches it once into LDS (what exceeds the stage is read from memory by every wavefront); the barrier
+     * of the previous step's reduction has made the stage free. */
     const double* rcol = &a.Rt[(int64_t)c * a.ldr * WE];
+    const int staged = k < STAGE ? k : STAGE;
+    for (int e = tid; e < staged * WE; e += P_THREADS) { stage[e] = __hip_atomic_load(const_cast<double*>(rcol) + e, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+    __syncthreads();
     bx = by = tr = 0.; bi = -1;
     int slot = 0;
     for (int l = gwave; l < N; l += nwaves, ++slot) {
@@ -214,7 +222,14 @@ __global__ __launch_bounds__(P_THREADS) void potrfp_kernel(const PotrfArgs a) {
       const R gre0 = R::load(g), d0 = R::load(&a.D[(int64_t)l * WR]); R gim0 = R::zero(); if constexpr (CPLX) { gim0 = R::load(g + WR); }
       R sre = R::zero(), sim = R::zero();
       #pragma unroll 8
-      for (int t = lane; t < k; t += 64) {
+      for (int t = lane; t < staged; t += 64) {
+        if constexpr (CPLX) {
+          R ar = R::load(&rl[(int64_t)t * WE]), ai = R::load(&rl[(int64_t)t * WE + WR]), br = R::load(&stage[t * WE]), bim = R::load(&stage[t * WE + WR]);
+          sre = R::fnma(ar, br, sre); sre = R::fnma(ai, bim, sre); sim = R::fnma(ar, bim, sim); sim = R::fnma(ai.neg(), br, sim);
+        } else { sre = R::fnma(R::load(&rl[(int64_t)t * WE]), R::load(&stage[t * WE]), sre); }
+      }
+      #pragma unroll 2
+      for (int t = staged + lane; t < k; t += 64) {
         if constexpr (CPLX) {
           R ar = R::load(&rl[(int64_t)t * WE]), ai = R::load(&rl[(int64_t)t * WE + WR]), br = R::load_shared(&rcol[(int64_t)t * WE]), bim = R::load_shared(&rcol[(int64_t)t * WE + WR]);
           /* S -= conj(a) b:  re -= ar br + ai bi;  im -= ar bi - ai br */
