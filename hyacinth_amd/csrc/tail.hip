@@ -81,28 +81,44 @@ __global__ __launch_bounds__(T_THREADS) void jacobi_round_kernel(int32_t N, int3
  * t, t + 256, ...) and rotates every cross pair (BC steps of BC disjoint pairs) before writing them back: BC times fewer
  * passes over B per sweep.  In the first round of a sweep the 2 BC columns go through a full round-robin instead, which
  * also covers the pairs inside each block.  Column norms are summed once per round and carried through the rotations
- * (alpha' = alpha - t gamma, beta' = beta + t gamma); only the BC cross products of a step need a workgroup reduction. */
-template <int NV>
-__device__ __forceinline__ void block_sum_many(double (&v)[NV], double* red, int parity) {
+ * (alpha' = alpha - t gamma, beta' = beta + t gamma); only the BC cross products of a step need a workgroup reduction.
+ * Blocks of 8 columns (512 threads, 4 rows each) halve the passes again but take 2.7 times as long per round on this
+ * device (half as many workgroups as compute units, twice the reduction work per workgroup): 4-column blocks stay. */
+/* Sums NV values over the workgroup; lane i < NV of every wavefront returns the sum of value i.  `red` holds two halves of
+ * HALF doubles used alternately (`parity`), so that one barrier per call is enough: a wavefront can only be two calls
+ * ahead of the slowest one after that one has left the half. */
+template <int NV, int THREADS, int HALF>
+__device__ __forceinline__ double block_sum_lanes(double (&v)[NV], double* red, int parity) {
+  static_assert((THREADS / 64) * NV <= HALF, "a half holds one value per wavefront and summand");
+  static_assert(NV <= 64, "one lane per summand");
   #pragma unroll
   for (int i = 0; i < NV; ++i) {
     #pragma unroll
     for (int off = 32; off > 0; off >>= 1) { v[i] += __shfl_xor(v[i], off, 64); }
   }
-  double* mine = red + parity * (T_THREADS / 64) * NV;
+  double* mine = red + parity * HALF;
   if ((threadIdx.x & 63) == 0) {
     #pragma unroll
     for (int i = 0; i < NV; ++i) { mine[(threadIdx.x >> 6) * NV + i] = v[i]; }
   }
   __syncthreads();
+  double s = 0.; const int lane = threadIdx.x & 63;
+  if (lane < NV) { for (int w = 0; w < THREADS / 64; ++w) { s += mine[w * NV + lane]; } }
+  return s;
+}
+/* the same, every thread gets all NV sums */
+template <int NV, int THREADS, int HALF>
+__device__ __forceinline__ void block_sum_many(double (&v)[NV], double* red, int parity) {
+  const double s = block_sum_lanes<NV, THREADS, HALF>(v, red, parity);
   #pragma unroll
-  for (int i = 0; i < NV; ++i) { double s = 0.; for (int w = 0; w < T_THREADS / 64; ++w) { s += mine[w * NV + i]; } v[i] = s; }
+  for (int i = 0; i < NV; ++i) { v[i] = __shfl(s, i, 64); }
 }
 
-template <bool CPLX, int ROWS, int BC, bool FULL>
-__global__ __launch_bounds__(T_THREADS) void jacobi_block_round_kernel(int32_t N, int32_t nb, int32_t r, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations) {
+template <bool CPLX, int ROWS, int BC, bool FULL, int THREADS>
+__global__ __launch_bounds__(THREADS) void jacobi_block_round_kernel(int32_t N, int32_t nb, int32_t r, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations) {
   constexpr int W = CPLX ? 2 : 1, NC = 2 * BC, GV = BC * W;
-  __shared__ double red[2 * (T_THREADS / 64) * (NC > GV ? NC : GV)];
+  constexpr int HALF = (THREADS / 64) * (NC > GV ? NC : GV);
+  __shared__ double red[2 * HALF];
   const int i = blockIdx.x; int P, Q;
   if (i == 0) { P = nb - 1; Q = round; } else { P = (round + i) % (nb - 1); Q = (round - i + (nb - 1)) % (nb - 1); }
   if (P > Q) { const int t = P; P = Q; Q = t; }
@@ -116,7 +132,7 @@ __global__ __launch_bounds__(T_THREADS) void jacobi_block_round_kernel(int32_t N
   for (int c = 0; c < NC; ++c) {
     #pragma unroll
     for (int m = 0; m < ROWS; ++m) {
-      const int k = threadIdx.x + m * T_THREADS;
+      const int k = threadIdx.x + m * THREADS;
       #pragma unroll
       for (int w = 0; w < W; ++w) { x[c][m][w] = (live[c] && k < N) ? B[((int64_t)col[c] * N + k) * W + w] : 0.; }
     }
@@ -132,7 +148,7 @@ __global__ __launch_bounds__(T_THREADS) void jacobi_block_round_kernel(int32_t N
     }
     norm[c] = s;
   }
-  block_sum_many<NC>(norm, red, 0);
+  block_sum_many<NC, THREADS, HALF>(norm, red, 0);
   int applied = 0;
   /* FULL: first round of a sweep, all pairs of the 2 BC columns (round-robin); otherwise the BC x BC cross pairs */
   constexpr int STEPS = FULL ? NC - 1 : BC;
@@ -151,29 +167,46 @@ __global__ __launch_bounds__(T_THREADS) void jacobi_block_round_kernel(int32_t N
       }
       g[j * W] = gr; if constexpr (CPLX) { g[j * W + 1] = gi; }
     }
-    block_sum_many<GV>(g, red, (step + 1) & 1);
+    /* lane j < BC of every wavefront works out the rotation of pair j (square roots and divisions once instead of BC
+     * times per thread), then the lanes hand the parameters round */
+    const double sum = block_sum_lanes<GV, THREADS, HALF>(g, red, (step + 1) & 1);
+    const int lane = threadIdx.x & 63;
+    double gre = sum, gim = 0.;
+    if constexpr (CPLX) { gre = __shfl(sum, 2 * lane, 64); gim = __shfl(sum, 2 * lane + 1, 64); }
+    double alpha = 0., beta = 0.; bool pairLive = false;
     #pragma unroll
     for (int j = 0; j < BC; ++j) {
       const int fa = (j == 0) ? NC - 1 : (step + j) % (NC - 1), fb = (j == 0) ? step : (step - j + (NC - 1)) % (NC - 1);
       const int c0 = FULL ? (fa < fb ? fa : fb) : j, c1 = FULL ? (fa < fb ? fb : fa) : BC + (j + step) % BC;
-      const double gre = g[j * W], gim = CPLX ? g[j * W + (CPLX ? 1 : 0)] : 0.;
-      const double alpha = norm[c0], beta = norm[c1], g2 = gre * gre + gim * gim;
-      if (live[c0] && live[c1] && g2 > tol * tol * alpha * beta && g2 > 0.) {
-        const double gabs = sqrt(g2), zeta = (beta - alpha) / (2. * gabs);
-        const double t = (zeta >= 0. ? 1. : -1.) / (fabs(zeta) + sqrt(1. + zeta * zeta)), cs = 1. / sqrt(1. + t * t), sn = cs * t;
-        const double er = gre / gabs, ei = gim / gabs;
+      if (lane == j) { alpha = norm[c0]; beta = norm[c1]; pairLive = live[c0] && live[c1]; }
+    }
+    const double g2 = gre * gre + gim * gim;
+    const bool rotate = pairLive && g2 > tol * tol * alpha * beta && g2 > 0.;
+    double cs = 1., sn = 0., er = 1., ei = 0., shift = 0.;
+    if (rotate) {
+      const double gabs = sqrt(g2), zeta = (beta - alpha) / (2. * gabs);
+      const double t = (zeta >= 0. ? 1. : -1.) / (fabs(zeta) + sqrt(1. + zeta * zeta));
+      cs = 1. / sqrt(1. + t * t); sn = cs * t; er = gre / gabs; ei = gim / gabs; shift = t * gabs;
+    }
+    #pragma unroll
+    for (int j = 0; j < BC; ++j) {
+      const int fa = (j == 0) ? NC - 1 : (step + j) % (NC - 1), fb = (j == 0) ? step : (step - j + (NC - 1)) % (NC - 1);
+      const int c0 = FULL ? (fa < fb ? fa : fb) : j, c1 = FULL ? (fa < fb ? fb : fa) : BC + (j + step) % BC;
+      if (__shfl((int)rotate, j, 64)) {
+        const double csj = __shfl(cs, j, 64), snj = __shfl(sn, j, 64), erj = __shfl(er, j, 64), shj = __shfl(shift, j, 64);
+        [[maybe_unused]] const double eij = CPLX ? __shfl(ei, j, 64) : 0.;
         #pragma unroll
         for (int m = 0; m < ROWS; ++m) {
           if constexpr (CPLX) {
             const double pr = x[c0][m][0], pi = x[c0][m][1], q0 = x[c1][m][0], q1 = x[c1][m][1];
-            const double qr = q0 * er + q1 * ei, qi = q1 * er - q0 * ei;
-            x[c0][m][0] = cs * pr - sn * qr; x[c0][m][1] = cs * pi - sn * qi; x[c1][m][0] = sn * pr + cs * qr; x[c1][m][1] = sn * pi + cs * qi;
+            const double qr = q0 * erj + q1 * eij, qi = q1 * erj - q0 * eij;
+            x[c0][m][0] = csj * pr - snj * qr; x[c0][m][1] = csj * pi - snj * qi; x[c1][m][0] = snj * pr + csj * qr; x[c1][m][1] = snj * pi + csj * qi;
           } else {
-            const double pv = x[c0][m][0], qv = x[c1][m][0] * er;
-            x[c0][m][0] = cs * pv - sn * qv; x[c1][m][0] = sn * pv + cs * qv;
+            const double pv = x[c0][m][0], qv = x[c1][m][0] * erj;
+            x[c0][m][0] = csj * pv - snj * qv; x[c1][m][0] = snj * pv + csj * qv;
           }
         }
-        norm[c0] = alpha - t * gabs; norm[c1] = beta + t * gabs; ++applied;
+        norm[c0] -= shj; norm[c1] += shj; ++applied;
       }
     }
   }
@@ -182,7 +215,7 @@ __global__ __launch_bounds__(T_THREADS) void jacobi_block_round_kernel(int32_t N
   for (int c = 0; c < NC; ++c) {
     #pragma unroll
     for (int m = 0; m < ROWS; ++m) {
-      const int k = threadIdx.x + m * T_THREADS;
+      const int k = threadIdx.x + m * THREADS;
       if (live[c] && k < N) {
         #pragma unroll
         for (int w = 0; w < W; ++w) { B[((int64_t)col[c] * N + k) * W + w] = x[c][m][w]; }
@@ -266,11 +299,11 @@ extern "C" int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t
 }
 
 /* one sweep = every pair of the r columns of B (N x r, FP64, complex interleaved) once; rotations counts the rotations applied */
-template <bool CPLX, int ROWS, int BC>
+template <bool CPLX, int ROWS, int BC, int THREADS = T_THREADS>
 static int blocked_sweep(hipStream_t stream, int32_t N, int32_t r, double* B, double tol, int32_t* rotations) {
   const int blocks = (r + BC - 1) / BC, nb = (blocks + 1) & ~1;
-  jacobi_block_round_kernel<CPLX, ROWS, BC, true><<<nb / 2, T_THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations);
-  for (int round = 1; round < nb - 1; ++round) { jacobi_block_round_kernel<CPLX, ROWS, BC, false><<<nb / 2, T_THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations); }
+  jacobi_block_round_kernel<CPLX, ROWS, BC, true, THREADS><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations);
+  for (int round = 1; round < nb - 1; ++round) { jacobi_block_round_kernel<CPLX, ROWS, BC, false, THREADS><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations); }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
