@@ -113,3 +113,39 @@ def test_repeated_integer_block(env, name, at, M, N, eps, alg, bound, m0):
     assert np.array_equal(got_re, want_re), name
     if comps == 2:
         assert np.array_equal(got_im, want_im), name
+
+
+@pytest.mark.parametrize("at,M,N,K,eps", [(F64, 16384, 2048, 1024, 1e-12), (F64C, 8192, 1024, 512, 1e-12)], ids=["real", "complex"])
+def test_fit_at_full_width(env, at, M, N, K, eps):
+    """hyacinTsvdFit with the column count of the benchmark target (the Cholesky and Jacobi kernels then run on every
+    compute unit, with many workgroups exchanging data): singular values against sqrt(eigvalsh(A^H A)) computed by
+    torch in FP64, an orthonormal basis, and the same bits on a second run (every reduction order is fixed)."""
+    ha, h, torch = env
+    L = ha.lib()
+    g = torch.Generator(device="cuda")
+    g.manual_seed(97)
+    cplx = at & 1
+    scale = torch.pow(10.0, -torch.arange(N, device="cuda", dtype=torch.float64) / (N / 8.0))
+    A = (torch.randn((N, M, 2 if cplx else 1), generator=g, device="cuda", dtype=torch.float64) * scale[:, None, None]).contiguous()
+    outs = []
+    for rep in range(2):
+        S = torch.zeros(K, dtype=torch.float64, device="cuda")
+        V = torch.zeros(N * K * (2 if cplx else 1), dtype=torch.float64, device="cuda")
+        rank = L.hyacinTsvdFit(C.byref(h), eps, b"N", M, N, K, C.c_void_p(A.data_ptr()), M, C.c_void_p(S.data_ptr()), C.c_void_p(V.data_ptr()), N, 0, at)
+        torch.cuda.synchronize()
+        outs.append((rank, S, V))
+    rank, S, V = outs[0]
+    assert rank == K
+    Am = torch.view_as_complex(A).reshape(N, M) if cplx else A.reshape(N, M)       # row j = column j of A
+    G = Am.conj() @ Am.T                                                            # G[y, x] = sum_k conj(a_ky) a_kx
+    ev = torch.linalg.eigvalsh(G).flip(0).clamp_min(0).sqrt()
+    rel = ((S - ev[:K]).abs() / ev[:K]).max().item()
+    assert rel <= 1e-9, rel
+    Vm = (torch.view_as_complex(V.reshape(K, N, 2)) if cplx else V.reshape(K, N))   # row i = basis vector i
+    eye = torch.eye(K, device="cuda", dtype=Vm.dtype)
+    assert (Vm.conj() @ Vm.T - eye).abs().max().item() <= 1e-12
+    # the basis spans the dominant right singular subspace: the residual of A outside it is the tail of the spectrum
+    resid2 = (Am.abs() ** 2).sum().item() - ((Vm @ Am).abs() ** 2).sum().item()   # row i of Vm @ Am = (A v_i)^T
+    tail2 = (ev[K:] ** 2).sum().item()
+    assert abs(resid2 - tail2) <= 1e-6 * tail2 + 1e-12 * (ev ** 2).sum().item()
+    assert outs[1][0] == rank and torch.equal(outs[1][1], S) and torch.equal(outs[1][2], V)
