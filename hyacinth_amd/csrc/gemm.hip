@@ -8,7 +8,8 @@
  * copy; here: the interleaved operands are multiplied directly with FP32
  * accumulation, which is at least as accurate as the reference's FP16
  * accumulation).  FP64 types accumulate in FP64, FP32 / FP16 types in FP32.
- * LDS-tiled 64 x 64 x 16, 256 threads, a 4 x 4 register tile per thread.
+ * General kernel: LDS-tiled 64 x 64 x 16, 256 threads, a 4 x 4 register tile per thread (vector ALU).  The FP16 products
+ * C = op(A) B, the shape of matmul_cf16_{cn,tn,nn}, run on the matrix cores (second kernel below).
  */
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
@@ -89,6 +90,165 @@ template <typename S, bool CPLX> int run(hipStream_t stream, char opA, char opB,
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
+/* ------------------------------------------------------------------ FP16 products on the matrix cores
+ * C = op(A) B for real and complex FP16 (interleaved), FP32 accumulation, `v_mfma_f32_32x32x16_f16`.
+ *
+ * Complex as a real product of twice the depth: with k' = 2 k + s, B seen as a real (2 K) x N matrix is exactly its
+ * interleaved storage (B'[2k] = Br, B'[2k+1] = Bi), and op(A) expands to A're[m][2k] = Ar, [2k+1] = -Ai for the real part
+ * of C and A'im[m][2k] = Ai, [2k+1] = Ar for the imaginary part.  Both expansions are made in registers from the same
+ * 16 bytes (four complex numbers) a lane reads from LDS: a sign flip of the upper halves, and a 16-bit rotation of every
+ * word (the conjugate for op 'C' moves the sign flip).  No planar copy of either operand is made (the reference builds
+ * [Ar; -+Ai] and [-Bi; Br; Bi] in memory, src/matmul_fp16_complex.cu:4-14).
+ *
+ * Workgroup = 4 wavefronts (2 x 2), tile 128 rows of op(A) x 128 columns of B, wavefront 64 x 64 = 2 x 2 MFMA blocks (x 2
+ * accumulator sets when complex).  The contraction advances in slabs of 128 bytes per row (32 complex or 64 real
+ * numbers = four MFMA steps), double-buffered in LDS, next slab prefetched into registers during the MFMAs.  LDS rows are
+ * 128 bytes with XOR-swizzled 16-byte slots, so the fragment reads are bank-conflict-free.  The MFMA's row operand is B
+ * and its column operand op(A): a lane then owns one row m of C and stores run along the contiguous index.
+ * Needs 16-byte aligned operands and leading dimensions; other calls take the vector-ALU kernel above. */
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float16_t __attribute__((ext_vector_type(16)));
+constexpr int HT = 128, HROW = 128, HTILE = HT * HROW;
+
+__device__ __forceinline__ int h_swz(int row) { return ((row ^ (row >> 3)) & 1) | (row & 6); }
+
+/* 16 bytes of tile row `q`, piece `p`, from a matrix whose contraction index runs along memory (B, or A under op 'T' / 'C') */
+template <int E>
+__device__ __forceinline__ uint4 load_piece_contiguous(const char* X, int64_t ldx, int64_t q, int64_t Q, int64_t k, int64_t K) {
+  constexpr int PE = 16 / E; uint4 v = make_uint4(0u, 0u, 0u, 0u);
+  if (q >= Q || k >= K) { return v; }
+  const char* src = X + (k + q * ldx) * E;
+  if (k + PE <= K) { return *reinterpret_cast<const uint4*>(src); }
+  uint16_t h[8] = { 0, 0, 0, 0, 0, 0, 0, 0 };
+  for (int i = 0; i < (int)(K - k) * (E / 2); ++i) { h[i] = reinterpret_cast<const uint16_t*>(src)[i]; }
+  v.x = h[0] | ((uint32_t)h[1] << 16); v.y = h[2] | ((uint32_t)h[3] << 16); v.z = h[4] | ((uint32_t)h[5] << 16); v.w = h[6] | ((uint32_t)h[7] << 16);
+  return v;
+}
+/* the same piece of op(A) = A (rows run along memory): PE strided elements */
+template <int E>
+__device__ __forceinline__ uint4 load_piece_strided(const char* X, int64_t ldx, int64_t q, int64_t Q, int64_t k, int64_t K) {
+  constexpr int PE = 16 / E; uint32_t w[4] = { 0u, 0u, 0u, 0u };
+  if (q < Q) {
+    #pragma unroll
+    for (int i = 0; i < PE; ++i) {
+      if (k + i < K) {
+        const char* src = X + (q + (k + i) * ldx) * E;
+        if constexpr (E == 4) { w[i] = *reinterpret_cast<const uint32_t*>(src); } else { w[i >> 1] |= (uint32_t)*reinterpret_cast<const uint16_t*>(src) << (16 * (i & 1)); }
+      }
+    }
+  }
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+template <bool CPLX, int OPA>   /* OPA: 0 'N', 1 'T', 2 'C' */
+__global__ __launch_bounds__(256) void gemm_f16_mfma_kernel(int32_t M, int32_t N, int32_t K, const char* __restrict__ A, int64_t lda, const char* __restrict__ B, int64_t ldb, char* __restrict__ C, int64_t ldc) {
+  constexpr int E = CPLX ? 4 : 2, PE = 16 / E, KS = HROW / E;   /* bytes per element, elements per 16-byte piece, elements per slab */
+  __shared__ __attribute__((aligned(16))) char lds[2][2][HTILE];  /* [buffer][A | B][row * 128 + slot * 16] */
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave & 1, wn = wave >> 1;
+  const int64_t m0 = (int64_t)blockIdx.x * HT, n0 = (int64_t)blockIdx.y * HT;
+  uint4 ra[4], rb[4];
+  auto fetch = [&](int64_t k0) {
+    #pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      if constexpr (OPA == 0) { const int row = tid & 127, p = (tid >> 7) + 2 * r; ra[r] = load_piece_strided<E>(A, lda, m0 + row, M, k0 + p * PE, K); }
+      else { const int row = (tid >> 3) + 32 * r, p = tid & 7; ra[r] = load_piece_contiguous<E>(A, lda, m0 + row, M, k0 + p * PE, K); }
+      { const int row = (tid >> 3) + 32 * r, p = tid & 7; rb[r] = load_piece_contiguous<E>(B, ldb, n0 + row, N, k0 + p * PE, K); }
+    }
+  };
+  auto park = [&](int buf) {
+    #pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      { const int row = OPA == 0 ? (tid & 127) : (tid >> 3) + 32 * r, p = OPA == 0 ? (tid >> 7) + 2 * r : (tid & 7);
+        *reinterpret_cast<uint4*>(&lds[buf][0][row * HROW + ((p ^ h_swz(row)) << 4)]) = ra[r]; }
+      { const int row = (tid >> 3) + 32 * r, p = tid & 7; *reinterpret_cast<uint4*>(&lds[buf][1][row * HROW + ((p ^ h_swz(row)) << 4)]) = rb[r]; }
+    }
+  };
+  constexpr int SETS = CPLX ? 2 : 1;
+  float16_t acc[SETS][2][2];   /* [re | im][block of n][block of m] */
+  #pragma unroll
+  for (int s = 0; s < SETS; ++s) {
+    #pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      #pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        #pragma unroll
+        for (int e = 0; e < 16; ++e) { acc[s][i][j][e] = 0.f; }
+      }
+    }
+  }
+  const int slabs = (K + KS - 1) / KS;
+  const int rowM = (wm * 64 + (lane & 31)) * HROW, rowN = (wn * 64 + (lane & 31)) * HROW, sw = h_swz(lane & 31), hi = lane >> 5;
+  if (slabs > 0) { fetch(0); park(0); }
+  __syncthreads();
+  for (int it = 0; it < slabs; ++it) {
+    const int buf = it & 1;
+    if (it + 1 < slabs) { fetch((int64_t)(it + 1) * KS); }
+    #pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int slot = ((2 * s + hi) ^ sw) << 4;
+      uint4 fm[2], fn[2];
+      #pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        fm[b] = *reinterpret_cast<const uint4*>(&lds[buf][0][rowM + b * 32 * HROW + slot]);
+        fn[b] = *reinterpret_cast<const uint4*>(&lds[buf][1][rowN + b * 32 * HROW + slot]);
+      }
+      #pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        if constexpr (CPLX) {
+          /* word = Ar | Ai << 16.  Real part of C: (Ar, -Ai), conjugated A: (Ar, Ai).  Imaginary part: (Ai, Ar), conjugated: (-Ai, Ar). */
+          const uint32_t w[4] = { fm[j].x, fm[j].y, fm[j].z, fm[j].w }; uint32_t wr[4], wi[4];
+          #pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            wr[q] = OPA == 2 ? w[q] : (w[q] ^ 0x80000000u);
+            const uint32_t rot = __builtin_amdgcn_alignbit(w[q], w[q], 16); wi[q] = OPA == 2 ? (rot ^ 0x00008000u) : rot;
+          }
+          const uint4 ure = make_uint4(wr[0], wr[1], wr[2], wr[3]), uim = make_uint4(wi[0], wi[1], wi[2], wi[3]);
+          #pragma unroll
+          for (int i = 0; i < 2; ++i) {
+            acc[0][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, fn[i]), __builtin_bit_cast(half8_t, ure), acc[0][i][j], 0, 0, 0);
+            acc[1][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, fn[i]), __builtin_bit_cast(half8_t, uim), acc[1][i][j], 0, 0, 0);
+          }
+        } else {
+          #pragma unroll
+          for (int i = 0; i < 2; ++i) { acc[0][i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, fn[i]), __builtin_bit_cast(half8_t, fm[j]), acc[0][i][j], 0, 0, 0); }
+        }
+      }
+    }
+    if (it + 1 < slabs) { park(buf ^ 1); }   /* the other buffer was last read before the previous barrier */
+    __syncthreads();
+  }
+  /* lane: row m of the block; register e: column n = 8 (e / 4) + 4 (lane / 32) + e % 4 of the block */
+  #pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    #pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int64_t m = m0 + wm * 64 + j * 32 + (lane & 31); if (m >= M) { continue; }
+      #pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int64_t n = n0 + wn * 64 + i * 32 + ((e >> 2) << 3) + (hi << 2) + (e & 3); if (n >= N) { continue; }
+        char* dst = C + (m + n * ldc) * E;
+        if constexpr (CPLX) { *reinterpret_cast<__half2*>(dst) = __floats2half2_rn(acc[0][i][j][e], acc[1][i][j][e]); }
+        else { *reinterpret_cast<__half*>(dst) = __float2half(acc[0][i][j][e]); }
+      }
+    }
+  }
+}
+
+template <bool CPLX> int run_f16_mfma(hipStream_t stream, char opA, int32_t M, int32_t N, int32_t K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C, int64_t ldc) {
+  dim3 grid((M + HT - 1) / HT, (N + HT - 1) / HT); const char* a = (const char*)A; const char* b = (const char*)B; char* c = (char*)C;
+  if (opA == 'N') { gemm_f16_mfma_kernel<CPLX, 0><<<grid, 256, 0, stream>>>(M, N, K, a, lda, b, ldb, c, ldc); }
+  else if (opA == 'T' || !CPLX) { gemm_f16_mfma_kernel<CPLX, 1><<<grid, 256, 0, stream>>>(M, N, K, a, lda, b, ldb, c, ldc); }
+  else { gemm_f16_mfma_kernel<CPLX, 2><<<grid, 256, 0, stream>>>(M, N, K, a, lda, b, ldb, c, ldc); }
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+/* the matrix-core kernel covers C = op(A) B (alpha 1, beta 0, B as stored) on 16-byte aligned operands */
+bool f16_mfma_applies(char opB, double alpha, double beta, int32_t type, const void* A, int64_t lda, const void* B, int64_t ldb, const void* C, int32_t N) {
+  if ((type != HYK_F16 && type != HYK_F16C) || opB != 'N' || alpha != 1.0 || beta != 0.0 || (N + HT - 1) / HT > 65535) { return false; }
+  const int64_t e = type == HYK_F16C ? 4 : 2;
+  return ((uintptr_t)A % 16 == 0) && ((uintptr_t)B % 16 == 0) && ((uintptr_t)C % e == 0) && (lda * e) % 16 == 0 && (ldb * e) % 16 == 0;
+}
+
 char norm_op(char c) { return (c == 't' || c == 'T') ? 'T' : ((c == 'c' || c == 'C') ? 'C' : 'N'); }
 
 }  // namespace
@@ -97,6 +257,9 @@ extern "C" int hykGemm(hipStream_t stream, char opA, char opB, int32_t M, int32_
   if (M <= 0 || N <= 0) { return 0; }
   if (K < 0 || (N + GT - 1) / GT > 65535) { return -1; }
   opA = norm_op(opA); opB = norm_op(opB);
+  if (K > 0 && f16_mfma_applies(opB, alpha, beta, type, A, lda, B, ldb, C, N)) {
+    return type == HYK_F16C ? run_f16_mfma<true>(stream, opA, M, N, K, A, lda, B, ldb, C, ldc) : run_f16_mfma<false>(stream, opA, M, N, K, A, lda, B, ldb, C, ldc);
+  }
   switch (type) {
     case HYK_F64: return run<double, false>(stream, opA, opB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc);
     case HYK_F32: return run<float, false>(stream, opA, opB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc);

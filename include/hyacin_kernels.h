@@ -95,13 +95,16 @@ int hykMatcopy(hipStream_t stream, char mode, int64_t M, int64_t N, int32_t srcT
 /* *out += sum of squares.  Replaces cublasDnrm2_64, src/lra.cpp:170,204. */
 int hykSumSquares(hipStream_t stream, int64_t M, int64_t N, const double* A, int64_t lda, double* out);
 
-/* Complex FP16 matrix product C = op(A) B on interleaved half pairs, FP32 accumulation (LDS-tiled vector-ALU kernel).
+/* Complex FP16 matrix product C = op(A) B on interleaved half pairs, FP32 accumulation, on the matrix cores
+ * (v_mfma_f32_32x32x16_f16; the complex product is a real one of twice the depth, expanded in registers) when the
+ * operands and leading dimensions are 16-byte aligned, else on the vector ALU.
  * Replaces internal::matmul_cf16_{cn,tn,nn}, src/matmul_fp16_complex.cu:21-89. opA: 'N', 'T' or 'C'. */
 int hykMatmulCf16(hipStream_t stream, char opA, int32_t M, int32_t N, int32_t K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C, int64_t ldc);
 
 /* Real / complex matrix product C = op(A) B in the storage type (FP64, FP32, FP16 and complex FP64 / FP32), used by the
  * column-segmented fit and the residual check.  Replaces the cuBLAS gemm calls of src/lra.cpp:86-105,202-203.
- * alpha/beta are real scalars. opA 'N' | 'T' | 'C', opB 'N' | 'T' | 'C'. */
+ * alpha/beta are real scalars. opA 'N' | 'T' | 'C', opB 'N' | 'T' | 'C'.  FP16 and complex FP16 calls of the form
+ * C = op(A) B (alpha 1, beta 0, opB 'N') run on the matrix cores like hykMatmulCf16. */
 int hykGemm(hipStream_t stream, char opA, char opB, int32_t M, int32_t N, int32_t K, double alpha, int32_t type, const void* A, int64_t lda, const void* B, int64_t ldb, double beta, void* C, int64_t ldc);
 
 /* V (N x r, FP64 or complex FP64, interleaved) is overwritten by an orthonormal basis of its column space (one-sided

@@ -54,7 +54,8 @@ def test_slice_range_and_gram_range(gl, oracle):
         v = oracle.quantize_scale_batch(A, 5, 128, 128, pl["u"])
         Cq = oracle.herk_batch(A, 5, 128, 128, pl["u"], v, pl["lP"])
         out = zeros(4)
-        assert gl.L.hykGramRange(stream(), 40, pl["lP"], ptr(dev(Cq)), ptr(dev(v)), ptr(out)) == 0
+        dC, dv = dev(Cq), dev(v)                  # named: a temporary would hand its memory back before the kernel has run
+        assert gl.L.hykGramRange(stream(), 40, pl["lP"], ptr(dC), ptr(dv), ptr(out)) == 0
         sync()
         assert host(out, np.int32)[0] == oracle.dequantize_init(40, pl["lP"], Cq, v, 0)[2]
 
@@ -171,7 +172,8 @@ def test_dequantize(gl, oracle, cplx):
         for gtype in (oracle.F32 + cplx, oracle.F64 + cplx, oracle.DD + cplx):
             want = oracle.dequantize(N, pl["lP"], Cq, vexp, gtype)
             G = zeros(want.nbytes)
-            assert gl.L.hykDequantize(stream(), N, pl["lP"], ptr(dev(Cq)), ptr(dev(vexp)), gtype, ptr(G), N) == 0
+            dC, dv = dev(Cq), dev(vexp)
+            assert gl.L.hykDequantize(stream(), N, pl["lP"], ptr(dC), ptr(dv), gtype, ptr(G), N) == 0
             sync()
             got = host(G, want.dtype, want.shape)
             if gtype in (oracle.DD, oracle.DDC):
@@ -261,7 +263,8 @@ def test_potrfp_kernel(gl, oracle, gbase, cplx, N, r, K, eps64, epsdd, floor, un
     jp = zeros(N * 4)
     rk = zeros(4)
     ws = zeros(gl.L.hykPotrfpWorkspaceBytes(N, gtype))
-    assert gl.L.hykPotrfp(stream(), units, eps, K, N, gtype, ptr(dev(raw)), N, ptr(Rt), ldr, ptr(jp), ptr(ws), ptr(rk)) == 0
+    dG = dev(raw)
+    assert gl.L.hykPotrfp(stream(), units, eps, K, N, gtype, ptr(dG), N, ptr(Rt), ldr, ptr(jp), ptr(ws), ptr(rk)) == 0
     sync()
     rank = int(host(rk, np.int32)[0])
     piv = host(jp, np.int32)
@@ -285,3 +288,40 @@ def test_potrfp_kernel(gl, oracle, gbase, cplx, N, r, K, eps64, epsdd, floor, un
     # entries below the diagonal (in pivot order) stay zero
     for t in range(1, rank):
         assert not got[p[:t], t, :].any()
+
+
+@pytest.mark.parametrize("cplx", [0, 1])
+@pytest.mark.parametrize("opA", ["N", "T", "C"])
+@pytest.mark.parametrize("M,N,K,pad", [(300, 70, 45, 0), (128, 128, 64, 0), (1000, 260, 333, 8), (257, 129, 1, 0), (96, 40, 200, 3)])
+def test_f16_products(gl, cplx, opA, M, N, K, pad):
+    """hykMatmulCf16 / hykGemm on FP16 operands (src/matmul_fp16_complex.cu:21-89, the GemmEx calls of src/lra.cpp:86-105):
+    C = op(A) B against numpy in FP32 on the same half-rounded inputs.  Ragged tiles, K tails inside a 16-byte piece, padded
+    leading dimensions; pad = 3 makes the leading dimensions unaligned, which takes the vector-ALU kernel."""
+    from gpu_util import dev, zeros, ptr, stream, sync, host
+    rng = np.random.default_rng(77 + cplx)
+    comps = 2 if cplx else 1
+    rowsA, colsA = (M, K) if opA == "N" else (K, M)
+    lda, ldb, ldc = rowsA + (8 - rowsA % 8) % 8 + pad, K + (8 - K % 8) % 8 + pad, M + pad
+    def rand(rows, cols, ld):
+        buf = np.zeros((cols, ld, comps), np.float16)
+        buf[:, :rows, :] = rng.standard_normal((cols, rows, comps)).astype(np.float16)
+        v = buf[:, :rows, :].astype(np.float32)
+        m = (v[..., 0] + 1j * v[..., 1]).T if cplx else v[..., 0].T        # rows x cols
+        return buf, m
+    bufA, mA = rand(rowsA, colsA, lda)
+    bufB, mB = rand(K, N, ldb)
+    opm = mA if opA == "N" else (mA.T if opA == "T" else mA.conj().T)
+    want = opm.astype(np.complex64 if cplx else np.float32) @ mB
+    Cd = zeros(N * ldc * comps * 2)
+    dA, dB = dev(bufA), dev(bufB)
+    if cplx:
+        rc = gl.L.hykMatmulCf16(stream(), opA.encode(), M, N, K, ptr(dA), lda, ptr(dB), ldb, ptr(Cd), ldc)
+    else:
+        rc = gl.L.hykGemm(stream(), opA.encode(), b"N", M, N, K, C.c_double(1.0), 4, ptr(dA), C.c_int64(lda), ptr(dB), C.c_int64(ldb), C.c_double(0.0), ptr(Cd), C.c_int64(ldc))
+    assert rc == 0
+    sync()
+    got = host(Cd, np.float16, (N, ldc, comps))[:, :M, :].astype(np.float32)
+    got = (got[..., 0] + 1j * got[..., 1]).T if cplx else got[..., 0].T
+    scale = np.sqrt(np.mean(np.abs(want) ** 2))
+    assert np.all(np.abs(got - want) <= 2.0**-10 * np.abs(want) + 2.0**-12 * scale + 1e-6)
+    assert not host(Cd, np.float16, (N, ldc, comps))[:, M:, :].any()       # nothing written into the padding
