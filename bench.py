@@ -20,6 +20,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 INT8_PEAK_TOPS = 5000.0   # MI355X dense INT8 MFMA peak, 5.0 POP/s
+HBM_PEAK_GBS = 8000.0     # MI355X HBM3E peak, 8 TB/s
 
 # HBM bytes per launch of the contraction kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script
 # (profiles/gram_ring_kernel_target_hbm_traffic.md), each scaled by what the counter reads for copy_kernel's known 1 GiB.
@@ -94,6 +95,7 @@ def main():
     ap.add_argument("--workload", default="target", choices=sorted(WORKLOADS))
     ap.add_argument("--no-fit", action="store_true", help="skip the end-to-end hyacinTsvdFit timing")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-stages", action="store_true", help="skip the separate timing of the HBM-bound stages (exponents, quantize, dequantize)")
     ap.add_argument("--no-ceiling", action="store_true", help="skip the register-only MFMA ceiling measurement")
     ap.add_argument("--cpu-rows", type=int, default=65536, help="rows of the workload the CPU baseline is timed on (about 15 s of host work)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -150,7 +152,7 @@ def main():
 
     # the plan the library followed (same planner, host side)
     from oracle import ho
-    plan_alg, order, _ = ho.gram_algorithm(alg.decode(), M if batches <= 1 else M, u + cplx, cplx, h.TCGemmTargetK, h.StrideBatchPerfPenalty)
+    plan_alg, order, plan_rows = ho.gram_algorithm(alg.decode(), M if batches <= 1 else M, u + cplx, cplx, h.TCGemmTargetK, h.StrideBatchPerfPenalty)
     ops = algorithmic_ops(plan_alg, order, cplx, M, N)
     feff = M * N * (N + 1) * (4 if cplx else 1)
     launches_per_step = max(1, kn.value // a.steps)
@@ -163,6 +165,45 @@ def main():
         if L.hykMfmaCeiling(stream, h.DeviceSMs, 20000, 1, C.byref(tops), C.byref(ghz)) == 0:
             ceiling = {"value": tops.value, "unit": "TFLOP/s", "clock_ghz": ghz.value,
                        "what": "register-only v_mfma_i32_32x32x32_i8 loop, random int8 operands, one workgroup of 4 waves per CU"}
+
+    # HBM-bound stages on their own (HIP events on the launch stream, outside the timed region): algorithmic bytes / time
+    def timed_ms(fn, reps=3):
+        best = None
+        for _ in range(reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(); fn(); e1.record(); torch.cuda.synchronize()
+            t = e0.elapsed_time(e1)
+            best = t if best is None or t < best else best
+        return best
+    eb = {0: 8, 1: 16, 2: 4, 3: 8, 4: 2, 5: 4}[at]
+    stages = {}
+    if not a.no_stages:
+        t = timed_ms(lambda: L.hyacinXquantizeScaleBatch(C.byref(h), batches, seg, lastM, N, at, pA, lda, u, pV))
+        stages["column_exponents"] = {"ms": t, "bytes": M * N * eb, "GB/s": M * N * eb / t / 1e6, "frac_of_hbm_peak": M * N * eb / t / 1e6 / HBM_PEAK_GBS}
+        rows = min(M, plan_rows) if plan_alg == "C" and plan_rows > 0 else M   # the rows the library quantizes per call (one residue chunk, or all)
+        if plan_alg == "C":
+            npan = 2 * min(order, 20) + 3 * max(order - 20, 0) if cplx else order
+        else:
+            npan = 3 * order if cplx else order
+        ldb = (rows + 127) // 128 * 128
+        panels = torch.empty(npan * N * ldb, dtype=torch.int8, device="cuda")
+        pB = C.c_void_p(panels.data_ptr())
+        if plan_alg == "C":
+            quant = lambda: L.hykQuantizeCrt(stream, rows, N, order, at, pA, lda, pV, pB, ldb, u + cplx)
+        else:
+            quant = lambda: L.hykQuantizeLimbs(stream, rows, N, order, at, pA, lda, pV, pB, ldb)
+        assert quant() == 0
+        t = timed_ms(quant)
+        qbytes = rows * N * eb + npan * rows * N
+        stages["quantize"] = {"ms": t, "rows": rows, "panels": npan, "bytes": qbytes, "GB/s": qbytes / t / 1e6, "frac_of_hbm_peak": qbytes / t / 1e6 / HBM_PEAK_GBS}
+        del panels
+        gt, gb = C.c_int(), C.c_int32()
+        L.hyacinXdequantizeInit(C.byref(h), N, lP, pC, pV, at, C.byref(gt), C.byref(gb))
+        G = torch.empty(N * N * gb.value, dtype=torch.uint8, device="cuda")
+        t = timed_ms(lambda: L.hyacinXdequantize(C.byref(h), N, lP, pC, pV, gt.value, C.c_void_p(G.data_ptr()), N))
+        dbytes = cP * lP * stride * 8 + N * N * gb.value
+        stages["dequantize"] = {"ms": t, "bytes": dbytes, "GB/s": dbytes / t / 1e6, "frac_of_hbm_peak": dbytes / t / 1e6 / HBM_PEAK_GBS}
+        del G
 
     fit_ms = None
     if not a.no_fit:
@@ -186,6 +227,7 @@ def main():
                    "quant_bits": u, "gram_limbs": lP, "row_slices": batches},
         "pct_int8_mfma_peak": 100.0 * achieved / INT8_PEAK_TOPS,
         "tsvd_fit_ms": fit_ms,
+        "hbm_stages": stages,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s", "frac": achieved / INT8_PEAK_TOPS,
                      "traffic": MEASURED_TRAFFIC.get((a.workload, max(a.slab, 0))),
                      "kernel": "gram_ring_kernel" if a.slab <= 0 else ("gram_dma_kernel" if a.slab == 2 else "gram_kernel<%d>" % a.slab), "ops": "int8 multiply-adds x2, upper triangle only", "launches_per_step": launches_per_step,
