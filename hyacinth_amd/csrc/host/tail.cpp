@@ -70,9 +70,13 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
     hyh::Scratch B(handle, (size_t)N * rank * 8 * (1 + Complex)), sigma(handle, sizeof(double) * (size_t)rank), counter(handle, 64);
     HYH_KERNEL(hykFactorToB(s, N, rank, f.type, f.Rt.p, f.ldr, B.as<double>()));
     const int32_t maxSweeps = sweeps > 0 ? 5 * sweeps : 30; int32_t used = 0;
+    /* A pair is rotated while its cosine exceeds the storage precision, but never below sqrt(N) FP64 roundings: that is
+     * what the dot product of two columns of length N carries as noise (the threshold of LAPACK's xGESVJ); rotating
+     * below it costs sweeps and leaves the orthogonality where it was. */
+    const double rotateAbove = std::max(machineEps, std::sqrt((double)N) * 2.220446049250313e-16);
     for (int32_t sw = 0; sw < maxSweeps && rank > 1; ++sw) {
       HYH_KERNEL(hykGramWorkspaceClear(s, counter.p, 64));
-      HYH_KERNEL(hykJacobiSweep(s, Complex, N, rank, B.as<double>(), machineEps, counter.as<int32_t>())); ++used;
+      HYH_KERNEL(hykJacobiSweep(s, Complex, N, rank, B.as<double>(), rotateAbove, counter.as<int32_t>())); ++used;
       int32_t rotations = 0; HYH_CHECK(hipMemcpyAsync(&rotations, counter.p, sizeof(int32_t), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
       if (rotations == 0) { break; }
     }

@@ -394,7 +394,7 @@ extern "C" int hykOrthonormalize(hipStream_t stream, int32_t Complex, int32_t N,
   int32_t* counter = reinterpret_cast<int32_t*>(work); double* sigma = work + 8;
   for (int sweep = 0; sweep < 40 && r > 1; ++sweep) {
     if (hipMemsetAsync(counter, 0, 64, stream) != hipSuccess) { return -3; }
-    if (hykJacobiSweep(stream, Complex, N, r, V, 2.220446049250313e-16, counter) != 0) { return -3; }
+    if (hykJacobiSweep(stream, Complex, N, r, V, 2.220446049250313e-16 * sqrt((double)N), counter) != 0) { return -3; }
     int32_t rotations = 0;
     if (hipMemcpyAsync(&rotations, counter, sizeof(int32_t), hipMemcpyDeviceToHost, stream) != hipSuccess || hipStreamSynchronize(stream) != hipSuccess) { return -3; }
     if (rotations == 0) { break; }
