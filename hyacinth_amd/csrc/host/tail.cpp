@@ -77,8 +77,13 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
     for (int32_t sw = 0; sw < maxSweeps && rank > 1; ++sw) {
       HYH_KERNEL(hykGramWorkspaceClear(s, counter.p, 64));
       HYH_KERNEL(hykJacobiSweep(s, Complex, N, rank, B.as<double>(), rotateAbove, counter.as<int32_t>())); ++used;
-      int32_t rotations = 0; HYH_CHECK(hipMemcpyAsync(&rotations, counter.p, sizeof(int32_t), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
-      if (rotations == 0) { break; }
+      struct { int32_t rotations, pad; double cosine2; } seen = { 0, 0, 0. };
+      HYH_CHECK(hipMemcpyAsync(&seen, counter.p, sizeof(seen), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
+      /* Done when nothing was rotated, or when every cosine the sweep met was within 8 thresholds: rotating such pairs
+       * moves the other cosines by products of two of them, so the sweep has left all of them at the threshold's level
+       * and a further sweep would only confirm it. */
+      if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: %d rotations, largest cosine %.2le\n", used, seen.rotations, std::sqrt(seen.cosine2)); }
+      if (seen.rotations == 0 || seen.cosine2 <= 64. * rotateAbove * rotateAbove) { break; }
     }
     HYH_KERNEL(hykColumnNorms(s, Complex, N, rank, B.as<double>(), sigma.as<double>()));
     std::vector<double> sig((size_t)rank); HYH_CHECK(hipMemcpyAsync(sig.data(), sigma.p, sizeof(double) * (size_t)rank, hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));

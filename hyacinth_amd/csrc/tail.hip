@@ -43,6 +43,16 @@ __global__ void factor_to_b_kernel(int32_t N, int32_t rank, const double* __rest
   if constexpr (CPLX) { B[2 * ((int64_t)c + (int64_t)k * N)] = src[0]; B[2 * ((int64_t)c + (int64_t)k * N) + 1] = -src[WR]; } else { B[(int64_t)c + (int64_t)k * N] = src[0]; }
 }
 
+/* The sweep kernels report the largest squared cosine g^2 / (alpha beta) they met, rotated or not, as the bit pattern of a
+ * double at rotations + 2 (non-negative doubles order like their bit patterns, so an integer maximum does it). */
+__device__ __forceinline__ void report_cosine(int32_t* rotations, double cos2) {
+  if (cos2 > 0.) { atomicMax(reinterpret_cast<unsigned long long*>(rotations + 2), (unsigned long long)__double_as_longlong(cos2)); }
+}
+__device__ __forceinline__ double squared_cosine(double g2, double alpha, double beta) {
+  const double ab = alpha * beta;
+  return ab > 0. ? g2 / ab : (g2 > 0. ? 1. : 0.);   /* a column whose carried norm has collapsed counts as not converged */
+}
+
 template <bool CPLX>
 __global__ __launch_bounds__(T_THREADS) void jacobi_round_kernel(int32_t N, int32_t n, int32_t r, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations) {
   __shared__ double scratch[T_THREADS / 64];
@@ -61,6 +71,7 @@ __global__ __launch_bounds__(T_THREADS) void jacobi_round_kernel(int32_t N, int3
   }
   alpha = block_sum(alpha, scratch); beta = block_sum(beta, scratch); gre = block_sum(gre, scratch); if constexpr (CPLX) { gim = block_sum(gim, scratch); }
   const double g2 = gre * gre + gim * gim;
+  if (threadIdx.x == 0) { report_cosine(rotations, squared_cosine(g2, alpha, beta)); }
   if (!(g2 > tol * tol * alpha * beta) || !(g2 > 0.)) { return; }
   const double gabs = sqrt(g2), zeta = (beta - alpha) / (2. * gabs);
   const double t = (zeta >= 0. ? 1. : -1.) / (fabs(zeta) + sqrt(1. + zeta * zeta)), cs = 1. / sqrt(1. + t * t), sn = cs * t;
@@ -149,7 +160,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_block_round_kernel(int32_t N, 
     norm[c] = s;
   }
   block_sum_many<NC, THREADS, HALF>(norm, red, 0);
-  int applied = 0;
+  int applied = 0; double worst = 0.;
   /* FULL: first round of a sweep, all pairs of the 2 BC columns (round-robin); otherwise the BC x BC cross pairs */
   constexpr int STEPS = FULL ? NC - 1 : BC;
   #pragma unroll
@@ -181,6 +192,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_block_round_kernel(int32_t N, 
       if (lane == j) { alpha = norm[c0]; beta = norm[c1]; pairLive = live[c0] && live[c1]; }
     }
     const double g2 = gre * gre + gim * gim;
+    if (pairLive) { worst = fmax(worst, squared_cosine(g2, alpha, beta)); }
     const bool rotate = pairLive && g2 > tol * tol * alpha * beta && g2 > 0.;
     double cs = 1., sn = 0., er = 1., ei = 0., shift = 0.;
     if (rotate) {
@@ -210,6 +222,9 @@ __global__ __launch_bounds__(THREADS) void jacobi_block_round_kernel(int32_t N, 
       }
     }
   }
+  #pragma unroll
+  for (int off = BC / 2; off > 0; off >>= 1) { worst = fmax(worst, __shfl_xor(worst, off, 64)); }   /* lanes 0 .. BC-1 hold the pairs */
+  if (threadIdx.x == 0) { report_cosine(rotations, worst); }
   if (applied == 0) { return; }                  /* nothing rotated (same decision in every thread): the columns in memory are current */
   #pragma unroll
   for (int c = 0; c < NC; ++c) {
@@ -395,9 +410,9 @@ extern "C" int hykOrthonormalize(hipStream_t stream, int32_t Complex, int32_t N,
   for (int sweep = 0; sweep < 40 && r > 1; ++sweep) {
     if (hipMemsetAsync(counter, 0, 64, stream) != hipSuccess) { return -3; }
     if (hykJacobiSweep(stream, Complex, N, r, V, 2.220446049250313e-16 * sqrt((double)N), counter) != 0) { return -3; }
-    int32_t rotations = 0;
-    if (hipMemcpyAsync(&rotations, counter, sizeof(int32_t), hipMemcpyDeviceToHost, stream) != hipSuccess || hipStreamSynchronize(stream) != hipSuccess) { return -3; }
-    if (rotations == 0) { break; }
+    struct { int32_t rotations, pad; double cosine2; } seen = { 0, 0, 0. }; const double level = 8. * 2.220446049250313e-16 * sqrt((double)N);
+    if (hipMemcpyAsync(&seen, counter, sizeof(seen), hipMemcpyDeviceToHost, stream) != hipSuccess || hipStreamSynchronize(stream) != hipSuccess) { return -3; }
+    if (seen.rotations == 0 || seen.cosine2 <= level * level) { break; }
   }
   if (hykColumnNorms(stream, Complex, N, r, V, sigma) != 0) { return -3; }
   const int W = Complex ? 2 : 1; dim3 grid((N * W + T_THREADS - 1) / T_THREADS, r);

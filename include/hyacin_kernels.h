@@ -80,6 +80,9 @@ int hykPotrfp(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, i
 
 /* SVD tail.  Replaces the cuSOLVER gesvdj call and the copies around it, src/gram_evd.cu:110-137. */
 int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t Gtype, const void* Rt, int32_t ldr, double* B);
+/* One sweep of one-sided Jacobi over the r columns of B (N x r, FP64, complex interleaved): every pair whose cosine exceeds
+ * tol is rotated.  rotations: 16 bytes of device memory, zero before the call; afterwards rotations[0] = pairs rotated and
+ * the double at rotations + 2 = the largest squared cosine the sweep met (rotated or not). */
 int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations);
 int hykColumnNorms(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, const double* B, double* sigma);
 int hykBasisOut(hipStream_t stream, int32_t N, int32_t rank, int32_t Atype, const double* B, const double* sigma, const int32_t* order, void* X, int64_t ldx);
