@@ -116,7 +116,7 @@ extern "C" int32_t hyacinXGinterp(const hyacinHandle_t* handle, double eps, int3
   const int32_t rank = run_potrfp(handle, f, eps, K, N, jpiv);
   if (rank <= 0) { return rank; }
   if (rank >= N) { HYH_KERNEL(hykInterpOut(s, N, N, (int32_t)Atype, jpiv, nullptr, X, ldx)); return N; }
-  hyh::Scratch Rp(handle, (size_t)rank * N * 8 * (1 + Complex)), Tt(handle, (size_t)rank * (N - rank) * 8 * (1 + Complex));
+  hyh::Scratch Rp(handle, (size_t)rank * rank * 8 * (1 + Complex)), Tt(handle, (size_t)rank * (N - rank) * 8 * (1 + Complex));
   HYH_KERNEL(hykInterpSolve(s, N, rank, f.type, f.Rt.p, f.ldr, jpiv, Rp.as<double>(), Tt.as<double>()));
   HYH_KERNEL(hykInterpOut(s, N, rank, (int32_t)Atype, jpiv, Tt.as<double>(), X, ldx));
   if (handle->logger) { std::fprintf((FILE*)handle->logger, "TRSM-LEFT-%s [M=%d] [N=%d]\n", Complex ? "FP64-COMPLEX" : "FP64", rank, N - rank); }

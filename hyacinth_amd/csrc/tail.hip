@@ -270,36 +270,66 @@ __global__ void normalize_columns_kernel(int32_t N, int W, double* B, const doub
 
 template <typename T> __global__ void values_out_kernel(int32_t K, const double* __restrict__ S, T* __restrict__ out) { const int i = blockIdx.x * T_THREADS + threadIdx.x; if (i < K) { store_real<T>(&out[i], S[i]); } }
 
-/* Rp[k + x*K] = R[k, jpiv[x]-1] (high word), K x N upper trapezoid in pivot order */
+/* R in pivot order, high words: R11[k + x K] = R[k, jpiv[x] - 1] for x < K (upper triangle, zero below), and the right-hand
+ * sides T[k + (x - K) K] = R[k, jpiv[x] - 1] for x >= K */
 template <bool CPLX>
-__global__ void gather_factor_kernel(int32_t N, int32_t K, const double* __restrict__ Rt, int32_t ldr, int WE, int WR, const int32_t* __restrict__ jpiv, double* __restrict__ Rp) {
+__global__ void gather_factor_kernel(int32_t N, int32_t K, const double* __restrict__ Rt, int32_t ldr, int WE, int WR, const int32_t* __restrict__ jpiv, double* __restrict__ R11, double* __restrict__ T) {
   const int k = blockIdx.x * T_THREADS + threadIdx.x, x = blockIdx.y; if (k >= K) { return; }
   const double* src = &Rt[((int64_t)(jpiv[x] - 1) * ldr + k) * WE]; const bool low = k > x;
-  if constexpr (CPLX) { Rp[2 * ((int64_t)k + (int64_t)x * K)] = low ? 0. : src[0]; Rp[2 * ((int64_t)k + (int64_t)x * K) + 1] = low ? 0. : src[WR]; } else { Rp[(int64_t)k + (int64_t)x * K] = low ? 0. : src[0]; }
+  double* dst = x < K ? &R11[((int64_t)k + (int64_t)x * K) * (CPLX ? 2 : 1)] : &T[((int64_t)k + (int64_t)(x - K) * K) * (CPLX ? 2 : 1)];
+  dst[0] = low ? 0. : src[0]; if constexpr (CPLX) { dst[1] = low ? 0. : src[WR]; }
 }
 
-/* back substitution R11 T = R12, one thread per right-hand side; Tt[col + i*ncols] = T[i, col] */
+/* One block row of the blocked back substitution R11 T = R12: T[i0 .. i0+rows) <- R11[i0.., i0..]^-1 T[i0 .. i0+rows), the
+ * rows below already eliminated from it by a matrix product.  One thread per right-hand side keeps its `rows` entries in
+ * registers; the triangle sits in LDS (every thread reads the same entry: a broadcast). */
+constexpr int SOLVE_ROWS = 32;
 template <bool CPLX>
-__global__ void upper_solve_kernel(int32_t K, int32_t ncols, const double* __restrict__ Rp, double* __restrict__ Tt) {
+__global__ __launch_bounds__(T_THREADS) void block_solve_kernel(int32_t K, int32_t ncols, int32_t i0, int32_t rows, const double* __restrict__ R11, double* __restrict__ T) {
+  constexpr int W = CPLX ? 2 : 1;
+  __shared__ double tri[SOLVE_ROWS][SOLVE_ROWS][W];
+  for (int e = threadIdx.x; e < SOLVE_ROWS * SOLVE_ROWS; e += T_THREADS) {
+    const int i = e % SOLVE_ROWS, j = e / SOLVE_ROWS; const bool in = i < rows && j < rows;
+    #pragma unroll
+    for (int w = 0; w < W; ++w) { tri[i][j][w] = in ? R11[((int64_t)(i0 + i) + (int64_t)(i0 + j) * K) * W + w] : 0.; }
+  }
+  __syncthreads();
   const int col = blockIdx.x * T_THREADS + threadIdx.x; if (col >= ncols) { return; }
-  constexpr int W = CPLX ? 2 : 1; const double* rhs = &Rp[(int64_t)(K + col) * K * W];
-  for (int i = K - 1; i >= 0; --i) {
-    double sr = rhs[(int64_t)i * W], si = CPLX ? rhs[(int64_t)i * W + 1] : 0.;
-    for (int j = i + 1; j < K; ++j) {
-      const double* rij = &Rp[((int64_t)i + (int64_t)j * K) * W]; const double* xj = &Tt[((int64_t)col + (int64_t)j * ncols) * W];
-      if constexpr (CPLX) { sr -= rij[0] * xj[0] - rij[1] * xj[1]; si -= rij[0] * xj[1] + rij[1] * xj[0]; } else { sr -= rij[0] * xj[0]; }
+  double* t = &T[((int64_t)i0 + (int64_t)col * K) * W];
+  double x[SOLVE_ROWS][W];
+  #pragma unroll
+  for (int i = 0; i < SOLVE_ROWS; ++i) {
+    #pragma unroll
+    for (int w = 0; w < W; ++w) { x[i][w] = i < rows ? t[i * W + w] : 0.; }
+  }
+  #pragma unroll
+  for (int i = SOLVE_ROWS - 1; i >= 0; --i) {
+    if (i < rows) {
+      double sr = x[i][0], si = CPLX ? x[i][W - 1] : 0.;
+      #pragma unroll
+      for (int j = i + 1; j < SOLVE_ROWS; ++j) {
+        if constexpr (CPLX) { sr -= tri[i][j][0] * x[j][0] - tri[i][j][1] * x[j][1]; si -= tri[i][j][0] * x[j][1] + tri[i][j][1] * x[j][0]; }
+        else { sr -= tri[i][j][0] * x[j][0]; }
+      }
+      const double d = tri[i][i][0];   /* the diagonal of R is real */
+      x[i][0] = sr / d; if constexpr (CPLX) { x[i][1] = si / d; }
     }
-    const double d = Rp[((int64_t)i + (int64_t)i * K) * W];   /* the diagonal of R is real */
-    double* out = &Tt[((int64_t)col + (int64_t)i * ncols) * W]; out[0] = sr / d; if constexpr (CPLX) { out[1] = si / d; }
+  }
+  #pragma unroll
+  for (int i = 0; i < SOLVE_ROWS; ++i) {
+    if (i < rows) {
+      #pragma unroll
+      for (int w = 0; w < W; ++w) { t[i * W + w] = x[i][w]; }
+    }
   }
 }
 
-/* X[jpiv[x]-1, y] = (x < K) ? (x == y) : conj(T[y, x-K]) for y < K (reference: scatter mode 'I', src/matcopy.cu:48-52) */
+/* X[jpiv[x]-1, y] = (x < K) ? (x == y) : conj(T[y, x-K]) for y < K (reference: scatter mode 'I', src/matcopy.cu:48-52); T is K x (N - K), column-major */
 template <typename T, bool CPLX>
 __global__ void interp_out_kernel(int32_t N, int32_t K, const int32_t* __restrict__ jpiv, const double* __restrict__ Tt, T* __restrict__ X, int64_t ldx) {
   const int y = blockIdx.x * T_THREADS + threadIdx.x, x = blockIdx.y; if (y >= K) { return; }
   const int64_t row = jpiv[x] - 1; double vr, vi = 0.;
-  if (x < K) { vr = (x == y) ? 1. : 0.; } else { const int ncols = N - K; const double* t = &Tt[((int64_t)(x - K) + (int64_t)y * ncols) * (CPLX ? 2 : 1)]; vr = t[0]; if constexpr (CPLX) { vi = -t[1]; } }
+  if (x < K) { vr = (x == y) ? 1. : 0.; } else { const double* t = &Tt[((int64_t)y + (int64_t)(x - K) * K) * (CPLX ? 2 : 1)]; vr = t[0]; if constexpr (CPLX) { vi = -t[1]; } }
   if constexpr (CPLX) { T* o = &X[2 * (row + (int64_t)y * ldx)]; store_real<T>(o, vr); store_real<T>(o + 1, vi); } else { store_real<T>(&X[row + (int64_t)y * ldx], vr); }
 }
 
@@ -375,13 +405,24 @@ extern "C" int hykValuesOut(hipStream_t stream, int32_t K, int32_t Atype, const 
   return 0;
 }
 
-/* interpolation: Rp (K x N, FP64) and Tt ((N-K) x K) are scratch */
-extern "C" int hykInterpSolve(hipStream_t stream, int32_t N, int32_t K, int32_t Gtype, const void* Rt, int32_t ldr, const int32_t* jpiv, double* Rp, double* Tt) {
+/* interpolation: R11 (K x K) and T (K x (N - K)) are FP64 (complex: interleaved) column-major outputs with leading
+ * dimension K; T returns the solution of R11 T = R12.  Blocked back substitution: from the last block of SOLVE_ROWS rows
+ * upwards, the rows already solved are eliminated from the block by one matrix product, then the block is solved
+ * against its own triangle. */
+extern "C" int hykInterpSolve(hipStream_t stream, int32_t N, int32_t K, int32_t Gtype, const void* Rt, int32_t ldr, const int32_t* jpiv, double* R11, double* T) {
   if (N <= 0 || K <= 0 || K >= N) { return 0; }
-  const bool dd = (Gtype & ~1) == HYK_DD, cplx = Gtype & 1; const int WR = dd ? 2 : 1, WE = WR * (cplx ? 2 : 1);
+  const bool dd = (Gtype & ~1) == HYK_DD, cplx = Gtype & 1; const int WR = dd ? 2 : 1, WE = WR * (cplx ? 2 : 1), W = cplx ? 2 : 1;
   dim3 grid((K + T_THREADS - 1) / T_THREADS, N); const int ncols = N - K, sgrid = (ncols + T_THREADS - 1) / T_THREADS;
-  if (cplx) { gather_factor_kernel<true><<<grid, T_THREADS, 0, stream>>>(N, K, (const double*)Rt, ldr, WE, WR, jpiv, Rp); upper_solve_kernel<true><<<sgrid, T_THREADS, 0, stream>>>(K, ncols, Rp, Tt); }
-  else { gather_factor_kernel<false><<<grid, T_THREADS, 0, stream>>>(N, K, (const double*)Rt, ldr, WE, WR, jpiv, Rp); upper_solve_kernel<false><<<sgrid, T_THREADS, 0, stream>>>(K, ncols, Rp, Tt); }
+  if (cplx) { gather_factor_kernel<true><<<grid, T_THREADS, 0, stream>>>(N, K, (const double*)Rt, ldr, WE, WR, jpiv, R11, T); }
+  else { gather_factor_kernel<false><<<grid, T_THREADS, 0, stream>>>(N, K, (const double*)Rt, ldr, WE, WR, jpiv, R11, T); }
+  for (int i0 = (K - 1) / SOLVE_ROWS * SOLVE_ROWS; i0 >= 0; i0 -= SOLVE_ROWS) {
+    const int rows = K - i0 < SOLVE_ROWS ? K - i0 : SOLVE_ROWS, below = K - i0 - rows;
+    if (below > 0) {   /* T[i0 .. i0+rows) -= R11[i0 .. i0+rows, i0+rows .. K) T[i0+rows .. K) */
+      const int rc = hykGemm(stream, 'N', 'N', rows, ncols, below, -1.0, cplx ? HYK_F64C : HYK_F64, R11 + ((int64_t)i0 + (int64_t)(i0 + rows) * K) * W, K, T + (int64_t)(i0 + rows) * W, K, 1.0, T + (int64_t)i0 * W, K);
+      if (rc != 0) { return rc; }
+    }
+    if (cplx) { block_solve_kernel<true><<<sgrid, T_THREADS, 0, stream>>>(K, ncols, i0, rows, R11, T); } else { block_solve_kernel<false><<<sgrid, T_THREADS, 0, stream>>>(K, ncols, i0, rows, R11, T); }
+  }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 

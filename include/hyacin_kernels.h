@@ -88,8 +88,11 @@ int hykColumnNorms(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, co
 int hykBasisOut(hipStream_t stream, int32_t N, int32_t rank, int32_t Atype, const double* B, const double* sigma, const int32_t* order, void* X, int64_t ldx);
 int hykValuesOut(hipStream_t stream, int32_t K, int32_t Atype, const double* S, void* out);
 
-/* Interpolation tail.  Replaces cuBLAS trsm + scatter modes 'U' / 'I', src/gram_id.cpp:40-46, src/matcopy.cu:48-52. */
-int hykInterpSolve(hipStream_t stream, int32_t N, int32_t K, int32_t Gtype, const void* Rt, int32_t ldr, const int32_t* jpiv, double* Rp, double* Tt);
+/* Interpolation tail.  Replaces cuBLAS trsm + scatter modes 'U' / 'I', src/gram_id.cpp:40-46, src/matcopy.cu:48-52.
+ * hykInterpSolve: R11 (K x K) and T (K x (N - K)), FP64 or complex FP64, column-major with leading dimension K, are
+ * written: the factor in pivot order and the solution of R11 T = R12 (blocked back substitution).  hykInterpOut scatters
+ * the identity and conj(T) into X. */
+int hykInterpSolve(hipStream_t stream, int32_t N, int32_t K, int32_t Gtype, const void* Rt, int32_t ldr, const int32_t* jpiv, double* R11, double* T);
 int hykInterpOut(hipStream_t stream, int32_t N, int32_t K, int32_t Atype, const int32_t* jpiv, const double* Tt, void* X, int64_t ldx);
 
 /* Converting copy / transpose.  Replaces scatter_matcopy modes 'A', 'T', 'C', src/matcopy.cu:23-44,58-96. */

@@ -325,3 +325,36 @@ def test_f16_products(gl, cplx, opA, M, N, K, pad):
     scale = np.sqrt(np.mean(np.abs(want) ** 2))
     assert np.all(np.abs(got - want) <= 2.0**-10 * np.abs(want) + 2.0**-12 * scale + 1e-6)
     assert not host(Cd, np.float16, (N, ldc, comps))[:, M:, :].any()       # nothing written into the padding
+
+
+@pytest.mark.parametrize("cplx", [0, 1])
+@pytest.mark.parametrize("N,K", [(40, 7), (150, 32), (300, 75), (700, 257)])
+def test_interp_solve(gl, cplx, N, K):
+    """hykInterpSolve (cuBLAS trsm of src/gram_id.cpp:40-46): T = R11^-1 R12 for a factor given column-wise in pivot order,
+    against numpy's triangular solve; K below, at and across the block size of the blocked back substitution."""
+    from gpu_util import dev, zeros, ptr, stream, sync, host
+    rng = np.random.default_rng(91 + cplx)
+    W = 2 if cplx else 1
+    R = rng.standard_normal((K, N)) + (1j * rng.standard_normal((K, N)) if cplx else 0)
+    R[:, :K] = np.triu(R[:, :K])
+    R[np.arange(K), np.arange(K)] = 2.0 + np.abs(R[np.arange(K), np.arange(K)])      # real positive diagonal, well conditioned
+    piv = rng.permutation(N).astype(np.int32) + 1                                     # column at pivot position x is piv[x] - 1
+    ldr = K + 3
+    Rt = np.zeros((N, ldr, W))                                                        # Rt[column][row]
+    for x in range(N):
+        col = piv[x] - 1
+        Rt[col, :K, 0] = R[:, x].real
+        if cplx:
+            Rt[col, :K, 1] = R[:, x].imag
+    dRt, dp = dev(Rt), dev(piv)
+    R11 = zeros(K * K * W * 8)
+    T = zeros(K * (N - K) * W * 8)
+    assert gl.L.hykInterpSolve(stream(), N, K, 1 if cplx else 0, ptr(dRt), ldr, ptr(dp), ptr(R11), ptr(T)) == 0
+    sync()
+    got = host(T, np.float64, (N - K, K, W))
+    got = (got[..., 0] + 1j * got[..., 1]).T if cplx else got[..., 0].T
+    want = np.linalg.solve(R[:, :K], R[:, K:])
+    assert np.abs(got - want).max() <= 1e-11 * np.abs(want).max()
+    g11 = host(R11, np.float64, (K, K, W))
+    g11 = (g11[..., 0] + 1j * g11[..., 1]).T if cplx else g11[..., 0].T
+    assert np.array_equal(g11, R[:, :K])
