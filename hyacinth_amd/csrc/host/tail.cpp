@@ -72,8 +72,9 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
     const int32_t maxSweeps = sweeps > 0 ? 5 * sweeps : 30; int32_t used = 0;
     /* A pair is rotated while its cosine exceeds the storage precision, but never below sqrt(N) FP64 roundings: that is
      * what the dot product of two columns of length N carries as noise (the threshold of LAPACK's xGESVJ); rotating
-     * below it costs sweeps and leaves the orthogonality where it was. */
-    const double rotateAbove = std::max(machineEps, std::sqrt((double)N) * 2.220446049250313e-16);
+     * below it costs sweeps and leaves the orthogonality where it was.  Nor below a sixteenth of the accuracy asked for:
+     * cosines of that size move a singular value by less than eps / 2 of the largest one. */
+    const double rotateAbove = std::max(std::max(machineEps, std::sqrt((double)N) * 2.220446049250313e-16), eps / 16.);
     for (int32_t sw = 0; sw < maxSweeps && rank > 1; ++sw) {
       HYH_KERNEL(hykGramWorkspaceClear(s, counter.p, 64));
       HYH_KERNEL(hykJacobiSweep(s, Complex, N, rank, B.as<double>(), rotateAbove, counter.as<int32_t>())); ++used;
