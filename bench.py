@@ -32,6 +32,8 @@ WORKLOADS = {
     "cfg1": (0, "N", 4096, 256, 256, 1e-10, b"L", "real FP64 M=4096 N=256 eps=1e-10 (limbs, 6 digits)"),
     "cfg2": (2, "T", 65536, 1024, 512, 1e-5, b"A", "real FP32 opA=T M=65536 N=1024 eps=1e-5 (CRT real, 8 moduli)"),
     "cfg3": (1, "N", 131072, 2048, 1024, 1e-12, b"A", "complex FP64 M=131072 N=2048 eps=1e-12 (CRT complex, 15 moduli)"),
+    "cfg4": (5, "C", 262144, 4096, 256, 1e-3, b"L", "complex FP16 opA=C M=262144 N=4096 eps=1e-3 (limbs, 3 digits x 3 groups)"),
+    "cfg5": (0, "N", 1048576, 4096, 2048, 1e-8, b"A", "real FP64 M=1048576 N=4096 eps=1e-8 (CRT real, 11 moduli)"),
 }
 
 
@@ -41,9 +43,11 @@ def synth(torch, at, M, N, seed):
     g.manual_seed(seed)
     real = torch.float64 if at in (0, 1) else torch.float32
     comps = 2 if at & 1 else 1
-    scale = torch.pow(10.0, -torch.arange(N, device="cuda", dtype=torch.float64) / (N / 8.0)).to(real)
-    A = torch.randn((N, M, comps), generator=g, device="cuda", dtype=real) * scale[:, None, None]
-    return A.contiguous()
+    decades = 2.0 if at in (4, 5) else 8.0          # FP16 storage holds five decades in all
+    scale = torch.pow(10.0, -torch.arange(N, device="cuda", dtype=torch.float64) * (decades / N)).to(real)
+    A = torch.randn((N, M, comps), generator=g, device="cuda", dtype=real)
+    A.mul_(scale[:, None, None])
+    return A.half().contiguous() if at in (4, 5) else A.contiguous()
 
 
 def algorithmic_ops(alg, order, cplx, M, N):
