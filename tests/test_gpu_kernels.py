@@ -358,3 +358,37 @@ def test_interp_solve(gl, cplx, N, K):
     g11 = host(R11, np.float64, (K, K, W))
     g11 = (g11[..., 0] + 1j * g11[..., 1]).T if cplx else g11[..., 0].T
     assert np.array_equal(g11, R[:, :K])
+
+
+@pytest.mark.parametrize("cplx", [0, 1])
+@pytest.mark.parametrize("opA,opB", [("N", "N"), ("T", "N"), ("C", "N"), ("N", "C"), ("N", "T"), ("C", "T")])
+@pytest.mark.parametrize("M,N,K", [(70, 33, 19), (600, 130, 75), (1025, 257, 64)])
+def test_gemm_fp64(gl, cplx, opA, opB, M, N, K):
+    """hykGemm in FP64 / complex FP64 (the cuBLAS gemm calls of src/lra.cpp:86-105,202-203): C = alpha op(A) op(B) + beta C
+    against numpy, all operand forms, sizes on both the 64 x 64 and the 128 x 128 tile paths, ragged edges."""
+    from gpu_util import dev, ptr, stream, sync, host
+    rng = np.random.default_rng(5 + cplx)
+    W = 2 if cplx else 1
+    def rand(r, c):
+        return rng.standard_normal((r, c)) + (1j * rng.standard_normal((r, c)) if cplx else 0)
+    def op(X, o):
+        return X if o == "N" else (X.T if o == "T" else X.conj().T)
+    def store(X, ld):                                   # column-major with leading dimension ld, interleaved complex
+        buf = np.zeros((X.shape[1], ld, W))
+        buf[:, :X.shape[0], 0] = X.real.T
+        if cplx:
+            buf[:, :X.shape[0], 1] = X.imag.T
+        return buf
+    A = rand(*((M, K) if opA == "N" else (K, M)))
+    B = rand(*((K, N) if opB == "N" else (N, K)))
+    C0 = rand(M, N)
+    alpha, beta = -1.5, 0.75
+    want = alpha * op(A, opA) @ op(B, opB) + beta * C0
+    lda, ldb, ldc = A.shape[0] + 3, B.shape[0] + 1, M + 2
+    dA, dB, dC = dev(store(A, lda)), dev(store(B, ldb)), dev(store(C0, ldc))
+    rc = gl.L.hykGemm(stream(), opA.encode(), opB.encode(), M, N, K, C.c_double(alpha), 1 if cplx else 0, ptr(dA), C.c_int64(lda), ptr(dB), C.c_int64(ldb), C.c_double(beta), ptr(dC), C.c_int64(ldc))
+    assert rc == 0
+    sync()
+    got = host(dC, np.float64, (N, ldc, W))[:, :M, :]
+    got = (got[..., 0] + 1j * got[..., 1]).T if cplx else got[..., 0].T
+    assert np.abs(got - want).max() <= 1e-13 * np.abs(want).max() * max(1, K) ** 0.5
