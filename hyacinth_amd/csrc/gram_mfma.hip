@@ -611,32 +611,54 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_ring_kernel(const GramArgs 
 
 /* ------------------------------------------------------------------ CRT reconstruction */
 struct ReconTable {
-  int32_t order;
-  uint32_t m[HYK_CRT_CPLX_COUNT], d[HYK_CRT_CPLX_COUNT], minv[HYK_CRT_CPLX_COUNT];
+  int32_t order, rot;   /* rot: the first `rot` moduli of a complex launch hold p and q = Re +- i Im instead of Re and Im */
+  uint32_t m[HYK_CRT_CPLX_COUNT], d[HYK_CRT_CPLX_COUNT], minv[HYK_CRT_CPLX_COUNT], iminv[HYK_CRT_CPLX_COUNT];
   uint64_t Pd[HYK_CRT_CPLX_COUNT][3], P[3];
 };
 
-/* entry e of plane z: residues from the uint32 sums, centred CRT lift, C (+)= value.  clear: zero the sums afterwards. */
-__global__ __launch_bounds__(256) void crt_reconstruct_kernel(const ReconTable tab, int64_t count, uint32_t* __restrict__ acc, int64_t planeStride, int32_t beta, int32_t orderC, uint64_t* __restrict__ C, int32_t clear) {
-  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; const int z = blockIdx.y;
-  if (e >= count) { return; }
-  hyk::I192 a; a.w[0] = a.w[1] = a.w[2] = 0;
-  for (int x = 0; x < tab.order; ++x) {
-    uint32_t* src = &acc[(int64_t)(z * tab.order + x) * planeStride + e];
-    const uint32_t r = hyk::reduce_u32(*src, tab.m[x], tab.d[x]); if (clear) { *src = 0u; }
-    const uint32_t tt = hyk::reduce_u32(r * tab.minv[x], tab.m[x], tab.d[x]);
-    hyk::I192 pd; pd.w[0] = tab.Pd[x][0]; pd.w[1] = tab.Pd[x][1]; pd.w[2] = tab.Pd[x][2];
-    /* keep |a| < P: add t * (P/m) when a < 0, (t - m) * (P/m) otherwise */
-    if (hyk::i192_is_neg(a)) { hyk::i192_add(a, hyk::i192_mul_small(pd, tt)); }
-    else { hyk::i192_add(a, hyk::i192_neg(hyk::i192_mul_small(pd, tab.m[x] - tt))); }
-  }
+/* one modulus of the centred lift: a += s (P/m) with s = (r minv mod m) - (a >= 0 ? m : 0), which keeps |a| < P */
+__device__ __forceinline__ void recon_step(hyk::I192& a, uint32_t r, const ReconTable& tab, int x) {
+  const uint32_t tt = hyk::reduce_u32(r * tab.minv[x], tab.m[x], tab.d[x]);
+  hyk::I192 pd; pd.w[0] = tab.Pd[x][0]; pd.w[1] = tab.Pd[x][1]; pd.w[2] = tab.Pd[x][2];
+  if (hyk::i192_is_neg(a)) { hyk::i192_add(a, hyk::i192_mul_small(pd, tt)); }
+  else { hyk::i192_add(a, hyk::i192_neg(hyk::i192_mul_small(pd, tab.m[x] - tt))); }
+}
+/* into [-P/2, P/2), then C (+)= a */
+__device__ __forceinline__ void recon_finish(hyk::I192 a, const ReconTable& tab, int32_t beta, int32_t orderC, uint64_t* out, int64_t count) {
   hyk::I192 P; P.w[0] = tab.P[0]; P.w[1] = tab.P[1]; P.w[2] = tab.P[2];
   if (hyk::i192_is_neg(a)) { hyk::i192_add(a, P); }
   hyk::I192 twice = a; hyk::i192_add(twice, a); hyk::I192 diff = twice; hyk::i192_add(diff, hyk::i192_neg(P));
-  if (!hyk::i192_is_neg(diff)) { hyk::i192_add(a, hyk::i192_neg(P)); }   /* 2a >= P  ->  a - P, result in [-P/2, P/2) */
-  uint64_t* out = &C[(int64_t)z * orderC * count + e];
+  if (!hyk::i192_is_neg(diff)) { hyk::i192_add(a, hyk::i192_neg(P)); }   /* 2a >= P  ->  a - P */
   if (beta) { hyk::I192 old = hyk::limbs_to_i192(orderC, out, count); hyk::i192_add(a, old); }
   hyk::i192_to_limbs(a, orderC, out, count);
+}
+
+/* Entry e: residues from the uint32 sums of its planes (real: plane x; complex: planes x and order + x), centred CRT
+ * lift, C (+)= value; the sums are zeroed afterwards.  The rotating moduli of a complex launch arrive as p = W[y, x] and
+ * q = W[x, y] of W = P^T Q (one plane each, each written by one group of the contraction): Re = (p + q) / 2,
+ * Im = (p - q) / (2 i) mod m are formed here (the reference's accumulate_crt_rotate, src/crt_rotate.cu:5-46, does it
+ * in the epilogue of its GEMM). */
+__global__ __launch_bounds__(256) void crt_reconstruct_kernel(const ReconTable tab, int64_t count, uint32_t* __restrict__ acc, int64_t planeStride, int32_t beta, int32_t orderC, uint64_t* __restrict__ C, int32_t cplx) {
+  const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (e >= count) { return; }
+  hyk::I192 re, im; re.w[0] = re.w[1] = re.w[2] = 0; im = re;
+  for (int x = 0; x < tab.order; ++x) {
+    uint32_t* s0 = &acc[(int64_t)x * planeStride + e];
+    uint32_t r0 = hyk::reduce_u32(*s0, tab.m[x], tab.d[x]); *s0 = 0u;
+    if (cplx) {
+      uint32_t* s1 = &acc[(int64_t)(tab.order + x) * planeStride + e];
+      uint32_t r1 = hyk::reduce_u32(*s1, tab.m[x], tab.d[x]); *s1 = 0u;
+      if (x < tab.rot) {
+        const uint32_t m = tab.m[x], sum = r0 + r1, dif = r0 + m - r1;
+        r0 = hyk::reduce_u32(hyk::reduce_u32(sum, m, tab.d[x]) * ((m + 1u) >> 1), m, tab.d[x]);
+        r1 = hyk::reduce_u32(hyk::reduce_u32(dif, m, tab.d[x]) * tab.iminv[x], m, tab.d[x]);
+      }
+      recon_step(im, r1, tab, x);
+    }
+    recon_step(re, r0, tab, x);
+  }
+  recon_finish(re, tab, beta, orderC, &C[e], count);
+  if (cplx) { recon_finish(im, tab, beta, orderC, &C[(int64_t)orderC * count + e], count); }
 }
 
 /* limb path: C (+)= sum_s T_s 2^(8 s) */
@@ -868,8 +890,9 @@ extern "C" int hykGramCrt(hipStream_t stream, int32_t Complex, int32_t N, int32_
   if (N <= 0) { return 0; }
   if (orderA < 1 || orderA > (Complex ? HYK_CRT_CPLX_COUNT : HYK_CRT_REAL_COUNT) || orderC < 1 || orderC > 3 || K <= 0 || (K & 127) || ldb < K || (ldb & 15) || ((uintptr_t)panels & 15)) { return -1; }
   /* 131072 products per int32: residues of every modulus but 256 are at most 125 in magnitude, and mod 256 a wrap is harmless */
-  GroupBuilder gb(stream, EPI_MOD, 131072, Complex == 0, panels, ldb, N, K, workspace);
-  ReconTable tab; tab.order = orderA;
+  /* planes are shared between groups only by the three-product moduli of a complex launch */
+  GroupBuilder gb(stream, EPI_MOD, 131072, Complex == 0 || orderA <= HYK_CRT_CPLX_SPLIT, panels, ldb, N, K, workspace);
+  ReconTable tab; tab.order = orderA; tab.rot = 0;
   if (!Complex) {
     for (int x = 0; x < orderA; ++x) { GramGroup& g = gb.begin(1); set_mod(g, hyk_crt_real_mo[x]); g.mulRe = 1; g.planeRe = (uint16_t)x; gb.pair(g, x, x); }
     for (int x = 0; x < orderA; ++x) { tab.m[x] = hyk_crt_real_mo[x]; tab.d[x] = (uint32_t)(0x100000000ull / tab.m[x]); tab.minv[x] = hyk_crt_real_minv[orderA - 1][x]; for (int k = 0; k < 3; ++k) { tab.Pd[x][k] = hyk_crt_real_Pd[orderA - 1][x][k]; } }
@@ -877,11 +900,12 @@ extern "C" int hykGramCrt(hipStream_t stream, int32_t Complex, int32_t N, int32_
   } else {
     const int rot = orderA < HYK_CRT_CPLX_SPLIT ? orderA : HYK_CRT_CPLX_SPLIT;
     for (int x = 0; x < rot; ++x) {
-      /* W = P^T Q: elements on or above the diagonal are p = Re + i Im, the transposed ones q = Re - i Im (mod m);
-       * Re = (p + q)/2, Im = (p - q)/(2 i).  On the diagonal both groups contribute: Re gets p, Im gets 0. */
-      const uint32_t m = hyk_crt_cplx_mo[x], inv2 = (m + 1) / 2, iminv = hyk_crt_cplx_iminv[x];
-      GramGroup& g0 = gb.begin(1); set_mod(g0, m); g0.mulRe = inv2; g0.mulIm = iminv; g0.planeRe = (uint16_t)x; g0.planeIm = (uint16_t)(orderA + x); gb.pair(g0, 2 * x, 2 * x + 1);
-      GramGroup& g1 = gb.begin(1); set_mod(g1, m); g1.mulRe = inv2; g1.mulIm = m - iminv; g1.planeRe = (uint16_t)x; g1.planeIm = (uint16_t)(orderA + x); gb.pair(g1, 2 * x + 1, 2 * x);
+      /* W = P^T Q: elements on or above the diagonal are p = Re + i Im, the transposed ones q = Re - i Im (mod m).  Each
+       * goes to a plane of its own (p: plane x, q: plane orderA + x), so every accumulator entry has one writer and the
+       * contraction can store instead of adding atomically; the reconstruction forms Re = (p + q)/2, Im = (p - q)/(2 i). */
+      const uint32_t m = hyk_crt_cplx_mo[x];
+      GramGroup& g0 = gb.begin(1); set_mod(g0, m); g0.mulRe = 1; g0.planeRe = (uint16_t)x; gb.pair(g0, 2 * x, 2 * x + 1);
+      GramGroup& g1 = gb.begin(1); set_mod(g1, m); g1.mulRe = 1; g1.planeRe = (uint16_t)(orderA + x); gb.pair(g1, 2 * x + 1, 2 * x);
     }
     for (int x = HYK_CRT_CPLX_SPLIT; x < orderA; ++x) {
       /* 3M scheme mod m: Re = S^T S - (R^T I + I^T R), Im = R^T I - I^T R with S = R + I */
@@ -890,12 +914,13 @@ extern "C" int hykGramCrt(hipStream_t stream, int32_t Complex, int32_t N, int32_
       GramGroup& g0 = gb.begin(1); set_mod(g0, m); g0.mulRe = m - 1; g0.mulIm = 1; g0.planeRe = (uint16_t)x; g0.planeIm = (uint16_t)(orderA + x); gb.pair(g0, base + 1, base + 2);
       GramGroup& g1 = gb.begin(1); set_mod(g1, m); g1.mulRe = m - 1; g1.mulIm = m - 1; g1.planeRe = (uint16_t)x; g1.planeIm = (uint16_t)(orderA + x); gb.pair(g1, base + 2, base + 1);
     }
-    for (int x = 0; x < orderA; ++x) { tab.m[x] = hyk_crt_cplx_mo[x]; tab.d[x] = (uint32_t)(0x100000000ull / tab.m[x]); tab.minv[x] = hyk_crt_cplx_minv[orderA - 1][x]; for (int k = 0; k < 3; ++k) { tab.Pd[x][k] = hyk_crt_cplx_Pd[orderA - 1][x][k]; } }
+    tab.rot = rot;
+    for (int x = 0; x < orderA; ++x) { tab.m[x] = hyk_crt_cplx_mo[x]; tab.d[x] = (uint32_t)(0x100000000ull / tab.m[x]); tab.minv[x] = hyk_crt_cplx_minv[orderA - 1][x]; tab.iminv[x] = x < HYK_CRT_CPLX_SPLIT ? hyk_crt_cplx_iminv[x] : 0u; for (int k = 0; k < 3; ++k) { tab.Pd[x][k] = hyk_crt_cplx_Pd[orderA - 1][x][k]; } }
     for (int k = 0; k < 3; ++k) { tab.P[k] = hyk_crt_cplx_P[orderA - 1][k]; }
   }
   gb.flush(); if (gb.err != hipSuccess) { return -3; }
-  const int64_t T = ((int64_t)N * N + N) / 2; dim3 grid((uint32_t)((T + 255) / 256), Complex ? 2u : 1u);
-  crt_reconstruct_kernel<<<grid, 256, 0, stream>>>(tab, T, reinterpret_cast<uint32_t*>(workspace), T, beta, orderC, C, 1);
+  const int64_t T = ((int64_t)N * N + N) / 2;
+  crt_reconstruct_kernel<<<(uint32_t)((T + 255) / 256), 256, 0, stream>>>(tab, T, reinterpret_cast<uint32_t*>(workspace), T, beta, orderC, C, Complex ? 1 : 0);
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
