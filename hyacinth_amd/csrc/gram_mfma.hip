@@ -75,6 +75,7 @@ struct GramArgs {
   uint32_t tileMagic, splitMagic;   /* floor(2^32 / d) + 1: x / d == mulhi(x, magic) while x * d < 2^32 (checked on the host); 0 for d == 1 */
   /* set-aligned schedule (ring kernel): a set = the tileCount tiles of one (group, K split); slots = compute units per XCD */
   int32_t slotShift, roundsPerXcd, setCount, mainRounds, leftover, perRound; uint32_t mainMagic, leftMagic;
+  int32_t pairShift;                /* 1: groups 2 s and 2 s + 1 read the same panels and take turns inside one set (complex residues) */
   GramGroup groups[MAX_GROUPS];
   uint32_t pairs[MAX_PAIRS];  /* lanePanel | aPanel << 16 */
 };
@@ -447,7 +448,7 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_ring_kernel(const GramArgs 
     if (inRound >= args.perRound || set >= args.setCount) { return; }
     t = (args.mainRounds << args.slotShift) + (slot - inRound * args.leftover);
   }
-  const int g = divide(set, args.splitMagic), ks = set - g * args.kSplits;
+  const int sg = divide(set, args.splitMagic), ks = set - sg * args.kSplits, g = (sg << args.pairShift) + (t & ((1 << args.pairShift) - 1)); t >>= args.pairShift;
   int tb = 0; while ((tb + 1) * (tb + 2) / 2 <= t) { ++tb; }
   const int ta = t - tb * (tb + 1) / 2;
   const GramGroup grp = args.groups[g];
@@ -730,7 +731,7 @@ int compute_units() {
   return units;
 }
 
-hipError_t launch_gram(hipStream_t stream, GramArgs& a, int epi, int maxProducts, bool unshared) {
+hipError_t launch_gram(hipStream_t stream, GramArgs& a, int epi, int maxProducts, bool unshared, bool paired) {
   int maxPairs = 1; for (int g = 0; g < a.groupCount; ++g) { maxPairs = a.groups[g].pairCount > maxPairs ? a.groups[g].pairCount : maxPairs; }
   const int bk = g_bk == 0 ? RING_K : (g_bk == 2 ? DMA_BK : g_bk); int kCap = (maxProducts / maxPairs) / bk * bk; if (kCap < bk) { return hipErrorInvalidValue; }
   /* K split.  One workgroup runs per compute unit, so a launch takes rounds = ceil(items / units) item times; an item costs
@@ -740,7 +741,12 @@ hipError_t launch_gram(hipStream_t stream, GramArgs& a, int epi, int maxProducts
   const int minSplits = (a.K + kCap - 1) / kCap; int splits = minSplits; double best = -1.;
   for (int cand = minSplits; cand <= minSplits + 15; ++cand) {
     const int len = ((a.K + cand - 1) / cand + bk - 1) / bk * bk; if (len < 16 * bk && cand > minSplits) { break; }
-    const int count = (a.K + len - 1) / len; const int64_t rounds = (base * count + units - 1) / units;
+    const int count = (a.K + len - 1) / len; int64_t rounds = (base * count + units - 1) / units;
+    if (g_bk == 0) {   /* the ring kernel's schedule hands out whole rounds of an XCD (set-aligned rounds, below) */
+      const int slots = units / XCDS >= 32 ? 32 : (units / XCDS >= 16 ? 16 : (units / XCDS >= 8 ? 8 : 1)), shift = (paired && (a.groupCount & 1) == 0) ? 1 : 0;
+      const int setTiles = a.tileCount << shift; const int64_t sets = (int64_t)(a.groupCount >> shift) * count; const int left = setTiles % slots, per = left ? slots / left : 0;
+      rounds = (sets * (setTiles / slots) + (left ? (sets + per - 1) / per : 0) + XCDS - 1) / XCDS;
+    }
     const double cost = (double)rounds * ((double)len / 64. + 48.);   /* in units of 64 K-bytes of contraction */
     if (best < 0. || cost < best * 0.98) { best = cost; splits = cand; }   /* a further split has to win by 2 % */
   }
@@ -754,7 +760,8 @@ hipError_t launch_gram(hipStream_t stream, GramArgs& a, int epi, int maxProducts
   if (g_bk == 0) {
     /* set-aligned schedule; compute units per XCD rounded down to a power of two (32 on this device) */
     int slots = units / XCDS; a.slotShift = 0; while ((2 << a.slotShift) <= slots) { ++a.slotShift; } slots = 1 << a.slotShift;
-    a.setCount = a.groupCount * a.kSplits; a.mainRounds = a.tileCount / slots; a.leftover = a.tileCount % slots; a.perRound = a.leftover ? slots / a.leftover : 0;
+    a.pairShift = (paired && (a.groupCount & 1) == 0) ? 1 : 0; const int setTiles = a.tileCount << a.pairShift;
+    a.setCount = (a.groupCount >> a.pairShift) * a.kSplits; a.mainRounds = setTiles / slots; a.leftover = setTiles % slots; a.perRound = a.leftover ? slots / a.leftover : 0;
     const int rounds = a.setCount * a.mainRounds + (a.leftover ? (a.setCount + a.perRound - 1) / a.perRound : 0);
     a.roundsPerXcd = (rounds + XCDS - 1) / XCDS;
     a.mainMagic = a.mainRounds > 1 ? (uint32_t)((1ull << 32) / (uint32_t)a.mainRounds) + 1u : 0u; a.leftMagic = a.leftover > 1 ? (uint32_t)((1ull << 32) / (uint32_t)a.leftover) + 1u : 0u;
@@ -776,10 +783,11 @@ void base_args(GramArgs& a, const int8_t* panels, int64_t ldb, int32_t N, int32_
 }
 
 struct GroupBuilder {
-  GramArgs a; int pairs = 0; int epi; int maxProducts; bool unshared; hipStream_t stream; hipError_t err = hipSuccess;
+  GramArgs a; int pairs = 0; int epi; int maxProducts; bool unshared; bool paired = false; hipStream_t stream; hipError_t err = hipSuccess;
+  /* paired: groups come in adjacent pairs that read the same two panels (set by the caller before the first group) */
   /* unshared: no two groups write the same accumulator plane (true for the real paths) */
   GroupBuilder(hipStream_t s, int epi_, int maxProducts_, bool unshared_, const int8_t* panels, int64_t ldb, int32_t N, int32_t K, void* acc) : epi(epi_), maxProducts(maxProducts_), unshared(unshared_), stream(s) { base_args(a, panels, ldb, N, K, acc); }
-  void flush() { if (a.groupCount > 0 && err == hipSuccess) { err = launch_gram(stream, a, epi, maxProducts, unshared); } a.groupCount = 0; pairs = 0; }
+  void flush() { if (a.groupCount > 0 && err == hipSuccess) { err = launch_gram(stream, a, epi, maxProducts, unshared, paired); } a.groupCount = 0; pairs = 0; }
   /* begins a group; flushes first when the tables are full */
   GramGroup& begin(int npairs) {
     if (a.groupCount == MAX_GROUPS || pairs + npairs > MAX_PAIRS) { flush(); }
@@ -893,6 +901,7 @@ extern "C" int hykGramCrt(hipStream_t stream, int32_t Complex, int32_t N, int32_
   /* planes are shared between groups only by the three-product moduli of a complex launch */
   GroupBuilder gb(stream, EPI_MOD, 131072, Complex == 0 || orderA <= HYK_CRT_CPLX_SPLIT, panels, ldb, N, K, workspace);
   ReconTable tab; tab.order = orderA; tab.rot = 0;
+  gb.paired = Complex != 0 && orderA <= HYK_CRT_CPLX_SPLIT;
   if (!Complex) {
     for (int x = 0; x < orderA; ++x) { GramGroup& g = gb.begin(1); set_mod(g, hyk_crt_real_mo[x]); g.mulRe = 1; g.planeRe = (uint16_t)x; gb.pair(g, x, x); }
     for (int x = 0; x < orderA; ++x) { tab.m[x] = hyk_crt_real_mo[x]; tab.d[x] = (uint32_t)(0x100000000ull / tab.m[x]); tab.minv[x] = hyk_crt_real_minv[orderA - 1][x]; for (int k = 0; k < 3; ++k) { tab.Pd[x][k] = hyk_crt_real_Pd[orderA - 1][x][k]; } }
