@@ -362,8 +362,8 @@ extern "C" int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, in
   }
   if (Complex && r >= 16) {
     if (N <= 4 * T_THREADS) { return blocked_sweep<true, 4, 4>(stream, N, r, B, tol, rotations); }
-    if (N <= 8 * T_THREADS) { return blocked_sweep<true, 8, 4>(stream, N, r, B, tol, rotations); }
-    if (N <= 16 * T_THREADS) { return blocked_sweep<true, 16, 2>(stream, N, r, B, tol, rotations); }
+    if (N <= 4 * 512) { return blocked_sweep<true, 4, 4, 512>(stream, N, r, B, tol, rotations); }
+    if (N <= 8 * 512) { return blocked_sweep<true, 8, 2, 512>(stream, N, r, B, tol, rotations); }
   }
   const int n = (r + 1) & ~1;
   for (int round = 0; round < n - 1; ++round) {
