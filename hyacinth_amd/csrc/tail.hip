@@ -358,7 +358,7 @@ extern "C" int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, in
   if (!Complex && r >= 16) {
     if (N <= 4 * T_THREADS) { return blocked_sweep<false, 4, 4>(stream, N, r, B, tol, rotations); }
     if (N <= 8 * T_THREADS) { return blocked_sweep<false, 8, 4>(stream, N, r, B, tol, rotations); }
-    if (N <= 16 * T_THREADS) { return blocked_sweep<false, 16, 4>(stream, N, r, B, tol, rotations); }
+    if (N <= 8 * 512) { return blocked_sweep<false, 8, 4, 512>(stream, N, r, B, tol, rotations); }
   }
   if (Complex && r >= 16) {
     if (N <= 4 * T_THREADS) { return blocked_sweep<true, 4, 4>(stream, N, r, B, tol, rotations); }

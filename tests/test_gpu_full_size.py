@@ -115,10 +115,11 @@ def test_repeated_integer_block(env, name, at, M, N, eps, alg, bound, m0):
         assert np.array_equal(got_im, want_im), name
 
 
-@pytest.mark.parametrize("at,M,N,K,eps", [(F64, 16384, 2048, 1024, 1e-12), (F64C, 8192, 1024, 512, 1e-12)], ids=["real", "complex"])
+@pytest.mark.parametrize("at,M,N,K,eps", [(F64, 16384, 2048, 1024, 1e-12), (F64C, 8192, 1024, 512, 1e-12), (F64, 8192, 4096, 256, 1e-7), (F64C, 6144, 3000, 128, 1e-6)],
+                         ids=["real", "complex", "real-4096", "complex-3000"])
 def test_fit_at_full_width(env, at, M, N, K, eps):
-    """hyacinTsvdFit with the column count of the benchmark target (the Cholesky and Jacobi kernels then run on every
-    compute unit, with many workgroups exchanging data): singular values against sqrt(eigvalsh(A^H A)) computed by
+    """hyacinTsvdFit with the column counts of the benchmark configurations (the Cholesky and Jacobi kernels then run on
+    every compute unit, with many workgroups exchanging data; above 2048 columns they take other variants): singular values against sqrt(eigvalsh(A^H A)) computed by
     torch in FP64, an orthonormal basis, and the same bits on a second run (every reduction order is fixed)."""
     ha, h, torch = env
     L = ha.lib()
@@ -139,13 +140,16 @@ def test_fit_at_full_width(env, at, M, N, K, eps):
     Am = torch.view_as_complex(A).reshape(N, M) if cplx else A.reshape(N, M)       # row j = column j of A
     G = Am.conj() @ Am.T                                                            # G[y, x] = sum_k conj(a_ky) a_kx
     ev = torch.linalg.eigvalsh(G).flip(0).clamp_min(0).sqrt()
-    rel = ((S - ev[:K]).abs() / ev[:K]).max().item()
-    assert rel <= 1e-9, rel
+    if eps <= 1e-10:
+        rel = ((S - ev[:K]).abs() / ev[:K]).max().item()
+        assert rel <= 1e-9, rel
+    else:                                                        # the bar of the path: 10 eps of the largest value
+        assert ((S - ev[:K]).abs().max() / ev[0]).item() <= 10 * eps
     Vm = (torch.view_as_complex(V.reshape(K, N, 2)) if cplx else V.reshape(K, N))   # row i = basis vector i
     eye = torch.eye(K, device="cuda", dtype=Vm.dtype)
-    assert (Vm.conj() @ Vm.T - eye).abs().max().item() <= 1e-12
+    assert (Vm.conj() @ Vm.T - eye).abs().max().item() <= max(1e-12, eps)    # rotations stop at cosines of eps / 16
     # the basis spans the dominant right singular subspace: the residual of A outside it is the tail of the spectrum
     resid2 = (Am.abs() ** 2).sum().item() - ((Vm @ Am).abs() ** 2).sum().item()   # row i of Vm @ Am = (A v_i)^T
     tail2 = (ev[K:] ** 2).sum().item()
-    assert abs(resid2 - tail2) <= 1e-6 * tail2 + 1e-12 * (ev ** 2).sum().item()
+    assert abs(resid2 - tail2) <= 1e-6 * tail2 + max(1e-12, (10 * eps) ** 2) * (ev ** 2).sum().item()
     assert outs[1][0] == rank and torch.equal(outs[1][1], S) and torch.equal(outs[1][2], V)
