@@ -277,6 +277,10 @@ constexpr int DMA_BK = 64, DMA_STAGES = 4, DMA_TILE_BYTES = TILE * DMA_BK, DMA_S
 __device__ __forceinline__ void dma16(uint32_t ldsAddr, const int8_t* src) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" :: "s"(ldsAddr), "v"(src) : "memory");
 }
+/* the same with the address as a wave-uniform base plus an unsigned 32-bit offset per lane: no vector arithmetic per load */
+__device__ __forceinline__ void dma16(uint32_t ldsAddr, const int8_t* base, uint32_t laneOffset) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" :: "s"(ldsAddr), "v"(laneOffset), "s"(base) : "memory");
+}
 
 template <int EPI, bool EXCL>
 __global__ __launch_bounds__(G_THREADS, 1) void gram_dma_kernel(const GramArgs args) {
@@ -456,7 +460,8 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_ring_kernel(const GramArgs 
   const int y0 = ta * TILE, x0 = tb * TILE;
 
   /* load r (0..3) of a unit: lane tid fills slot tid % 8 of row tid / 8 + 32 r (tile row + 128 for the second half) */
-  int64_t srcLane[2][4], srcA[2][4];
+  /* byte offsets from the first row of the tile (the host has checked that 256 rows fit 32 bits) */
+  uint32_t srcLane[2][4], srcA[2][4];
   {
     const int rowBase = tid >> 3, kq = (tid & 7) ^ S::swz(rowBase);   /* the swizzle depends on the row modulo 32 only */
     #pragma unroll
@@ -465,7 +470,7 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_ring_kernel(const GramArgs 
       for (int r = 0; r < 4; ++r) {
         const int row = h * 128 + rowBase + 32 * r;
         int cy = y0 + row; cy = cy < args.N ? cy : args.N - 1; int cx = x0 + row; cx = cx < args.N ? cx : args.N - 1;
-        srcLane[h][r] = (int64_t)cy * args.ldb + kq * 16; srcA[h][r] = (int64_t)cx * args.ldb + kq * 16;
+        srcLane[h][r] = (uint32_t)(cy - y0) * (uint32_t)args.ldb + (uint32_t)kq * 16u; srcA[h][r] = (uint32_t)(cx - x0) * (uint32_t)args.ldb + (uint32_t)kq * 16u;
       }
     }
   }
@@ -487,25 +492,26 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_ring_kernel(const GramArgs 
   const int iters = slabs * grp.pairCount;
   const uint32_t pp0 = args.pairs[grp.pairBegin];
   int pairL = 0, slabL = 0, issuedL = 1, pairA = 0, slabA = 0, issuedA = 1; uint32_t nextL = pp0, nextA = pp0;
-  const int8_t* baseLane = args.panels + (int64_t)(pp0 & 0xffffu) * args.panelStride + k0;
-  const int8_t* baseA = args.panels + (int64_t)(pp0 >> 16) * args.panelStride + k0;
+  const int64_t rowsLane = (int64_t)y0 * args.ldb + k0, rowsA = (int64_t)x0 * args.ldb + k0;
+  const int8_t* baseLane = args.panels + (int64_t)(pp0 & 0xffffu) * args.panelStride + rowsLane;
+  const int8_t* baseA = args.panels + (int64_t)(pp0 >> 16) * args.panelStride + rowsA;
   auto peekL = [&]() { const int q = pairL + 1 < (int)grp.pairCount ? pairL + 1 : (int)grp.pairCount - 1; nextL = args.pairs[grp.pairBegin + q]; };
   auto peekA = [&]() { const int q = pairA + 1 < (int)grp.pairCount ? pairA + 1 : (int)grp.pairCount - 1; nextA = args.pairs[grp.pairBegin + q]; };
   auto advanceL = [&]() {
     const bool more = issuedL < iters, wrap = more && (slabL + 1 == slabs);
-    const int8_t* cand = args.panels + (int64_t)(nextL & 0xffffu) * args.panelStride + k0;
+    const int8_t* cand = args.panels + (int64_t)(nextL & 0xffffu) * args.panelStride + rowsLane;
     baseLane = wrap ? cand : baseLane + (more ? RING_K : 0); slabL = wrap ? 0 : slabL + (more ? 1 : 0); pairL += wrap ? 1 : 0; issuedL += more ? 1 : 0;
   };
   auto advanceA = [&]() {
     const bool more = issuedA < iters, wrap = more && (slabA + 1 == slabs);
-    const int8_t* cand = args.panels + (int64_t)(nextA >> 16) * args.panelStride + k0;
+    const int8_t* cand = args.panels + (int64_t)(nextA >> 16) * args.panelStride + rowsA;
     baseA = wrap ? cand : baseA + (more ? RING_K : 0); slabA = wrap ? 0 : slabA + (more ? 1 : 0); pairA += wrap ? 1 : 0; issuedA += more ? 1 : 0;
   };
   /* ring position of the next unit to fill (byte offset, wraps at RING_BYTES) */
   uint32_t fillOff = 0;
   auto next_unit = [&]() { const uint32_t u = fillOff; fillOff += RING_UNIT_BYTES; fillOff = fillOff == (uint32_t)RING_BYTES ? 0u : fillOff; return u; };
-  auto fill_lane = [&](int h, int r, uint32_t unitOff) { dma16(dmaBase + unitOff + (uint32_t)r * 4096u, baseLane + srcLane[h][r]); };
-  auto fill_a = [&](int h, int r, uint32_t unitOff) { dma16(dmaBase + unitOff + (uint32_t)r * 4096u, baseA + srcA[h][r]); };
+  auto fill_lane = [&](int h, int r, uint32_t unitOff) { dma16(dmaBase + unitOff + (uint32_t)r * 4096u, baseLane, srcLane[h][r]); };
+  auto fill_a = [&](int h, int r, uint32_t unitOff) { dma16(dmaBase + unitOff + (uint32_t)r * 4096u, baseA, srcA[h][r]); };
 
   const int rowOff = (lane & 31) * RING_K, sw = S::swz(lane & 31), hi = lane >> 5;
   int kOff[4];
@@ -732,8 +738,10 @@ int compute_units() {
 }
 
 hipError_t launch_gram(hipStream_t stream, GramArgs& a, int epi, int maxProducts, bool unshared, bool paired) {
+  /* the ring kernel addresses the 256 rows of a tile with 32-bit byte offsets: longer rows go to the register-staged kernel */
+  const int mode = (g_bk == 0 && 255ll * a.ldb + RING_K > 0xffffffffll) ? 128 : g_bk;
   int maxPairs = 1; for (int g = 0; g < a.groupCount; ++g) { maxPairs = a.groups[g].pairCount > maxPairs ? a.groups[g].pairCount : maxPairs; }
-  const int bk = g_bk == 0 ? RING_K : (g_bk == 2 ? DMA_BK : g_bk); int kCap = (maxProducts / maxPairs) / bk * bk; if (kCap < bk) { return hipErrorInvalidValue; }
+  const int bk = mode == 0 ? RING_K : (mode == 2 ? DMA_BK : mode); int kCap = (maxProducts / maxPairs) / bk * bk; if (kCap < bk) { return hipErrorInvalidValue; }
   /* K split.  One workgroup runs per compute unit, so a launch takes rounds = ceil(items / units) item times; an item costs
    * its K range plus a fixed prologue / epilogue (65536 reductions and atomics) worth about 48 x 64 K-bytes of it.  Take
    * the split count that minimises rounds x (K range + epilogue); the cap keeps the int32 sums exact. */
@@ -742,7 +750,7 @@ hipError_t launch_gram(hipStream_t stream, GramArgs& a, int epi, int maxProducts
   for (int cand = minSplits; cand <= minSplits + 15; ++cand) {
     const int len = ((a.K + cand - 1) / cand + bk - 1) / bk * bk; if (len < 16 * bk && cand > minSplits) { break; }
     const int count = (a.K + len - 1) / len; int64_t rounds = (base * count + units - 1) / units;
-    if (g_bk == 0) {   /* the ring kernel's schedule hands out whole rounds of an XCD (set-aligned rounds, below) */
+    if (mode == 0) {   /* the ring kernel's schedule hands out whole rounds of an XCD (set-aligned rounds, below) */
       const int slots = units / XCDS >= 32 ? 32 : (units / XCDS >= 16 ? 16 : (units / XCDS >= 8 ? 8 : 1)), shift = (paired && (a.groupCount & 1) == 0) ? 1 : 0;
       const int setTiles = a.tileCount << shift; const int64_t sets = (int64_t)(a.groupCount >> shift) * count; const int left = setTiles % slots, per = left ? slots / left : 0;
       rounds = (sets * (setTiles / slots) + (left ? (sets + per - 1) / per : 0) + XCDS - 1) / XCDS;
@@ -752,12 +760,12 @@ hipError_t launch_gram(hipStream_t stream, GramArgs& a, int epi, int maxProducts
   }
   int kLen = ((a.K + splits - 1) / splits + bk - 1) / bk * bk; if (kLen > kCap) { kLen = kCap; }
   if (kLen > a.K) { kLen = a.K; }
-  a.kLen = kLen; a.kSplits = (a.K + kLen - 1) / kLen; a.exclusive = (unshared && a.kSplits == 1 && (g_bk == 0 || g_bk == 2)) ? 1 : 0;
+  a.kLen = kLen; a.kSplits = (a.K + kLen - 1) / kLen; a.exclusive = (unshared && a.kSplits == 1 && (mode == 0 || mode == 2)) ? 1 : 0;
   const int64_t total = base * a.kSplits; if (total > 0x7fffffff / 2) { return hipErrorInvalidValue; }
   a.totalItems = (int)total; a.itemsPerXcd = (int)((total + XCDS - 1) / XCDS);
   if (total * a.tileCount >= (1ll << 32) || total * a.kSplits >= (1ll << 32)) { return hipErrorInvalidValue; }
   a.tileMagic = a.tileCount > 1 ? (uint32_t)((1ull << 32) / (uint32_t)a.tileCount) + 1u : 0u; a.splitMagic = a.kSplits > 1 ? (uint32_t)((1ull << 32) / (uint32_t)a.kSplits) + 1u : 0u;
-  if (g_bk == 0) {
+  if (mode == 0) {
     /* set-aligned schedule; compute units per XCD rounded down to a power of two (32 on this device) */
     int slots = units / XCDS; a.slotShift = 0; while ((2 << a.slotShift) <= slots) { ++a.slotShift; } slots = 1 << a.slotShift;
     a.pairShift = (paired && (a.groupCount & 1) == 0) ? 1 : 0; const int setTiles = a.tileCount << a.pairShift;
@@ -769,7 +777,7 @@ hipError_t launch_gram(hipStream_t stream, GramArgs& a, int epi, int maxProducts
     if (a.exclusive) { return epi == EPI_MOD ? launch_ring<EPI_MOD, true>(stream, a) : launch_ring<EPI_I64, true>(stream, a); }
     return epi == EPI_MOD ? launch_ring<EPI_MOD, false>(stream, a) : launch_ring<EPI_I64, false>(stream, a);
   }
-  if (g_bk == 2) {
+  if (mode == 2) {
     if (a.exclusive) { return epi == EPI_MOD ? launch_dma<EPI_MOD, true>(stream, a) : launch_dma<EPI_I64, true>(stream, a); }
     return epi == EPI_MOD ? launch_dma<EPI_MOD, false>(stream, a) : launch_dma<EPI_I64, false>(stream, a);
   }
