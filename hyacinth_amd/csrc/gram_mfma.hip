@@ -488,24 +488,35 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_ring_kernel(const GramArgs 
   }
 
   /* Two request streams run through the same sequence of (pair, slab) positions: the lane units and, half a slab behind,
-   * the A units.  Each keeps the position it requested last; all of it is wave-uniform scalar state. */
-  const int iters = slabs * grp.pairCount;
-  const uint32_t pp0 = args.pairs[grp.pairBegin];
-  int pairL = 0, slabL = 0, issuedL = 1, pairA = 0, slabA = 0, issuedA = 1; uint32_t nextL = pp0, nextA = pp0;
+   * the A units.  Each keeps the position it requested last as wave-uniform scalar state: slabs still to request in the
+   * whole item and in the current pair, the pair, the address of the slab.  Past the last slab a stream stays where it
+   * is (the ring is filled two slabs ahead, so the last iterations request the last slab again).  The common step is
+   * branch-free scalar arithmetic; only the change of pair, once in `slabs` steps, takes a branch and a load. */
+  const int iters = __builtin_amdgcn_readfirstlane(slabs * (int)grp.pairCount);
+  const int lastPair = __builtin_amdgcn_readfirstlane((int)grp.pairCount - 1), pairBegin = __builtin_amdgcn_readfirstlane((int)grp.pairBegin);
+  const int perPair = __builtin_amdgcn_readfirstlane(slabs);
+  const uint32_t pp0 = args.pairs[pairBegin];
   const int64_t rowsLane = (int64_t)y0 * args.ldb + k0, rowsA = (int64_t)x0 * args.ldb + k0;
   const int8_t* baseLane = args.panels + (int64_t)(pp0 & 0xffffu) * args.panelStride + rowsLane;
   const int8_t* baseA = args.panels + (int64_t)(pp0 >> 16) * args.panelStride + rowsA;
-  auto peekL = [&]() { const int q = pairL + 1 < (int)grp.pairCount ? pairL + 1 : (int)grp.pairCount - 1; nextL = args.pairs[grp.pairBegin + q]; };
-  auto peekA = [&]() { const int q = pairA + 1 < (int)grp.pairCount ? pairA + 1 : (int)grp.pairCount - 1; nextA = args.pairs[grp.pairBegin + q]; };
+  int leftL = iters - 1, inPairL = perPair - 1, pairL = 0, leftA = iters - 1, inPairA = perPair - 1, pairA = 0;
+  /* (the step is written without booleans that outlive a basic block: such a condition is held as a lane mask and
+   * drags the counters into vector registers and vector compares) */
   auto advanceL = [&]() {
-    const bool more = issuedL < iters, wrap = more && (slabL + 1 == slabs);
-    const int8_t* cand = args.panels + (int64_t)(nextL & 0xffffu) * args.panelStride + rowsLane;
-    baseLane = wrap ? cand : baseLane + (more ? RING_K : 0); slabL = wrap ? 0 : slabL + (more ? 1 : 0); pairL += wrap ? 1 : 0; issuedL += more ? 1 : 0;
+    const int go = leftL < 1 ? leftL : 1;                      /* 0 once every slab has been requested */
+    baseLane += go * RING_K; leftL -= go; inPairL -= go;
+    if (__builtin_expect(inPairL < 0, 0)) {
+      pairL = pairL + 1 < lastPair ? pairL + 1 : lastPair; inPairL = perPair - 1;
+      baseLane = args.panels + (int64_t)(args.pairs[pairBegin + pairL] & 0xffffu) * args.panelStride + rowsLane;
+    }
   };
   auto advanceA = [&]() {
-    const bool more = issuedA < iters, wrap = more && (slabA + 1 == slabs);
-    const int8_t* cand = args.panels + (int64_t)(nextA >> 16) * args.panelStride + rowsA;
-    baseA = wrap ? cand : baseA + (more ? RING_K : 0); slabA = wrap ? 0 : slabA + (more ? 1 : 0); pairA += wrap ? 1 : 0; issuedA += more ? 1 : 0;
+    const int go = leftA < 1 ? leftA : 1;
+    baseA += go * RING_K; leftA -= go; inPairA -= go;
+    if (__builtin_expect(inPairA < 0, 0)) {
+      pairA = pairA + 1 < lastPair ? pairA + 1 : lastPair; inPairA = perPair - 1;
+      baseA = args.panels + (int64_t)(args.pairs[pairBegin + pairA] >> 16) * args.panelStride + rowsA;
+    }
   };
   /* ring position of the next unit to fill (byte offset, wraps at RING_BYTES) */
   uint32_t fillOff = 0;
@@ -543,7 +554,7 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_ring_kernel(const GramArgs 
   /* prologue: slabs 0 and 1 requested in full (eight units); slab 0 landed and published; its first fragments requested */
   #pragma unroll
   for (int s0 = 0; s0 < 2; ++s0) {
-    if (s0) { peekL(); advanceL(); peekA(); advanceA(); }
+    if (s0) { advanceL(); advanceA(); }
     #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const uint32_t u = next_unit();
@@ -557,7 +568,7 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_ring_kernel(const GramArgs 
       for (int r = 0; r < 4; ++r) { fill_a(h, r, u); }
     }
   }
-  peekL(); advanceL();                     /* lane stream: next to request is slab 2; A stream stays on slab 1 until the first barrier */
+  advanceL();                              /* lane stream: next to request is slab 2; A stream stays on slab 1 until the first barrier */
   asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
   __syncthreads();
   uint32_t slabOff = 0;                    /* ring offset of the first unit of the slab being contracted */
@@ -573,7 +584,6 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_ring_kernel(const GramArgs 
     const uint32_t lu = unit_offset(slabOff, wy), au = unit_offset(slabOff, 2 + wx);
     uint32_t nextOff = slabOff + 4u * RING_UNIT_BYTES; nextOff = nextOff >= (uint32_t)RING_BYTES ? nextOff - (uint32_t)RING_BYTES : nextOff;
     const uint32_t nlu = unit_offset(nextOff, wy), nau = unit_offset(nextOff, 2 + wx);
-    peekL(); peekA();
     /* K step 0: MFMAs on set 0, fragments of step 1 into set 1, lane unit 0 of slab it + 2 */
     { const uint32_t u = next_unit();
       run(IC<0>{}, IC<4>{}, IC<0>{}, IC<0>{}, IC<4>{}, IC<1>{}, IC<1>{}, lu, au); fill_lane(0, 0, u); __builtin_amdgcn_sched_barrier(0);
