@@ -534,21 +534,6 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_ring_kernel(const GramArgs 
     if (i < 4) { fl[set][i] = *reinterpret_cast<const v4i*>(lds + laneUnit + rowOff + i * 32 * RING_K + kOff[kk]); }
     else { fa[set][i - 4] = *reinterpret_cast<const v4i*>(lds + aUnit + rowOff + (i - 4) * 32 * RING_K + kOff[kk]); }
   };
-  auto mm = [&](int n, int set) { const int a = n >> 2, b = n & 3; acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[set][a], fl[set][b], acc[a][b], 0, 0, 0); };
-  /* a run of MFMAs with fragment reads paired to the first of them, closed for the scheduler */
-  auto run = [&](auto mmFirst_, auto mmCount_, auto mmSet_, auto rdFirst_, auto rdCount_, auto rdSet_, auto rdKk_, uint32_t laneUnit, uint32_t aUnit) {
-    constexpr int mmFirst = decltype(mmFirst_)::value, mmCount = decltype(mmCount_)::value, mmSet = decltype(mmSet_)::value;
-    constexpr int rdFirst = decltype(rdFirst_)::value, rdCount = decltype(rdCount_)::value, rdSet = decltype(rdSet_)::value, rdKk = decltype(rdKk_)::value;
-    #pragma unroll
-    for (int i = 0; i < rdCount; ++i) { rd(rdFirst + i, rdSet, rdKk, laneUnit, aUnit); }
-    #pragma unroll
-    for (int n = 0; n < mmCount; ++n) { mm(mmFirst + n, mmSet); }
-    #pragma unroll
-    for (int i = 0; i < rdCount; ++i) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); }
-    if constexpr (mmCount > rdCount) { __builtin_amdgcn_sched_group_barrier(0x008, mmCount - rdCount, 0); }
-    __builtin_amdgcn_sched_barrier(0);
-  };
-  /* a whole K step whose loads are spread four MFMAs apart: reads under the first eight MFMAs */
   auto unit_offset = [&](uint32_t slabOff, int unit) { uint32_t o = slabOff + (uint32_t)unit * RING_UNIT_BYTES; return o >= (uint32_t)RING_BYTES ? o - (uint32_t)RING_BYTES : o; };
 
   /* prologue: slabs 0 and 1 requested in full (eight units); slab 0 landed and published; its first fragments requested */
@@ -580,46 +565,72 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_ring_kernel(const GramArgs 
   __builtin_amdgcn_s_waitcnt(0xC07F);
   __builtin_amdgcn_sched_barrier(0);
 
-  for (int it = 0; it < iters; ++it) {
-    const uint32_t lu = unit_offset(slabOff, wy), au = unit_offset(slabOff, 2 + wx);
-    uint32_t nextOff = slabOff + 4u * RING_UNIT_BYTES; nextOff = nextOff >= (uint32_t)RING_BYTES ? nextOff - (uint32_t)RING_BYTES : nextOff;
-    const uint32_t nlu = unit_offset(nextOff, wy), nau = unit_offset(nextOff, 2 + wx);
-    /* K step 0: MFMAs on set 0, fragments of step 1 into set 1, lane unit 0 of slab it + 2 */
-    { const uint32_t u = next_unit();
-      run(IC<0>{}, IC<4>{}, IC<0>{}, IC<0>{}, IC<4>{}, IC<1>{}, IC<1>{}, lu, au); fill_lane(0, 0, u); __builtin_amdgcn_sched_barrier(0);
-      run(IC<4>{}, IC<4>{}, IC<0>{}, IC<4>{}, IC<4>{}, IC<1>{}, IC<1>{}, lu, au); fill_lane(0, 1, u); __builtin_amdgcn_sched_barrier(0);
-      run(IC<8>{}, IC<4>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<1>{}, IC<1>{}, lu, au); fill_lane(0, 2, u); __builtin_amdgcn_sched_barrier(0);
-      run(IC<12>{}, IC<4>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<1>{}, IC<1>{}, lu, au); fill_lane(0, 3, u); __builtin_amdgcn_sched_barrier(0); }
-    /* K step 1: MFMAs on set 1, fragments of step 2 into set 0, lane unit 1 of slab it + 2 */
-    { const uint32_t u = next_unit();
-      run(IC<0>{}, IC<4>{}, IC<1>{}, IC<0>{}, IC<4>{}, IC<0>{}, IC<2>{}, lu, au); fill_lane(1, 0, u); __builtin_amdgcn_sched_barrier(0);
-      run(IC<4>{}, IC<4>{}, IC<1>{}, IC<4>{}, IC<4>{}, IC<0>{}, IC<2>{}, lu, au); fill_lane(1, 1, u); __builtin_amdgcn_sched_barrier(0);
-      run(IC<8>{}, IC<4>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<2>{}, lu, au); fill_lane(1, 2, u); __builtin_amdgcn_sched_barrier(0);
-      run(IC<12>{}, IC<4>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<2>{}, lu, au); fill_lane(1, 3, u); __builtin_amdgcn_sched_barrier(0); }
-    /* K step 2: MFMAs on set 0, fragments of step 3 into set 1, no loads */
-    run(IC<0>{}, IC<4>{}, IC<0>{}, IC<0>{}, IC<4>{}, IC<1>{}, IC<3>{}, lu, au);
-    run(IC<4>{}, IC<8>{}, IC<0>{}, IC<4>{}, IC<4>{}, IC<1>{}, IC<3>{}, lu, au);
-    /* slab it + 1 has landed (own loads: only the eight lane loads above may be outstanding) and every wave has read
-     * its last fragments of slab it: publish, release */
-    asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-    __syncthreads();
-    __builtin_amdgcn_sched_barrier(0);
-    run(IC<12>{}, IC<4>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<1>{}, IC<3>{}, lu, au);
-    advanceL(); advanceA();
-    __builtin_amdgcn_sched_barrier(0);
-    /* K step 3: MFMAs on set 1, first fragments of slab it + 1 into set 0, both A units of slab it + 2 */
-    { const uint32_t u0 = next_unit(), u1 = next_unit();
-      run(IC<0>{}, IC<2>{}, IC<1>{}, IC<0>{}, IC<2>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(0, 0, u0); __builtin_amdgcn_sched_barrier(0);
-      run(IC<2>{}, IC<2>{}, IC<1>{}, IC<2>{}, IC<2>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(0, 1, u0); __builtin_amdgcn_sched_barrier(0);
-      run(IC<4>{}, IC<2>{}, IC<1>{}, IC<4>{}, IC<2>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(0, 2, u0); __builtin_amdgcn_sched_barrier(0);
-      run(IC<6>{}, IC<2>{}, IC<1>{}, IC<6>{}, IC<2>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(0, 3, u0); __builtin_amdgcn_sched_barrier(0);
-      run(IC<8>{}, IC<2>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(1, 0, u1); __builtin_amdgcn_sched_barrier(0);
-      run(IC<10>{}, IC<2>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(1, 1, u1); __builtin_amdgcn_sched_barrier(0);
-      run(IC<12>{}, IC<2>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(1, 2, u1); __builtin_amdgcn_sched_barrier(0);
-      run(IC<14>{}, IC<2>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(1, 3, u1); __builtin_amdgcn_sched_barrier(0); }
-    __builtin_amdgcn_s_waitcnt(0xC07F);   /* lgkmcnt(0): the fragments of the next slab were requested eight MFMAs ago */
-    slabOff = nextOff;
-  }
+  /* The loop in three versions, chosen once per wavefront.  In a diagonal tile only y <= x is kept: of the 32x32 blocks
+   * (a, b) of wavefront (wy, wx), those with 4 wy + b > 4 wx + a lie wholly below the diagonal.  Version 1 (wy == wx)
+   * leaves out its six such blocks, version 2 (wy > wx) all sixteen: that wavefront only requests its share of the ring
+   * and keeps the barriers.  The device runs this kernel at its power limit, so MFMAs not issued turn into clock. */
+  auto contract = [&](auto mode_) {
+    constexpr int MODE = decltype(mode_)::value;
+    auto kept = [](int n) constexpr { return MODE == 0 || (MODE == 1 && (n & 3) <= (n >> 2)); };
+    auto mm = [&](int n, int set) { const int a = n >> 2, b = n & 3; acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[set][a], fl[set][b], acc[a][b], 0, 0, 0); };
+    /* a run of MFMAs with fragment reads paired to the first of them, closed for the scheduler */
+    auto run = [&](auto mmFirst_, auto mmCount_, auto mmSet_, auto rdFirst_, auto rdCount_, auto rdSet_, auto rdKk_, uint32_t laneUnit, uint32_t aUnit) {
+      constexpr int mmFirst = decltype(mmFirst_)::value, mmCount = decltype(mmCount_)::value, mmSet = decltype(mmSet_)::value;
+      constexpr int rdFirst = decltype(rdFirst_)::value, rdCount = MODE == 2 ? 0 : decltype(rdCount_)::value, rdSet = decltype(rdSet_)::value, rdKk = decltype(rdKk_)::value;
+      int keptCount = 0;
+      #pragma unroll
+      for (int i = 0; i < rdCount; ++i) { rd(rdFirst + i, rdSet, rdKk, laneUnit, aUnit); }
+      #pragma unroll
+      for (int n = 0; n < mmCount; ++n) { if (kept(mmFirst + n)) { mm(mmFirst + n, mmSet); ++keptCount; } }
+      #pragma unroll
+      for (int i = 0; i < rdCount; ++i) { if (i < keptCount) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); } __builtin_amdgcn_sched_group_barrier(0x100, 1, 0); }
+      #pragma unroll
+      for (int n = rdCount; n < mmCount; ++n) { if (n < keptCount) { __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); } }
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    for (int it = 0; it < iters; ++it) {
+      const uint32_t lu = unit_offset(slabOff, wy), au = unit_offset(slabOff, 2 + wx);
+      uint32_t nextOff = slabOff + 4u * RING_UNIT_BYTES; nextOff = nextOff >= (uint32_t)RING_BYTES ? nextOff - (uint32_t)RING_BYTES : nextOff;
+      const uint32_t nlu = unit_offset(nextOff, wy), nau = unit_offset(nextOff, 2 + wx);
+      /* K step 0: MFMAs on set 0, fragments of step 1 into set 1, lane unit 0 of slab it + 2 */
+      { const uint32_t u = next_unit();
+        run(IC<0>{}, IC<4>{}, IC<0>{}, IC<0>{}, IC<4>{}, IC<1>{}, IC<1>{}, lu, au); fill_lane(0, 0, u); __builtin_amdgcn_sched_barrier(0);
+        run(IC<4>{}, IC<4>{}, IC<0>{}, IC<4>{}, IC<4>{}, IC<1>{}, IC<1>{}, lu, au); fill_lane(0, 1, u); __builtin_amdgcn_sched_barrier(0);
+        run(IC<8>{}, IC<4>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<1>{}, IC<1>{}, lu, au); fill_lane(0, 2, u); __builtin_amdgcn_sched_barrier(0);
+        run(IC<12>{}, IC<4>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<1>{}, IC<1>{}, lu, au); fill_lane(0, 3, u); __builtin_amdgcn_sched_barrier(0); }
+      /* K step 1: MFMAs on set 1, fragments of step 2 into set 0, lane unit 1 of slab it + 2 */
+      { const uint32_t u = next_unit();
+        run(IC<0>{}, IC<4>{}, IC<1>{}, IC<0>{}, IC<4>{}, IC<0>{}, IC<2>{}, lu, au); fill_lane(1, 0, u); __builtin_amdgcn_sched_barrier(0);
+        run(IC<4>{}, IC<4>{}, IC<1>{}, IC<4>{}, IC<4>{}, IC<0>{}, IC<2>{}, lu, au); fill_lane(1, 1, u); __builtin_amdgcn_sched_barrier(0);
+        run(IC<8>{}, IC<4>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<2>{}, lu, au); fill_lane(1, 2, u); __builtin_amdgcn_sched_barrier(0);
+        run(IC<12>{}, IC<4>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<2>{}, lu, au); fill_lane(1, 3, u); __builtin_amdgcn_sched_barrier(0); }
+      /* K step 2: MFMAs on set 0, fragments of step 3 into set 1, no loads */
+      run(IC<0>{}, IC<4>{}, IC<0>{}, IC<0>{}, IC<4>{}, IC<1>{}, IC<3>{}, lu, au);
+      run(IC<4>{}, IC<8>{}, IC<0>{}, IC<4>{}, IC<4>{}, IC<1>{}, IC<3>{}, lu, au);
+      /* slab it + 1 has landed (own loads: only the eight lane loads above may be outstanding) and every wave has read
+       * its last fragments of slab it: publish, release */
+      asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+      __syncthreads();
+      __builtin_amdgcn_sched_barrier(0);
+      run(IC<12>{}, IC<4>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<1>{}, IC<3>{}, lu, au);
+      advanceL(); advanceA();
+      __builtin_amdgcn_sched_barrier(0);
+      /* K step 3: MFMAs on set 1, first fragments of slab it + 1 into set 0, both A units of slab it + 2 */
+      { const uint32_t u0 = next_unit(), u1 = next_unit();
+        run(IC<0>{}, IC<2>{}, IC<1>{}, IC<0>{}, IC<2>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(0, 0, u0); __builtin_amdgcn_sched_barrier(0);
+        run(IC<2>{}, IC<2>{}, IC<1>{}, IC<2>{}, IC<2>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(0, 1, u0); __builtin_amdgcn_sched_barrier(0);
+        run(IC<4>{}, IC<2>{}, IC<1>{}, IC<4>{}, IC<2>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(0, 2, u0); __builtin_amdgcn_sched_barrier(0);
+        run(IC<6>{}, IC<2>{}, IC<1>{}, IC<6>{}, IC<2>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(0, 3, u0); __builtin_amdgcn_sched_barrier(0);
+        run(IC<8>{}, IC<2>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(1, 0, u1); __builtin_amdgcn_sched_barrier(0);
+        run(IC<10>{}, IC<2>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(1, 1, u1); __builtin_amdgcn_sched_barrier(0);
+        run(IC<12>{}, IC<2>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(1, 2, u1); __builtin_amdgcn_sched_barrier(0);
+        run(IC<14>{}, IC<2>{}, IC<1>{}, IC<0>{}, IC<0>{}, IC<0>{}, IC<0>{}, nlu, nau); fill_a(1, 3, u1); __builtin_amdgcn_sched_barrier(0); }
+      __builtin_amdgcn_s_waitcnt(0xC07F);   /* lgkmcnt(0): the fragments of the next slab were requested eight MFMAs ago */
+      slabOff = nextOff;
+    }
+  };
+  const int mode = (ta == tb) ? (wy > wx ? 2 : (wy == wx ? 1 : 0)) : 0;
+  if (mode == 0) { contract(IC<0>{}); } else if (mode == 1) { contract(IC<1>{}); } else { contract(IC<2>{}); }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   /* no direct load may still be writing LDS when the workgroup ends */
 
   constexpr int aBegin = 0, aEnd = 4;
