@@ -633,8 +633,60 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_ring_kernel(const GramArgs 
   if (mode == 0) { contract(IC<0>{}); } else if (mode == 1) { contract(IC<1>{}); } else { contract(IC<2>{}); }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   /* no direct load may still be writing LDS when the workgroup ends */
 
-  constexpr int aBegin = 0, aEnd = 4;
-  HYK_GRAM_EPILOGUE(EXCL)
+  /* Epilogue: the same entries, values and order of operations per entry as HYK_GRAM_EPILOGUE, with everything that is
+   * uniform over the workgroup decided once.  Lane dimension j <-> y (contiguous in the packed triangle), register
+   * dimension i <-> x; register r of a block is row xb + 8 (r / 4) + r % 4, so the packed index runs along with
+   * tri(x + s) - tri(x) = s x + s (s + 1) / 2.  A signed sum w is reduced as (w + bias) mod m with bias the smallest
+   * multiple of m that is >= 2^31: w + bias is non-negative and below 2^32 for every sum the K cap allows (for m = 256
+   * a wrap is harmless), so one unsigned reduction gives the canonical residue.  Blocks of a diagonal tile wholly below
+   * the diagonal are skipped, those wholly above need no test.  CHECKED: the tile touches the matrix edge or the diagonal.
+   * SIMPLE: the group adds its sums unchanged to its real plane only (every real launch, the paired complex residues). */
+  if constexpr (EPI == EPI_I64) {   /* 64-bit sums: the shared epilogue (its values and addresses leave no room for more) */
+    HYK_GRAM_EPILOGUE(EXCL)
+    return;
+  }
+  const bool inner = (ta != tb) && (x0 + TILE <= args.N) && (y0 + TILE <= args.N);
+  const bool simple = grp.mulRe == 1u && grp.mulIm == 0u;
+  uint32_t bias = 0u;
+  if constexpr (EPI == EPI_MOD) { const uint32_t over = 0x80000000u % grp.m; bias = 0x80000000u + (over ? grp.m - over : 0u); }
+  auto emit = [&](auto checked_, auto simple_) {
+    constexpr bool CHECKED = decltype(checked_)::value != 0, SIMPLE = decltype(simple_)::value != 0;
+    #pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      #pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        __builtin_amdgcn_sched_barrier(0);   /* one 32x32 block at a time: keeps the accumulator copies out of scratch */
+        bool diagBlock = false;
+        if constexpr (CHECKED) { if (ta == tb) { const int by = 4 * wy + b, bx = 4 * wx + a; if (by > bx) { continue; } diagBlock = by == bx; } }
+        const int y = y0 + wy * WAVE_TILE + b * 32 + (lane & 31);
+        int x = x0 + wx * WAVE_TILE + a * 32 + ((lane >> 5) << 2);
+        int64_t e = hyk::tri_index(y, x);
+        #pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          if (r) { if (r & 3) { e += x + 1; x += 1; } else { e += 5 * (int64_t)x + 15; x += 5; } }
+          bool ok = true;
+          if constexpr (CHECKED) { ok = x < args.N && y < args.N && (!diagBlock || y <= x); }
+          if (ok) {
+            const int32_t w = acc[a][b][r];
+            if constexpr (EPI == EPI_MOD) {
+              uint32_t* dst = reinterpret_cast<uint32_t*>(args.acc);
+              const uint32_t v = hyk::reduce_u32((uint32_t)w + bias, grp.m, grp.d);
+              if constexpr (SIMPLE) {
+                uint32_t* at = &dst[(int64_t)grp.planeRe * args.planeStride + e];
+                if constexpr (EXCL) { *at = v; } else { atomicAdd(at, v); }
+              } else {
+                if (grp.mulRe) { uint32_t* at = &dst[(int64_t)grp.planeRe * args.planeStride + e]; const uint32_t t = grp.mulRe == 1u ? v : hyk::reduce_u32(v * grp.mulRe, grp.m, grp.d); if constexpr (EXCL) { *at = t; } else { atomicAdd(at, t); } }
+                if (grp.mulIm) { uint32_t* at = &dst[(int64_t)grp.planeIm * args.planeStride + e]; const uint32_t t = grp.mulIm == 1u ? v : hyk::reduce_u32(v * grp.mulIm, grp.m, grp.d); if constexpr (EXCL) { *at = t; } else { atomicAdd(at, t); } }
+              }
+            }
+          }
+        }
+      }
+    }
+  };
+  if (mode == 2) { /* every block of this wavefront lies below the diagonal */ }
+  else if (inner) { if (simple) { emit(IC<0>{}, IC<1>{}); } else { emit(IC<0>{}, IC<0>{}); } }
+  else { if (simple) { emit(IC<1>{}, IC<1>{}); } else { emit(IC<1>{}, IC<0>{}); } }
 }
 
 /* ------------------------------------------------------------------ CRT reconstruction */
