@@ -571,8 +571,11 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_ring_kernel(const GramArgs 
    * and keeps the barriers.  The device runs this kernel at its power limit, so MFMAs not issued turn into clock. */
   auto contract = [&](auto mode_) {
     constexpr int MODE = decltype(mode_)::value;
-    auto kept = [](int n) constexpr { return MODE == 0 || (MODE == 1 && (n & 3) <= (n >> 2)); };
-    auto mm = [&](int n, int set) { const int a = n >> 2, b = n & 3; acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[set][a], fl[set][b], acc[a][b], 0, 0, 0); };
+    /* MFMA n of a K step works on block (a, b) = (n / 4, n % 4 run back and forth): between consecutive MFMAs only one
+     * of the two operands changes */
+    auto b_of = [](int n) constexpr { return ((n >> 2) & 1) ? 3 - (n & 3) : (n & 3); };
+    auto kept = [b_of](int n) constexpr { return MODE == 0 || (MODE == 1 && b_of(n) <= (n >> 2)); };
+    auto mm = [&](int n, int set) { const int a = n >> 2, b = b_of(n); acc[a][b] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[set][a], fl[set][b], acc[a][b], 0, 0, 0); };
     /* a run of MFMAs with fragment reads paired to the first of them, closed for the scheduler */
     auto run = [&](auto mmFirst_, auto mmCount_, auto mmSet_, auto rdFirst_, auto rdCount_, auto rdSet_, auto rdKk_, uint32_t laneUnit, uint32_t aUnit) {
       constexpr int mmFirst = decltype(mmFirst_)::value, mmCount = decltype(mmCount_)::value, mmSet = decltype(mmSet_)::value;
