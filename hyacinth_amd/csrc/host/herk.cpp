@@ -74,6 +74,11 @@ const void* row_ptr(const Ctx& c, int64_t row) { return c.A + row * (int64_t)hyh
 
 int32_t crt_panels(int32_t order, int32_t Complex) { return Complex ? 2 * order + std::max(0, order - HYK_CRT_CPLX_SPLIT) : order; }
 
+/* Leading dimension of the panel rows for a capacity of `cap` K-bytes: a row length that is a multiple of 4096 bytes gets
+ * 256 more, so that the rows of a tile (one cache line each per K slab) do not all fall on the same few cache sets and
+ * memory channels. */
+int64_t panel_ld(int64_t cap) { return cap + ((cap % 4096 == 0) ? 256 : 0); }
+
 /* a list of row runs [first, first + count) of A, quantized back to back into one compact panel set and contracted */
 struct Run { int64_t first; int32_t count; };
 
@@ -86,19 +91,20 @@ void limb_bucket(Ctx& c, const std::vector<Run>& runs, int32_t order) {
   const int32_t groups = c.Complex ? 3 : 1; const int64_t rowBytes = (int64_t)c.N * order * groups;
   int64_t cap = std::max<int64_t>(8192, (int64_t)(kPanelBudget / (size_t)rowBytes) / 128 * 128); cap = std::min<int64_t>(cap, (rows + 127) / 128 * 128);
   const size_t wsBytes = hykGramWorkspaceBytes(HYK_GRAM_LIMBS, c.Complex, c.N, order);
-  hyh::Scratch W(c.h, (size_t)cap * (size_t)rowBytes), ws(c.h, wsBytes);
+  const int64_t ld = panel_ld(cap);
+  hyh::Scratch W(c.h, (size_t)ld * (size_t)rowBytes), ws(c.h, wsBytes);
   HYH_KERNEL(hykGramWorkspaceClear(c.s, ws.p, wsBytes));
   int32_t filled = 0;
   auto flush = [&]() {
     if (filled <= 0) { return; } const int32_t K = hyh::round_up(filled, 128);
-    HYH_KERNEL(hykZeroRows(c.s, W.as<int8_t>(), cap, (int64_t)c.N * order * groups, filled, K));
-    HYH_KERNEL(hykGramLimbs(c.s, c.Complex, c.N, order, W.as<int8_t>(), cap, K, c.beta, c.orderC, c.C, ws.p)); c.beta = 1; log_gemm(c, "limbs", K, order); filled = 0;
+    HYH_KERNEL(hykZeroRows(c.s, W.as<int8_t>(), ld, (int64_t)c.N * order * groups, filled, K));
+    HYH_KERNEL(hykGramLimbs(c.s, c.Complex, c.N, order, W.as<int8_t>(), ld, K, c.beta, c.orderC, c.C, ws.p)); c.beta = 1; log_gemm(c, "limbs", K, order); filled = 0;
   };
   for (const Run& r : runs) {
     int64_t first = r.first; int32_t left = r.count;
     while (left > 0) {
       const int32_t take = (int32_t)std::min<int64_t>(left, cap - filled);
-      HYH_KERNEL(hykQuantizeLimbs(c.s, take, c.N, order, c.Atype, row_ptr(c, first), c.lda, c.vexp, W.as<int8_t>() + filled, cap));
+      HYH_KERNEL(hykQuantizeLimbs(c.s, take, c.N, order, c.Atype, row_ptr(c, first), c.lda, c.vexp, W.as<int8_t>() + filled, ld));
       filled += take; first += take; left -= take; if (filled == cap) { flush(); }
     }
   }
@@ -111,19 +117,20 @@ void crt_bucket(Ctx& c, const std::vector<Run>& runs, int32_t order, int32_t chu
   int64_t cap = std::max<int64_t>(8192, (int64_t)(kPanelBudget / (size_t)rowBytes) / 128 * 128);
   cap = std::min<int64_t>(cap, std::max(128, chunkRows / 128 * 128)); cap = std::min<int64_t>(cap, (rows + 127) / 128 * 128);
   const size_t wsBytes = hykGramWorkspaceBytes(HYK_GRAM_CRT, c.Complex, c.N, order);
-  hyh::Scratch W(c.h, (size_t)cap * (size_t)rowBytes), ws(c.h, wsBytes);
+  const int64_t ld = panel_ld(cap);
+  hyh::Scratch W(c.h, (size_t)ld * (size_t)rowBytes), ws(c.h, wsBytes);
   HYH_KERNEL(hykGramWorkspaceClear(c.s, ws.p, wsBytes));
   int32_t filled = 0;
   auto flush = [&]() {
     if (filled <= 0) { return; } const int32_t K = hyh::round_up(filled, 128);
-    HYH_KERNEL(hykZeroRows(c.s, W.as<int8_t>(), cap, (int64_t)c.N * panels, filled, K));
-    HYH_KERNEL(hykGramCrt(c.s, c.Complex, c.N, order, W.as<int8_t>(), cap, K, c.beta, c.orderC, c.C, ws.p)); c.beta = 1; log_gemm(c, "crt", K, order); filled = 0;
+    HYH_KERNEL(hykZeroRows(c.s, W.as<int8_t>(), ld, (int64_t)c.N * panels, filled, K));
+    HYH_KERNEL(hykGramCrt(c.s, c.Complex, c.N, order, W.as<int8_t>(), ld, K, c.beta, c.orderC, c.C, ws.p)); c.beta = 1; log_gemm(c, "crt", K, order); filled = 0;
   };
   for (const Run& r : runs) {
     int64_t first = r.first; int32_t left = r.count;
     while (left > 0) {
       const int32_t take = (int32_t)std::min<int64_t>(left, cap - filled);
-      HYH_KERNEL(hykQuantizeCrt(c.s, take, c.N, order, c.Atype, row_ptr(c, first), c.lda, c.vexp, W.as<int8_t>() + filled, cap, maxBits));
+      HYH_KERNEL(hykQuantizeCrt(c.s, take, c.N, order, c.Atype, row_ptr(c, first), c.lda, c.vexp, W.as<int8_t>() + filled, ld, maxBits));
       filled += take; first += take; left -= take; if (filled == cap) { flush(); }
     }
   }
