@@ -24,7 +24,7 @@ HBM_PEAK_GBS = 8000.0     # MI355X HBM3E peak, 8 TB/s
 
 # HBM bytes per launch of the contraction kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script
 # (profiles/gram_ring_kernel_target_hbm_traffic.md), each scaled by what the counter reads for copy_kernel's known 1 GiB.
-MEASURED_TRAFFIC = {("target", 0): 6.21e9 + 0.12e9}
+MEASURED_TRAFFIC = {("target", 0): 5.65e9 + 0.12e9}
 
 WORKLOADS = {
     # name: (type, opA, M, N, K, eps, algorithm, description)

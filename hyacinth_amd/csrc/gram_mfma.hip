@@ -453,8 +453,10 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_ring_kernel(const GramArgs 
     t = (args.mainRounds << args.slotShift) + (slot - inRound * args.leftover);
   }
   const int sg = divide(set, args.splitMagic), ks = set - sg * args.kSplits, g = (sg << args.pairShift) + (t & ((1 << args.pairShift) - 1)); t >>= args.pairShift;
-  int tb = 0; while ((tb + 1) * (tb + 2) / 2 <= t) { ++tb; }
-  const int ta = t - tb * (tb + 1) / 2;
+  /* tiles row by row, (ta, ta), (ta, ta + 1), ..., (ta, nT - 1): the tiles at the end of this order, which the schedule
+   * packs into the left-over rounds, form the smallest triangle in the corner and share the fewest row blocks */
+  int ta = 0, rowStart = 0; while (rowStart + (args.nT - ta) <= t) { rowStart += args.nT - ta; ++ta; }
+  const int tb = ta + (t - rowStart);
   const GramGroup grp = args.groups[g];
   const int k0 = ks * args.kLen, kEnd = (k0 + args.kLen) < args.K ? (k0 + args.kLen) : args.K, slabs = (kEnd - k0) / RING_K;
   const int y0 = ta * TILE, x0 = tb * TILE;
