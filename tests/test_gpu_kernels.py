@@ -142,6 +142,29 @@ def test_gram_extreme_values_and_long_k(gl, oracle):
     assert np.array_equal(gl.gram("crt", 0, N, 2, panels, 2), want)
 
 
+def test_gram_rows_too_long_for_tile_offsets(gl, oracle):
+    """Panel rows so long that the 256 rows of a tile do not fit 32-bit byte offsets: the launch takes the register-staged
+    kernel and gives the same bits as the compact layout."""
+    import torch
+    import hyacinth_amd as ha
+    from gpu_util import ptr, stream, sync, host, zeros, check, DEV
+    rng = np.random.default_rng(41)
+    N, K, order, orderC = 5, 640, 2, 2
+    ldb = 16_900_096                               # 255 * ldb > 2^32, a multiple of 16
+    panels = random_panels(rng, order, N, K, 600, -125, 126)
+    want = oracle.i8herk("crt", 0, N, order, panels, 0, orderC)
+    wide = torch.zeros((order, N, ldb), dtype=torch.int8, device=DEV)
+    wide[:, :, :K] = torch.from_numpy(panels).to(DEV)
+    T = N * (N + 1) // 2
+    Cd = zeros(8 * orderC * T)
+    wsb = gl.L.hykGramWorkspaceBytes(ha.GRAM_CRT, 0, N, order)
+    ws = torch.zeros(int(wsb), dtype=torch.uint8, device=DEV)
+    print("gram crt, ldb", ldb, flush=True)
+    check(gl.L.hykGramCrt(stream(), 0, N, order, ptr(wide), ldb, K, 0, orderC, ptr(Cd), ptr(ws)))
+    sync()
+    assert np.array_equal(host(Cd, np.uint64), want)
+
+
 @pytest.mark.parametrize("slab", [0, 2, 64, 128])
 @pytest.mark.parametrize("cplx,order,K,rows", [(0, 3, 640, 600), (1, 2, 1536, 1500), (0, 2, 4224, 4200)])
 def test_gram_kernel_variants(gl, oracle, slab, cplx, order, K, rows):
