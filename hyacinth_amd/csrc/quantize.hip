@@ -231,9 +231,10 @@ __device__ __forceinline__ void crt_cplx_f64_step(int32_t order, const double (&
       #pragma unroll
       for (int r = 0; r < Q_ROWS; ++r) {
         if constexpr (X < HYK_CRT_CPLX_SPLIT) {
-          const double ra = hyk::residue_f64(ar[r], K::sym), rb = hyk::residue_f64(ai[r], K::sym);   /* |ra|, |rb| <= m / 2 */
-          w0[r] = low_word(hyk::residue_f64(__builtin_fma(-K::im, rb, ra), K::stored));
-          w1[r] = low_word(hyk::residue_f64(__builtin_fma(K::im, rb, ra), K::stored)); w2[r] = 0u;
+          /* only the imaginary part is reduced first: |rb| <= m / 2, so re -+ iota rb is exact and stays below 2^51 */
+          const double rb = hyk::residue_f64(ai[r], K::sym);
+          w0[r] = low_word(hyk::residue_f64(__builtin_fma(-K::im, rb, ar[r]), K::stored));
+          w1[r] = low_word(hyk::residue_f64(__builtin_fma(K::im, rb, ar[r]), K::stored)); w2[r] = 0u;
         } else {
           w0[r] = low_word(hyk::residue_f64(ar[r] + ai[r], K::stored)); w1[r] = low_word(hyk::residue_f64(ar[r], K::stored)); w2[r] = low_word(hyk::residue_f64(ai[r], K::stored));
         }
