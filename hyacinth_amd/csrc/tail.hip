@@ -26,6 +26,45 @@ namespace {
 
 constexpr int T_THREADS = 256;
 
+/* value of lane `j` (the same j in every lane, known at compile time after unrolling) in every lane: two scalar
+ * register reads instead of a trip through the LDS crossbar */
+__device__ __forceinline__ double lane_value(double v, int j) {
+  const long long b = __double_as_longlong(v);
+  const unsigned lo = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)b, j), hi = (unsigned)__builtin_amdgcn_readlane((int)(unsigned)(b >> 32), j);
+  return __longlong_as_double((long long)(((unsigned long long)hi << 32) | lo));
+}
+__device__ __forceinline__ int lane_value(int v, int j) { return __builtin_amdgcn_readlane(v, j); }
+
+/* Sums NV values (a power of two, at most 64) over the wavefront with NV - 1 + 6 - log2(NV) exchanges instead of 6 NV: in
+ * the first log2(NV) steps a lane keeps one half of its values and trades the other half with its partner, so that it
+ * ends with one value.  Returns, in every lane, the sum of value index_of(lane): the low log2(NV) bits of the lane,
+ * reversed. */
+template <int NV>
+__device__ __forceinline__ double wave_sum_split(double (&v)[NV]) {
+  static_assert(NV >= 1 && NV <= 64 && (NV & (NV - 1)) == 0, "a power of two");
+  const int lane = threadIdx.x & 63;
+  int off = 1;
+  #pragma unroll
+  for (int n = NV; n > 1; n >>= 1, off <<= 1) {
+    const bool upper = (lane & off) != 0;
+    #pragma unroll
+    for (int i = 0; i < n / 2; ++i) {
+      const double keep = upper ? v[i + n / 2] : v[i], send = upper ? v[i] : v[i + n / 2];
+      v[i] = keep + __shfl_xor(send, off, 64);
+    }
+  }
+  double s = v[0];
+  #pragma unroll
+  for (; off < 64; off <<= 1) { s += __shfl_xor(s, off, 64); }
+  return s;
+}
+template <int NV> __device__ __forceinline__ int split_index(int lane) {
+  int idx = 0, half = NV >> 1;
+  #pragma unroll
+  for (int bit = 1; bit < NV; bit <<= 1, half >>= 1) { if (lane & bit) { idx += half; } }
+  return idx;
+}
+
 __device__ __forceinline__ double block_sum(double v, double* scratch) {
   for (int off = 32; off > 0; off >>= 1) { v += __shfl_xor(v, off, 64); }
   __syncthreads();
@@ -102,15 +141,20 @@ template <int NV, int THREADS, int HALF>
 __device__ __forceinline__ double block_sum_lanes(double (&v)[NV], double* red, int parity) {
   static_assert((THREADS / 64) * NV <= HALF, "a half holds one value per wavefront and summand");
   static_assert(NV <= 64, "one lane per summand");
-  #pragma unroll
-  for (int i = 0; i < NV; ++i) {
-    #pragma unroll
-    for (int off = 32; off > 0; off >>= 1) { v[i] += __shfl_xor(v[i], off, 64); }
-  }
   double* mine = red + parity * HALF;
-  if ((threadIdx.x & 63) == 0) {
+  if constexpr ((NV & (NV - 1)) == 0) {
+    const double part = wave_sum_split<NV>(v);
+    if ((threadIdx.x & 63) < NV) { mine[(threadIdx.x >> 6) * NV + split_index<NV>(threadIdx.x & 63)] = part; }
+  } else {
     #pragma unroll
-    for (int i = 0; i < NV; ++i) { mine[(threadIdx.x >> 6) * NV + i] = v[i]; }
+    for (int i = 0; i < NV; ++i) {
+      #pragma unroll
+      for (int off = 32; off > 0; off >>= 1) { v[i] += __shfl_xor(v[i], off, 64); }
+    }
+    if ((threadIdx.x & 63) == 0) {
+      #pragma unroll
+      for (int i = 0; i < NV; ++i) { mine[(threadIdx.x >> 6) * NV + i] = v[i]; }
+    }
   }
   __syncthreads();
   double s = 0.; const int lane = threadIdx.x & 63;
@@ -122,7 +166,7 @@ template <int NV, int THREADS, int HALF>
 __device__ __forceinline__ void block_sum_many(double (&v)[NV], double* red, int parity) {
   const double s = block_sum_lanes<NV, THREADS, HALF>(v, red, parity);
   #pragma unroll
-  for (int i = 0; i < NV; ++i) { v[i] = __shfl(s, i, 64); }
+  for (int i = 0; i < NV; ++i) { v[i] = lane_value(s, i); }
 }
 
 template <bool CPLX, int ROWS, int BC, bool FULL, int THREADS>
@@ -204,9 +248,9 @@ __global__ __launch_bounds__(THREADS) void jacobi_block_round_kernel(int32_t N, 
     for (int j = 0; j < BC; ++j) {
       const int fa = (j == 0) ? NC - 1 : (step + j) % (NC - 1), fb = (j == 0) ? step : (step - j + (NC - 1)) % (NC - 1);
       const int c0 = FULL ? (fa < fb ? fa : fb) : j, c1 = FULL ? (fa < fb ? fb : fa) : BC + (j + step) % BC;
-      if (__shfl((int)rotate, j, 64)) {
-        const double csj = __shfl(cs, j, 64), snj = __shfl(sn, j, 64), erj = __shfl(er, j, 64), shj = __shfl(shift, j, 64);
-        [[maybe_unused]] const double eij = CPLX ? __shfl(ei, j, 64) : 0.;
+      if (lane_value((int)rotate, j)) {
+        const double csj = lane_value(cs, j), snj = lane_value(sn, j), erj = lane_value(er, j), shj = lane_value(shift, j);
+        [[maybe_unused]] const double eij = CPLX ? lane_value(ei, j) : 0.;
         #pragma unroll
         for (int m = 0; m < ROWS; ++m) {
           if constexpr (CPLX) {
