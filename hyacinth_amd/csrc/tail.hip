@@ -17,6 +17,7 @@
  *
  * R arrives column-wise: Rt[c * ldr + k] = R[k, c] for physical column c.
  */
+#include <type_traits>
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 #include "hyk_common.h"
@@ -39,23 +40,54 @@ __device__ __forceinline__ int lane_value(int v, int j) { return __builtin_amdgc
  * the first log2(NV) steps a lane keeps one half of its values and trades the other half with its partner, so that it
  * ends with one value.  Returns, in every lane, the sum of value index_of(lane): the low log2(NV) bits of the lane,
  * reversed. */
+/* lane exchange inside a row of 16 lanes through the data-parallel primitives (no LDS round trip):
+ * CTRL 0xB1 / 0x4E: partner lane ^ 1 / lane ^ 2 (quad permutations); 0x124 / 0x128: lane - 4 / lane - 8 modulo 16 */
+template <int CTRL>
+__device__ __forceinline__ double row_exchange(double v) {
+  const long long b = __double_as_longlong(v);
+  const unsigned lo = (unsigned)__builtin_amdgcn_update_dpp(0, (int)(unsigned)b, CTRL, 0xf, 0xf, false);
+  const unsigned hi = (unsigned)__builtin_amdgcn_update_dpp(0, (int)(unsigned)(b >> 32), CTRL, 0xf, 0xf, false);
+  return __longlong_as_double((long long)(((unsigned long long)hi << 32) | lo));
+}
+/* partner at distance OFF (1, 2: exchange with lane ^ OFF; 4, 8: the value of lane - OFF modulo 16, which sums a row just
+ * as well and keeps the low bits of the lane; 16, 32: lane ^ OFF through the LDS crossbar) */
+template <int OFF>
+__device__ __forceinline__ double partner_value(double v) {
+  if constexpr (OFF == 1) { return row_exchange<0xB1>(v); }
+  else if constexpr (OFF == 2) { return row_exchange<0x4E>(v); }
+  else if constexpr (OFF == 4) { return row_exchange<0x124>(v); }
+  else if constexpr (OFF == 8) { return row_exchange<0x128>(v); }
+  else { return __shfl_xor(v, OFF, 64); }
+}
+
 template <int NV>
 __device__ __forceinline__ double wave_sum_split(double (&v)[NV]) {
   static_assert(NV >= 1 && NV <= 64 && (NV & (NV - 1)) == 0, "a power of two");
   const int lane = threadIdx.x & 63;
-  int off = 1;
-  #pragma unroll
-  for (int n = NV; n > 1; n >>= 1, off <<= 1) {
+  /* splitting steps exchange with lane ^ off and need a true exchange: distances 1 and 2 by quad permutation, further
+   * ones through the crossbar; the summing steps after them take the cheapest form of each distance */
+  auto split = [&](auto n_, auto off_) {
+    constexpr int n = decltype(n_)::value, off = decltype(off_)::value;
     const bool upper = (lane & off) != 0;
     #pragma unroll
     for (int i = 0; i < n / 2; ++i) {
       const double keep = upper ? v[i + n / 2] : v[i], send = upper ? v[i] : v[i + n / 2];
-      v[i] = keep + __shfl_xor(send, off, 64);
+      if constexpr (off <= 2) { v[i] = keep + partner_value<off>(send); } else { v[i] = keep + __shfl_xor(send, off, 64); }
     }
-  }
+  };
+  if constexpr (NV >= 2) { split(std::integral_constant<int, NV>{}, std::integral_constant<int, 1>{}); }
+  if constexpr (NV >= 4) { split(std::integral_constant<int, NV / 2>{}, std::integral_constant<int, 2>{}); }
+  if constexpr (NV >= 8) { split(std::integral_constant<int, NV / 4>{}, std::integral_constant<int, 4>{}); }
+  if constexpr (NV >= 16) { split(std::integral_constant<int, NV / 8>{}, std::integral_constant<int, 8>{}); }
+  if constexpr (NV >= 32) { split(std::integral_constant<int, NV / 16>{}, std::integral_constant<int, 16>{}); }
+  if constexpr (NV >= 64) { split(std::integral_constant<int, NV / 32>{}, std::integral_constant<int, 32>{}); }
   double s = v[0];
-  #pragma unroll
-  for (; off < 64; off <<= 1) { s += __shfl_xor(s, off, 64); }
+  if constexpr (NV < 2) { s += partner_value<1>(s); }
+  if constexpr (NV < 4) { s += partner_value<2>(s); }
+  if constexpr (NV < 8) { s += partner_value<4>(s); }
+  if constexpr (NV < 16) { s += partner_value<8>(s); }
+  if constexpr (NV < 32) { s += partner_value<16>(s); }
+  if constexpr (NV < 64) { s += partner_value<32>(s); }
   return s;
 }
 template <int NV> __device__ __forceinline__ int split_index(int lane) {
