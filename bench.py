@@ -7,7 +7,8 @@ reconstruction of the exact integer Gram.  Prints ONE JSON line:
   value      effective Gram TFLOP/s = M N (N+1) (x4 complex) / step time  (the FP SYRK/HERK flops replaced)
   roofline   the contraction kernel alone, timed with HIP events on its stream: algorithmic int8 ops / time
              against the dense INT8 MFMA peak
-  cpu_baseline  the same limb / CRT algorithm compiled for the host (the oracle), timed on a row sample
+  cpu_baseline  the same limb / CRT algorithm compiled for the host (the oracle), timed on a row sample, with
+             OpenBLAS DSYRK / ZHERK on the same sample and LAPACK syevd / heevd on its N x N Gram beside it
 """
 import argparse
 import ctypes as C
@@ -78,13 +79,19 @@ def cpu_baseline(at, M, N, eps, alg, order, u, sample_rows):
     ho.i8herk(kind, cplx, N, order, panels, 0, 2)
     dt = time.perf_counter() - t0
     feff = sample_rows * N * (N + 1) * (4 if cplx else 1)
-    out = {"value": feff / dt / 1e12, "unit": "TFLOP/s (FP-equivalent Gram flops)", "cores": os.cpu_count(), "kind": "port",
+    threads = int(os.environ.get("OMP_NUM_THREADS") or len(os.sched_getaffinity(0)))   # what the OpenMP loops of the oracle run on
+    out = {"value": feff / dt / 1e12, "unit": "TFLOP/s (FP-equivalent Gram flops)", "cores": threads, "kind": "port",
            "sample": "first %d of %d rows (int8 work is linear in rows), %s order %d, %.2f s" % (sample_rows, M, kind, order, dt)}
     try:   # FP reference: SYRK / HERK from the BLAS scipy ships, on the same sample
         from scipy.linalg import blas
         t0 = time.perf_counter()
-        (blas.zherk if cplx else blas.dsyrk)(1.0, np.asfortranarray(A.astype(np.complex128 if cplx else np.float64)), trans=2 if cplx else 1)
+        G = (blas.zherk if cplx else blas.dsyrk)(1.0, np.asfortranarray(A.astype(np.complex128 if cplx else np.float64)), trans=2 if cplx else 1)
         out["fp_blas_tflops"] = feff / (time.perf_counter() - t0) / 1e12
+        # eigenvalues of the N x N Gram with LAPACK's divide and conquer: the FP counterpart of the fit's tail
+        from scipy.linalg import lapack
+        t0 = time.perf_counter()
+        (lapack.zheevd if cplx else lapack.dsyevd)(G, compute_v=1, lower=0)
+        out["fp_lapack_syevd_ms"] = (time.perf_counter() - t0) * 1e3
     except Exception as e:  # pragma: no cover
         out["fp_blas_tflops"] = None
         out["fp_blas_note"] = "BLAS unavailable: %s" % e
