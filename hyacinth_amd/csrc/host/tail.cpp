@@ -7,7 +7,8 @@
  * potrfp.hip and tail.hip; no vendor solver is involved.  Differences that are visible to a caller:
  *  - an FP32 Gram is widened to FP64 before the Cholesky (the reference factors it in FP32);
  *  - the SVD always runs in FP64, also for FP32 / FP16 storage (the reference uses FP32 there);
- *  - the Jacobi iteration stops as soon as a sweep applies no rotation; a sweep here is one plain round-robin pass over all
+ *  - the Jacobi iteration stops as soon as a sweep applies no rotation, or leaves only cosines that the quadratic
+ *    contraction measured over the last two sweeps puts within 8 thresholds; a sweep here is one plain round-robin pass over all
  *    column pairs, which does less work than a sweep of the vendor's blocked solver, so the cap is 5 x |JacobiSVDSweeps|
  *    plain sweeps (15 by default); JacobiSVDSweeps == 0 (the reference's "bidiagonalization backend") caps at 30.
  * G is left untouched (the reference overwrites it with the factor).
@@ -75,6 +76,7 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
      * below it costs sweeps and leaves the orthogonality where it was.  Nor below a sixteenth of the accuracy asked for:
      * cosines of that size move a singular value by less than eps / 2 of the largest one. */
     const double rotateAbove = std::max(std::max(machineEps, std::sqrt((double)N) * 2.220446049250313e-16), eps / 16.);
+    double lastCosine2 = 0.;
     for (int32_t sw = 0; sw < maxSweeps && rank > 1; ++sw) {
       HYH_KERNEL(hykGramWorkspaceClear(s, counter.p, 64));
       HYH_KERNEL(hykJacobiSweep(s, Complex, N, rank, B.as<double>(), rotateAbove, counter.as<int32_t>())); ++used;
@@ -85,6 +87,16 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
        * and a further sweep would only confirm it. */
       if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: %d rotations, largest cosine %.2le\n", used, seen.rotations, std::sqrt(seen.cosine2)); }
       if (seen.rotations == 0 || seen.cosine2 <= 64. * rotateAbove * rotateAbove) { break; }
+      /* Or when the sweeps have reached their quadratic phase and the next one could only confirm: the largest cosine
+       * c_k of this sweep against c_{k-1}^2 of the one before gives the constant of the contraction as it is here
+       * (clusters of singular values make it larger); if that constant is moderate and, applied once more, puts the
+       * cosines this sweep has left behind (constant x c_k^2) within the same 8 thresholds, the columns are there. */
+      const double c2 = seen.cosine2;
+      if (lastCosine2 > 0. && c2 > 0.) {
+        const double contraction = std::max(1., std::sqrt(c2) / lastCosine2);   /* c_k / c_{k-1}^2 */
+        if (contraction <= 16. && contraction * c2 <= 8. * rotateAbove) { break; }
+      }
+      lastCosine2 = c2;
     }
     HYH_KERNEL(hykColumnNorms(s, Complex, N, rank, B.as<double>(), sigma.as<double>()));
     std::vector<double> sig((size_t)rank); HYH_CHECK(hipMemcpyAsync(sig.data(), sigma.p, sizeof(double) * (size_t)rank, hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));

@@ -268,30 +268,48 @@ __global__ __launch_bounds__(THREADS) void jacobi_block_round_kernel(int32_t N, 
       if (lane == j) { alpha = norm[c0]; beta = norm[c1]; pairLive = live[c0] && live[c1]; }
     }
     const double g2 = gre * gre + gim * gim;
-    if (pairLive) { worst = fmax(worst, squared_cosine(g2, alpha, beta)); }
+    if (pairLive) {                                /* worst = max(worst, squared_cosine(g2, alpha, beta)), dividing only where the maximum moves */
+      const double ab = alpha * beta;
+      if (ab > 0.) { if (g2 > worst * ab) { worst = g2 / ab; } } else if (g2 > 0.) { worst = fmax(worst, 1.); }
+    }
     const bool rotate = pairLive && g2 > tol * tol * alpha * beta && g2 > 0.;
     double cs = 1., sn = 0., er = 1., ei = 0., shift = 0.;
     if (rotate) {
-      const double gabs = sqrt(g2), zeta = (beta - alpha) / (2. * gabs);
-      const double t = (zeta >= 0. ? 1. : -1.) / (fabs(zeta) + sqrt(1. + zeta * zeta));
-      cs = 1. / sqrt(1. + t * t); sn = cs * t; er = gre / gabs; ei = gim / gabs; shift = t * gabs;
+      /* t = tan of the rotation angle = sign(d) h / (|d| + sqrt(d^2 + h^2)) with d = beta - alpha, h = 2 |g|: the smaller
+       * root of t^2 + 2 (d / h) t - 1 = 0 without the division by h; d and h are first scaled by one power of two, so
+       * that their squares neither overflow nor vanish.  One square root, one division and one reciprocal square root
+       * in sequence (the textbook order takes three of each kind, each waiting for the one before). */
+      double gabs;
+      if constexpr (CPLX) { gabs = sqrt(g2); const double inv = 1. / gabs; er = gre * inv; ei = gim * inv; }
+      else { gabs = fabs(gre); er = gre < 0. ? -1. : 1.; }
+      const double d = beta - alpha, h = 2. * gabs;
+      const int e = __builtin_amdgcn_frexp_exp(fmax(fabs(d), h));
+      const double ds = ldexp(fabs(d), -e), hs = ldexp(h, -e);
+      const double t = copysign(hs / (ds + sqrt(ds * ds + hs * hs)), d);
+      cs = rsqrt(1. + t * t); sn = cs * t; shift = t * gabs;
     }
     #pragma unroll
     for (int j = 0; j < BC; ++j) {
       const int fa = (j == 0) ? NC - 1 : (step + j) % (NC - 1), fb = (j == 0) ? step : (step - j + (NC - 1)) % (NC - 1);
       const int c0 = FULL ? (fa < fb ? fa : fb) : j, c1 = FULL ? (fa < fb ? fb : fa) : BC + (j + step) % BC;
       if (lane_value((int)rotate, j)) {
-        const double csj = lane_value(cs, j), snj = lane_value(sn, j), erj = lane_value(er, j), shj = lane_value(shift, j);
-        [[maybe_unused]] const double eij = CPLX ? lane_value(ei, j) : 0.;
-        #pragma unroll
-        for (int m = 0; m < ROWS; ++m) {
-          if constexpr (CPLX) {
+        const double csj = lane_value(cs, j), snj = lane_value(sn, j), shj = lane_value(shift, j);
+        if constexpr (CPLX) {
+          const double erj = lane_value(er, j), eij = lane_value(ei, j);
+          #pragma unroll
+          for (int m = 0; m < ROWS; ++m) {
             const double pr = x[c0][m][0], pi = x[c0][m][1], q0 = x[c1][m][0], q1 = x[c1][m][1];
             const double qr = q0 * erj + q1 * eij, qi = q1 * erj - q0 * eij;
             x[c0][m][0] = csj * pr - snj * qr; x[c0][m][1] = csj * pi - snj * qi; x[c1][m][0] = snj * pr + csj * qr; x[c1][m][1] = snj * pi + csj * qi;
-          } else {
-            const double pv = x[c0][m][0], qv = x[c1][m][0] * erj;
-            x[c0][m][0] = csj * pv - snj * qv; x[c1][m][0] = snj * pv + csj * qv;
+          }
+        } else {
+          /* real: e^{i phi} = +-1, folded into the coefficients of column c1 as a sign bit (same bits as multiplying the column first) */
+          const long long flip = (long long)(unsigned long long)(unsigned)lane_value((int)(er < 0.), j) << 63;
+          const double aj = __longlong_as_double(__double_as_longlong(snj) ^ flip), bj = __longlong_as_double(__double_as_longlong(csj) ^ flip);
+          #pragma unroll
+          for (int m = 0; m < ROWS; ++m) {
+            const double pv = x[c0][m][0], qv = x[c1][m][0];
+            x[c0][m][0] = csj * pv - aj * qv; x[c1][m][0] = snj * pv + bj * qv;
           }
         }
         norm[c0] -= shj; norm[c1] += shj; ++applied;
