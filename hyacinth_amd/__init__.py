@@ -31,7 +31,7 @@ API_SYMBOLS = [
 KERNEL_SYMBOLS = [
     "hykColumnExponents", "hykSliceRange", "hykQuantizeLimbs", "hykQuantizeCrt", "hykZeroRows",
     "hykGramWorkspaceBytes", "hykGramWorkspaceClear", "hykGramCrt", "hykGramLimbs", "hykGramSetSlab",
-    "hykGramProfile", "hykGramProfileRead", "hykMfmaCeiling", "hykGramRange", "hykDequantize", "hykPotrfpWorkspaceBytes", "hykPotrfp", "hykFactorToB", "hykJacobiSweep",
+    "hykGramProfile", "hykGramProfileRead", "hykMfmaCeiling", "hykGramRange", "hykDequantize", "hykPotrfpWorkspaceBytes", "hykPotrfp", "hykFactorToB", "hykJacobiSweep", "hykJacobiSetVariant",
     "hykColumnNorms", "hykBasisOut", "hykValuesOut", "hykInterpSolve", "hykInterpOut", "hykMatcopy",
     "hykSumSquares", "hykMatmulCf16", "hykGemm", "hykOrthonormalize",
 ]
@@ -87,6 +87,8 @@ def lib():
         L.hykGramCrt.argtypes = [vp, i32, i32, i32, vp, i64, i32, i32, i32, vp, vp]
         L.hykGramLimbs.argtypes = [vp, i32, i32, i32, vp, i64, i32, i32, i32, vp, vp]
         L.hykGramSetSlab.argtypes = [i32]
+        L.hykJacobiSetVariant.argtypes = [i32]
+        L.hykJacobiSweep.argtypes = [vp, i32, i32, i32, vp, dbl, vp]
         L.hykGramProfile.argtypes = [i32]
         L.hykGramProfileRead.argtypes = [C.POINTER(dbl), C.POINTER(i32)]
         L.hykMfmaCeiling.argtypes = [vp, i32, i32, i32, C.POINTER(dbl), C.POINTER(dbl)]

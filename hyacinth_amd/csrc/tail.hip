@@ -334,6 +334,165 @@ __global__ __launch_bounds__(THREADS) void jacobi_block_round_kernel(int32_t N, 
   if (threadIdx.x == 0) { atomicAdd(rotations, applied); }
 }
 
+/* ------------------------------------------------------------------ blocked one-sided Jacobi in Gram space (real)
+ * The kernel above pays one workgroup reduction, one barrier and one chain of square roots and divisions per step.  Here a
+ * round takes ONE reduction: the Gram matrix of the workgroup's 2 BC columns (all NC (NC + 1) / 2 products, summed over the
+ * rows).  The first wavefront then runs the steps on that small matrix alone (G <- J^T G J per step, kept in LDS; the
+ * entries a rotation fixes, alpha - t gamma, beta + t gamma and 0, are written as such) and leaves the list of rotations in
+ * LDS; after one more barrier every thread replays the list on its rows.  Same pairs, same order, same rotation rule as the
+ * step kernel; the cross products of later steps come out of the updated Gram matrix instead of fresh dot products (both
+ * carry rounding noise of the size eps |x_i| |x_j|; the next round starts from fresh sums again). */
+struct RotRec { double cs, sn, a, b; };   /* x_c0' = cs x_c0 - a x_c1,  x_c1' = sn x_c0 + b x_c1;  sn == 0: no rotation */
+
+__device__ __forceinline__ void wave_lds_sync() {   /* LDS operations of one wavefront complete in order: only the compiler must not move them */
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <int ROWS, int BC, bool FULL, int THREADS>
+__global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, int32_t nb, int32_t r, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations) {
+  constexpr int NC = 2 * BC, NG = NC * (NC + 1) / 2, WAVES = THREADS / 64, STEPS = FULL ? NC - 1 : BC, GS = NC + 1;
+  constexpr int CH = NG >= 32 ? 32 : NG, TAIL = NG % CH;
+  static_assert((TAIL & (TAIL - 1)) == 0 && BC * NC <= 128, "tail chunk a power of two; two passes of the first wavefront cover a phase");
+  __shared__ double part[WAVES][NG];
+  __shared__ double Gs[NC * GS];
+  __shared__ RotRec rot[STEPS][BC];
+  __shared__ double fixed[BC][2];
+  __shared__ int32_t pairCol[BC][2];
+  __shared__ int32_t appliedAll;
+  const int i = blockIdx.x; int P, Q;
+  if (i == 0) { P = nb - 1; Q = round; } else { P = (round + i) % (nb - 1); Q = (round - i + (nb - 1)) % (nb - 1); }
+  if (P > Q) { const int t = P; P = Q; Q = t; }
+  int col[NC]; bool live[NC];
+  #pragma unroll
+  for (int c = 0; c < NC; ++c) { col[c] = (c < BC ? P : Q) * BC + (c % BC); live[c] = col[c] < r; }
+  if (!live[0]) { return; }
+  double x[NC][ROWS];
+  #pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    #pragma unroll
+    for (int m = 0; m < ROWS; ++m) { const int k = threadIdx.x + m * THREADS; x[c][m] = (live[c] && k < N) ? B[(int64_t)col[c] * N + k] : 0.; }
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  /* products numbered by diagonal: p = d NC + c stands for (c, (c + d) % NC), d = 0 .. NC / 2 (the last diagonal only for
+   * c < NC / 2): every unordered pair once, and p splits back into the pair by shifts.  Summed over the wavefront 32 at a time. */
+  #pragma unroll
+  for (int chunk = 0; chunk < NG / CH; ++chunk) {
+    double v[CH];
+    #pragma unroll
+    for (int q = 0; q < CH; ++q) {
+      const int p = chunk * CH + q, c0 = p % NC, c1 = (c0 + p / NC) % NC;
+      double sum = 0.;
+      #pragma unroll
+      for (int m = 0; m < ROWS; ++m) { sum += x[c0][m] * x[c1][m]; }
+      v[q] = sum;
+    }
+    const double tot = wave_sum_split<CH>(v);
+    if (lane < CH) { part[wave][chunk * CH + split_index<CH>(lane)] = tot; }
+  }
+  if constexpr (TAIL > 0) {
+    double v[TAIL];
+    #pragma unroll
+    for (int q = 0; q < TAIL; ++q) {
+      const int p = (NG / CH) * CH + q, c0 = p % NC, c1 = (c0 + p / NC) % NC;
+      double sum = 0.;
+      #pragma unroll
+      for (int m = 0; m < ROWS; ++m) { sum += x[c0][m] * x[c1][m]; }
+      v[q] = sum;
+    }
+    const double tot = wave_sum_split<TAIL>(v);
+    if (lane < TAIL) { part[wave][(NG / CH) * CH + split_index<TAIL>(lane)] = tot; }
+  }
+  __syncthreads();
+  if (wave == 0) {
+    for (int idx = lane; idx < NG; idx += 64) {
+      double tot = 0.;
+      #pragma unroll
+      for (int w = 0; w < WAVES; ++w) { tot += part[w][idx]; }
+      const int c0 = idx % NC, c1 = (c0 + idx / NC) % NC;
+      Gs[c0 * GS + c1] = tot; Gs[c1 * GS + c0] = tot;
+    }
+    wave_lds_sync();
+    int applied = 0; double worst = 0.;
+    for (int step = 0; step < STEPS; ++step) {
+      if (lane < BC) {
+        const int j = lane;
+        int c0, c1;
+        if constexpr (FULL) {
+          const int fa = (j == 0) ? NC - 1 : (step + j) % (NC - 1), fb = (j == 0) ? step : (step - j + (NC - 1)) % (NC - 1);
+          c0 = fa < fb ? fa : fb; c1 = fa < fb ? fb : fa;
+        } else { c0 = j; c1 = BC + (j + step) % BC; }
+        const double alpha = Gs[c0 * GS + c0], beta = Gs[c1 * GS + c1], gre = Gs[c0 * GS + c1];
+        const bool pairLive = ((c0 < BC ? P : Q) * BC + (c0 % BC) < r) && ((c1 < BC ? P : Q) * BC + (c1 % BC) < r);
+        const double g2 = gre * gre;
+        if (pairLive) {
+          const double ab = alpha * beta;
+          if (ab > 0.) { if (g2 > worst * ab) { worst = g2 / ab; } } else if (g2 > 0.) { worst = fmax(worst, 1.); }
+        }
+        const bool rotate = pairLive && g2 > tol * tol * alpha * beta && g2 > 0.;
+        RotRec rr = { 1., 0., 0., 1. }; double na = alpha, nbeta = beta;
+        if (rotate) {
+          /* t = sign(d) h / (|d| + sqrt(d^2 + h^2)), d = beta - alpha, h = 2 |g|, scaled by one power of two (see the step kernel) */
+          const double gabs = fabs(gre), d = beta - alpha, h = 2. * gabs;
+          const int e = __builtin_amdgcn_frexp_exp(fmax(fabs(d), h));
+          const double ds = ldexp(fabs(d), -e), hs = ldexp(h, -e);
+          const double t = copysign(hs / (ds + sqrt(ds * ds + hs * hs)), d);
+          const double cs = rsqrt(1. + t * t), sn = cs * t, shift = t * gabs;
+          rr.cs = cs; rr.sn = sn; rr.a = gre < 0. ? -sn : sn; rr.b = gre < 0. ? -cs : cs;
+          na = alpha - shift; nbeta = beta + shift;
+          if (sn != 0.) { ++applied; }
+        }
+        rot[step][j] = rr; fixed[j][0] = na; fixed[j][1] = nbeta; pairCol[j][0] = c0; pairCol[j][1] = c1;
+      }
+      wave_lds_sync();
+      /* G <- G J: entry (row, c0) and (row, c1) of every pair */
+      #pragma unroll
+      for (int item = lane; item < BC * NC; item += 64) {
+        const int j = item / NC, row = item % NC, c0 = pairCol[j][0], c1 = pairCol[j][1]; const RotRec rr = rot[step][j];
+        const double u = Gs[row * GS + c0], w = Gs[row * GS + c1];
+        Gs[row * GS + c0] = rr.cs * u - rr.a * w; Gs[row * GS + c1] = rr.sn * u + rr.b * w;
+      }
+      wave_lds_sync();
+      /* G <- J^T G: entry (c0, k) and (c1, k); what the rotation fixes is written as such */
+      #pragma unroll
+      for (int item = lane; item < BC * NC; item += 64) {
+        const int j = item / NC, k = item % NC, c0 = pairCol[j][0], c1 = pairCol[j][1]; const RotRec rr = rot[step][j];
+        const double u = Gs[c0 * GS + k], w = Gs[c1 * GS + k];
+        double y0 = rr.cs * u - rr.a * w, y1 = rr.sn * u + rr.b * w;
+        if (rr.sn != 0.) { if (k == c0) { y0 = fixed[j][0]; y1 = 0.; } else if (k == c1) { y0 = 0.; y1 = fixed[j][1]; } }
+        Gs[c0 * GS + k] = y0; Gs[c1 * GS + k] = y1;
+      }
+      wave_lds_sync();
+    }
+    #pragma unroll
+    for (int off = BC / 2; off > 0; off >>= 1) { worst = fmax(worst, __shfl_xor(worst, off, 64)); applied += __shfl_xor(applied, off, 64); }
+    if (lane == 0) { report_cosine(rotations, worst); appliedAll = applied; if (applied > 0) { atomicAdd(rotations, applied); } }
+  }
+  __syncthreads();
+  if (appliedAll == 0) { return; }
+  /* replay the rotations on the rows of this thread (records fetched one ahead) */
+  RotRec cur = rot[0][0];
+  #pragma unroll
+  for (int n = 0; n < STEPS * BC; ++n) {
+    const int step = n / BC, j = n % BC;
+    const RotRec rr = cur;
+    if (n + 1 < STEPS * BC) { cur = rot[(n + 1) / BC][(n + 1) % BC]; }
+    const int fa = (j == 0) ? NC - 1 : (step + j) % (NC - 1), fb = (j == 0) ? step : (step - j + (NC - 1)) % (NC - 1);
+    const int c0 = FULL ? (fa < fb ? fa : fb) : j, c1 = FULL ? (fa < fb ? fb : fa) : BC + (j + step) % BC;
+    if (rr.sn != 0.) {
+      #pragma unroll
+      for (int m = 0; m < ROWS; ++m) {
+        const double pv = x[c0][m], qv = x[c1][m];
+        x[c0][m] = rr.cs * pv - rr.a * qv; x[c1][m] = rr.sn * pv + rr.b * qv;
+      }
+    }
+  }
+  #pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    #pragma unroll
+    for (int m = 0; m < ROWS; ++m) { const int k = threadIdx.x + m * THREADS; if (live[c] && k < N) { B[(int64_t)col[c] * N + k] = x[c][m]; } }
+  }
+}
+
 template <bool CPLX>
 __global__ __launch_bounds__(T_THREADS) void column_norm_kernel(int32_t N, const double* __restrict__ B, double* __restrict__ sigma) {
   __shared__ double scratch[T_THREADS / 64]; constexpr int W = CPLX ? 2 : 1;
@@ -438,6 +597,16 @@ extern "C" int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t
 }
 
 /* one sweep = every pair of the r columns of B (N x r, FP64, complex interleaved) once; rotations counts the rotations applied */
+static int g_jacobiVariant = 0;   /* 0: Gram-space rounds for real factors, 8-column blocks where they fit (default); 1: the step kernel everywhere; 2: Gram-space rounds, 4-column blocks */
+
+template <int ROWS, int BC, int THREADS = T_THREADS>
+static int gram_sweep(hipStream_t stream, int32_t N, int32_t r, double* B, double tol, int32_t* rotations) {
+  const int blocks = (r + BC - 1) / BC, nb = (blocks + 1) & ~1;
+  jacobi_gram_round_kernel<ROWS, BC, true, THREADS><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations);
+  for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations); }
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
 template <bool CPLX, int ROWS, int BC, int THREADS = T_THREADS>
 static int blocked_sweep(hipStream_t stream, int32_t N, int32_t r, double* B, double tol, int32_t* rotations) {
   const int blocks = (r + BC - 1) / BC, nb = (blocks + 1) & ~1;
@@ -446,9 +615,22 @@ static int blocked_sweep(hipStream_t stream, int32_t N, int32_t r, double* B, do
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
+extern "C" int hykJacobiSetVariant(int32_t variant) { if (variant < 0 || variant > 2) { return -1; } g_jacobiVariant = variant; return 0; }
+
 extern "C" int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations) {
   if (N <= 0 || r <= 1) { return 0; }
   /* blocked kernel when the rows of two column blocks fit the registers of a workgroup */
+  /* real factors: Gram-space rounds; blocks of 8 columns where the rows of 16 columns fit the registers of 512 threads
+   * (half as many rounds, each 1.4 times as long at N = 2048), blocks of 4 otherwise */
+  if (!Complex && r >= 32 && g_jacobiVariant == 0) {
+    if (N <= 2 * 512) { return gram_sweep<2, 8, 512>(stream, N, r, B, tol, rotations); }
+    if (N <= 4 * 512) { return gram_sweep<4, 8, 512>(stream, N, r, B, tol, rotations); }
+  }
+  if (!Complex && r >= 16 && g_jacobiVariant != 1) {
+    if (N <= 4 * T_THREADS) { return gram_sweep<4, 4>(stream, N, r, B, tol, rotations); }
+    if (N <= 8 * T_THREADS) { return gram_sweep<8, 4>(stream, N, r, B, tol, rotations); }
+    if (N <= 8 * 512) { return gram_sweep<8, 4, 512>(stream, N, r, B, tol, rotations); }
+  }
   if (!Complex && r >= 16) {
     if (N <= 4 * T_THREADS) { return blocked_sweep<false, 4, 4>(stream, N, r, B, tol, rotations); }
     if (N <= 8 * T_THREADS) { return blocked_sweep<false, 8, 4>(stream, N, r, B, tol, rotations); }

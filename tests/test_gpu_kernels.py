@@ -415,3 +415,42 @@ def test_gemm_fp64(gl, cplx, opA, opB, M, N, K):
     got = host(dC, np.float64, (N, ldc, W))[:, :M, :]
     got = (got[..., 0] + 1j * got[..., 1]).T if cplx else got[..., 0].T
     assert np.abs(got - want).max() <= 1e-13 * np.abs(want).max() * max(1, K) ** 0.5
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("cplx,N,r", [(0, 300, 40), (0, 1000, 130), (0, 2048, 96), (0, 2500, 70), (1, 600, 50), (0, 64, 64), (0, 700, 20)])
+def test_jacobi_sweep_kernels(gl, variant, cplx, N, r):
+    """One-sided Jacobi sweeps on a graded N x r factor: every kernel behind hykJacobiSweep (Gram-space rounds with blocks
+    of 8 and of 4 columns, the step kernel, the pair kernel for few columns) must leave orthogonal columns whose norms are
+    the singular values numpy finds, to 32 sqrt(r) eps of the largest (a column takes part in a few hundred rotations), and
+    whose span is unchanged."""
+    from gpu_util import dev, host, ptr, stream, sync, zeros
+    rng = np.random.default_rng(1000 * N + r + cplx)
+    B = rng.standard_normal((N, r)) + (1j * rng.standard_normal((N, r)) if cplx else 0)
+    mix = np.triu(rng.standard_normal((r, r))) * 0.1 + np.eye(r)          # columns correlated
+    B = (B @ mix) * 10.0 ** (-6.0 * np.arange(r) / r)                       # graded like a pivoted Cholesky factor
+    want = np.linalg.svd(B, compute_uv=False)
+    dB = dev(np.ascontiguousarray(B.T)); counter = zeros(64)
+    tol = float(2.220446049250313e-16 * np.sqrt(N))
+    assert gl.L.hykJacobiSetVariant(variant) == 0
+    try:
+        sweeps = 0
+        while True:
+            counter.zero_()
+            print("jacobi", variant, cplx, N, r, "sweep", sweeps, flush=True)
+            assert gl.L.hykJacobiSweep(stream(), cplx, N, r, ptr(dB), tol, ptr(counter)) == 0
+            sync(); sweeps += 1
+            rotations = int(host(counter, np.int32)[0]); cos2 = float(host(counter, np.float64)[1])
+            if rotations == 0:
+                break
+            assert sweeps < 30, "no convergence"
+        assert cos2 <= (8 * tol) ** 2
+    finally:
+        gl.L.hykJacobiSetVariant(0)
+    U = host(dB, np.complex128 if cplx else np.float64, (r, N)).T
+    got = np.sort(np.linalg.norm(U, axis=0))[::-1]
+    assert np.max(np.abs(got - want)) <= 32 * 2.220446049250313e-16 * want[0] * np.sqrt(r)
+    Un = U / np.linalg.norm(U, axis=0)
+    assert np.max(np.abs(Un.conj().T @ Un - np.eye(r))) <= 16 * tol
+    Qb, _ = np.linalg.qr(B)                                               # same column space
+    assert np.linalg.norm(Un - Qb @ (Qb.conj().T @ Un)) <= 1e-9 * np.sqrt(r)
