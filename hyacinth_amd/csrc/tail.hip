@@ -337,8 +337,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_block_round_kernel(int32_t N, 
 /* ------------------------------------------------------------------ blocked one-sided Jacobi in Gram space (real)
  * The kernel above pays one workgroup reduction, one barrier and one chain of square roots and divisions per step.  Here a
  * round takes ONE reduction: the Gram matrix of the workgroup's 2 BC columns (all NC (NC + 1) / 2 products, summed over the
- * rows).  The first wavefront then runs the steps on that small matrix alone (G <- J^T G J per step, kept in LDS; the
- * entries a rotation fixes, alpha - t gamma, beta + t gamma and 0, are written as such) and leaves the list of rotations in
+ * rows).  The first wavefront then runs the steps on that small matrix alone (G <- J^T G J per step, kept in LDS) and leaves the list of rotations in
  * LDS; after one more barrier every thread replays the list on its rows.  Same pairs, same order, same rotation rule as the
  * step kernel; the cross products of later steps come out of the updated Gram matrix instead of fresh dot products (both
  * carry rounding noise of the size eps |x_i| |x_j|; the next round starts from fresh sums again). */
@@ -352,7 +351,7 @@ template <int ROWS, int BC, bool FULL, int THREADS>
 __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, int32_t nb, int32_t r, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations) {
   constexpr int NC = 2 * BC, NG = NC * (NC + 1) / 2, WAVES = THREADS / 64, STEPS = FULL ? NC - 1 : BC, GS = NC + 1;
   constexpr int CH = NG >= 32 ? 32 : NG, TAIL = NG % CH;
-  static_assert((TAIL & (TAIL - 1)) == 0 && BC * NC <= 128, "tail chunk a power of two; two passes of the first wavefront cover a phase");
+  static_assert((TAIL & (TAIL - 1)) == 0 && BC * BC <= 64, "tail chunk a power of two; one lane of the first wavefront per pair of pairs");
   __shared__ double part[WAVES][NG];
   __shared__ double Gs[NC * GS];
   __shared__ RotRec rot[STEPS][BC];
@@ -444,22 +443,17 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
         rot[step][j] = rr; fixed[j][0] = na; fixed[j][1] = nbeta; pairCol[j][0] = c0; pairCol[j][1] = c1;
       }
       wave_lds_sync();
-      /* G <- G J: entry (row, c0) and (row, c1) of every pair */
-      #pragma unroll
-      for (int item = lane; item < BC * NC; item += 64) {
-        const int j = item / NC, row = item % NC, c0 = pairCol[j][0], c1 = pairCol[j][1]; const RotRec rr = rot[step][j];
-        const double u = Gs[row * GS + c0], w = Gs[row * GS + c1];
-        Gs[row * GS + c0] = rr.cs * u - rr.a * w; Gs[row * GS + c1] = rr.sn * u + rr.b * w;
-      }
-      wave_lds_sync();
-      /* G <- J^T G: entry (c0, k) and (c1, k); what the rotation fixes is written as such */
-      #pragma unroll
-      for (int item = lane; item < BC * NC; item += 64) {
-        const int j = item / NC, k = item % NC, c0 = pairCol[j][0], c1 = pairCol[j][1]; const RotRec rr = rot[step][j];
-        const double u = Gs[c0 * GS + k], w = Gs[c1 * GS + k];
-        double y0 = rr.cs * u - rr.a * w, y1 = rr.sn * u + rr.b * w;
-        if (rr.sn != 0.) { if (k == c0) { y0 = fixed[j][0]; y1 = 0.; } else if (k == c1) { y0 = 0.; y1 = fixed[j][1]; } }
-        Gs[c0 * GS + k] = y0; Gs[c1 * GS + k] = y1;
+      /* G <- J^T G J, one lane per pair of pairs: the 2 x 2 block (rows of pair jr, columns of pair jc) takes the column
+       * rotation of jc and the row rotation of jr at once; the blocks are disjoint, so one pass does the step.  What a
+       * rotation fixes (its own block: alpha - t gamma, beta + t gamma, 0) is written as such. */
+      if (lane < BC * BC) {
+        const int jr = lane / BC, jc = lane % BC, r0 = pairCol[jr][0], r1 = pairCol[jr][1], k0 = pairCol[jc][0], k1 = pairCol[jc][1];
+        const RotRec rw = rot[step][jr], cl = rot[step][jc];
+        const double g00 = Gs[r0 * GS + k0], g01 = Gs[r0 * GS + k1], g10 = Gs[r1 * GS + k0], g11 = Gs[r1 * GS + k1];
+        const double h00 = cl.cs * g00 - cl.a * g01, h01 = cl.sn * g00 + cl.b * g01, h10 = cl.cs * g10 - cl.a * g11, h11 = cl.sn * g10 + cl.b * g11;
+        double y00 = rw.cs * h00 - rw.a * h10, y10 = rw.sn * h00 + rw.b * h10, y01 = rw.cs * h01 - rw.a * h11, y11 = rw.sn * h01 + rw.b * h11;
+        if (jr == jc && rw.sn != 0.) { y00 = fixed[jr][0]; y11 = fixed[jr][1]; y01 = 0.; y10 = 0.; }
+        Gs[r0 * GS + k0] = y00; Gs[r0 * GS + k1] = y01; Gs[r1 * GS + k0] = y10; Gs[r1 * GS + k1] = y11;
       }
       wave_lds_sync();
     }
