@@ -90,6 +90,51 @@ __device__ __forceinline__ double wave_sum_split(double (&v)[NV]) {
   if constexpr (NV < 64) { s += partner_value<32>(s); }
   return s;
 }
+/* The same sums taken from the top: the halving steps at distances 32 and 16 are register swaps between lane halves
+ * (v_permlane32_swap / v_permlane16_swap: after swapping a and b, a + b holds the sum of a in the lower lanes and of b in
+ * the upper ones; three instructions per double instead of the seven of a select-and-exchange), and only NV / 4 values
+ * are left for the distances below.  NV a power of two, 4 .. 32.  Returns, in every lane, the sum of value
+ * lane >> (6 - log2 NV). */
+typedef unsigned v2u_t __attribute__((ext_vector_type(2)));
+template <int OFF>
+__device__ __forceinline__ double swap_add(double a, double b) {
+  const long long ab = __double_as_longlong(a), bb = __double_as_longlong(b);
+  v2u_t lo, hi;
+  if constexpr (OFF == 32) { lo = __builtin_amdgcn_permlane32_swap((unsigned)ab, (unsigned)bb, false, false); hi = __builtin_amdgcn_permlane32_swap((unsigned)(ab >> 32), (unsigned)(bb >> 32), false, false); }
+  else { lo = __builtin_amdgcn_permlane16_swap((unsigned)ab, (unsigned)bb, false, false); hi = __builtin_amdgcn_permlane16_swap((unsigned)(ab >> 32), (unsigned)(bb >> 32), false, false); }
+  return __longlong_as_double((long long)(((unsigned long long)hi.x << 32) | lo.x)) + __longlong_as_double((long long)(((unsigned long long)hi.y << 32) | lo.y));
+}
+template <int OFF>
+__device__ __forceinline__ double xor_value(double v) {   /* the value of lane ^ OFF, OFF <= 8 */
+  if constexpr (OFF == 4) { return __shfl_xor(v, 4, 64); } else { return partner_value<OFF>(v); }   /* a rotation by 8 inside a row of 16 is lane ^ 8 */
+}
+template <int NV>
+__device__ __forceinline__ double wave_sum_swap(double (&v)[NV]) {
+  static_assert(NV >= 4 && NV <= 32 && (NV & (NV - 1)) == 0, "a power of two, 4 .. 32");
+  const int lane = threadIdx.x & 63;
+  #pragma unroll
+  for (int i = 0; i < NV / 2; ++i) { v[i] = swap_add<32>(v[i], v[i + NV / 2]); }
+  #pragma unroll
+  for (int i = 0; i < NV / 4; ++i) { v[i] = swap_add<16>(v[i], v[i + NV / 4]); }
+  auto split = [&](auto n_, auto off_) {
+    constexpr int n = decltype(n_)::value, off = decltype(off_)::value;
+    const bool upper = (lane & off) != 0;
+    #pragma unroll
+    for (int i = 0; i < n / 2; ++i) {
+      const double keep = upper ? v[i + n / 2] : v[i], send = upper ? v[i] : v[i + n / 2];
+      v[i] = keep + xor_value<off>(send);
+    }
+  };
+  if constexpr (NV >= 8) { split(std::integral_constant<int, NV / 4>{}, std::integral_constant<int, 8>{}); }
+  if constexpr (NV >= 16) { split(std::integral_constant<int, NV / 8>{}, std::integral_constant<int, 4>{}); }
+  if constexpr (NV >= 32) { split(std::integral_constant<int, NV / 16>{}, std::integral_constant<int, 2>{}); }
+  double s = v[0];
+  if constexpr (NV < 8) { s += xor_value<8>(s); }
+  if constexpr (NV < 16) { s += xor_value<4>(s); }
+  if constexpr (NV < 32) { s += xor_value<2>(s); }
+  s += xor_value<1>(s);
+  return s;
+}
 template <int NV> __device__ __forceinline__ int split_index(int lane) {
   int idx = 0, half = NV >> 1;
   #pragma unroll
@@ -385,8 +430,8 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
       for (int m = 0; m < ROWS; ++m) { sum += x[c0][m] * x[c1][m]; }
       v[q] = sum;
     }
-    const double tot = wave_sum_split<CH>(v);
-    if (lane < CH) { part[wave][chunk * CH + split_index<CH>(lane)] = tot; }
+    const double tot = wave_sum_swap<CH>(v);
+    if ((lane & (64 / CH - 1)) == 0) { part[wave][chunk * CH + lane / (64 / CH)] = tot; }
   }
   if constexpr (TAIL > 0) {
     double v[TAIL];
@@ -398,8 +443,8 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
       for (int m = 0; m < ROWS; ++m) { sum += x[c0][m] * x[c1][m]; }
       v[q] = sum;
     }
-    const double tot = wave_sum_split<TAIL>(v);
-    if (lane < TAIL) { part[wave][(NG / CH) * CH + split_index<TAIL>(lane)] = tot; }
+    const double tot = wave_sum_swap<TAIL>(v);
+    if ((lane & (64 / TAIL - 1)) == 0) { part[wave][(NG / CH) * CH + lane / (64 / TAIL)] = tot; }
   }
   __syncthreads();
   if (wave == 0) {
