@@ -387,6 +387,11 @@ __global__ __launch_bounds__(THREADS) void jacobi_block_round_kernel(int32_t N, 
  * step kernel; the cross products of later steps come out of the updated Gram matrix instead of fresh dot products (both
  * carry rounding noise of the size eps |x_i| |x_j|; the next round starts from fresh sums again). */
 struct RotRec { double cs, sn, a, b; };   /* x_c0' = cs x_c0 - a x_c1,  x_c1' = sn x_c0 + b x_c1;  sn == 0: no rotation */
+/* The same rotation on columns kept as scale x vector (x_c = s_c u_c): u_c0' = u_c0 - t1 u_c1, u_c1' = u_c1 + t2 u_c0 with
+ * t1 = a s_c1 / (cs s_c0), t2 = sn s_c0 / (b s_c1), and s_c0' = cs s_c0, s_c1' = b s_c1: two multiply-adds per row instead of
+ * two products and two multiply-adds; the scales (within 2^-8 .. 1 over the at most 15 rotations a column meets in a round)
+ * are multiplied in once, before the columns are stored.  t1 == t2 == 0: no rotation. */
+struct FastRot { double t1, t2; };
 
 __device__ __forceinline__ void wave_lds_sync() {   /* LDS operations of one wavefront complete in order: only the compiler must not move them */
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -400,6 +405,8 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
   __shared__ double part[WAVES][NG];
   __shared__ double Gs[NC * GS];
   __shared__ RotRec rot[STEPS][BC];
+  __shared__ FastRot fast[STEPS][BC];
+  __shared__ double scale[NC];
   __shared__ double fixed[BC][2];
   __shared__ int32_t pairCol[BC][2];
   __shared__ int32_t appliedAll;
@@ -455,6 +462,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
       const int c0 = idx % NC, c1 = (c0 + idx / NC) % NC;
       Gs[c0 * GS + c1] = tot; Gs[c1 * GS + c0] = tot;
     }
+    if (lane < NC) { scale[lane] = 1.; }
     wave_lds_sync();
     int applied = 0; double worst = 0.;
     for (int step = 0; step < STEPS; ++step) {
@@ -473,7 +481,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
           if (ab > 0.) { if (g2 > worst * ab) { worst = g2 / ab; } } else if (g2 > 0.) { worst = fmax(worst, 1.); }
         }
         const bool rotate = pairLive && g2 > tol * tol * alpha * beta && g2 > 0.;
-        RotRec rr = { 1., 0., 0., 1. }; double na = alpha, nbeta = beta;
+        RotRec rr = { 1., 0., 0., 1. }; FastRot fr = { 0., 0. }; double na = alpha, nbeta = beta;
         if (rotate) {
           /* t = sign(d) h / (|d| + sqrt(d^2 + h^2)), d = beta - alpha, h = 2 |g|, scaled by one power of two (see the step kernel) */
           const double gabs = fabs(gre), d = beta - alpha, h = 2. * gabs;
@@ -483,9 +491,13 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
           const double cs = rsqrt(1. + t * t), sn = cs * t, shift = t * gabs;
           rr.cs = cs; rr.sn = sn; rr.a = gre < 0. ? -sn : sn; rr.b = gre < 0. ? -cs : cs;
           na = alpha - shift; nbeta = beta + shift;
-          if (sn != 0.) { ++applied; }
+          if (sn != 0.) {
+            ++applied;
+            const double s0 = scale[c0], s1 = scale[c1], n0 = cs * s0, n1 = rr.b * s1;
+            fr.t1 = rr.a * s1 / n0; fr.t2 = sn * s0 / n1; scale[c0] = n0; scale[c1] = n1;
+          }
         }
-        rot[step][j] = rr; fixed[j][0] = na; fixed[j][1] = nbeta; pairCol[j][0] = c0; pairCol[j][1] = c1;
+        rot[step][j] = rr; fast[step][j] = fr; fixed[j][0] = na; fixed[j][1] = nbeta; pairCol[j][0] = c0; pairCol[j][1] = c1;
       }
       wave_lds_sync();
       /* G <- J^T G J, one lane per pair of pairs: the 2 x 2 block (rows of pair jr, columns of pair jc) takes the column
@@ -509,21 +521,27 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
   __syncthreads();
   if (appliedAll == 0) { return; }
   /* replay the rotations on the rows of this thread (records fetched one ahead) */
-  RotRec cur = rot[0][0];
+  FastRot cur = fast[0][0];
   #pragma unroll
   for (int n = 0; n < STEPS * BC; ++n) {
     const int step = n / BC, j = n % BC;
-    const RotRec rr = cur;
-    if (n + 1 < STEPS * BC) { cur = rot[(n + 1) / BC][(n + 1) % BC]; }
+    const FastRot fr = cur;
+    if (n + 1 < STEPS * BC) { cur = fast[(n + 1) / BC][(n + 1) % BC]; }
     const int fa = (j == 0) ? NC - 1 : (step + j) % (NC - 1), fb = (j == 0) ? step : (step - j + (NC - 1)) % (NC - 1);
     const int c0 = FULL ? (fa < fb ? fa : fb) : j, c1 = FULL ? (fa < fb ? fb : fa) : BC + (j + step) % BC;
-    if (rr.sn != 0.) {
+    if (fr.t1 != 0. || fr.t2 != 0.) {
       #pragma unroll
       for (int m = 0; m < ROWS; ++m) {
         const double pv = x[c0][m], qv = x[c1][m];
-        x[c0][m] = rr.cs * pv - rr.a * qv; x[c1][m] = rr.sn * pv + rr.b * qv;
+        x[c0][m] = fma(-fr.t1, qv, pv); x[c1][m] = fma(fr.t2, pv, qv);
       }
     }
+  }
+  #pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const double sc = scale[c];
+    #pragma unroll
+    for (int m = 0; m < ROWS; ++m) { x[c][m] *= sc; }
   }
   #pragma unroll
   for (int c = 0; c < NC; ++c) {
