@@ -550,6 +550,156 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
   }
 }
 
+/* The same round for complex factors.  The Gram matrix is Hermitian, G[c0][c1] = x_c0^H x_c1: NC (NC + 1) / 2 real parts
+ * and NC (NC - 1) / 2 imaginary parts, NC^2 sums in all.  A rotation is x_c0' = cs x_c0 - a x_c1, x_c1' = sn x_c0 + b x_c1
+ * with a = sn conj(e), b = cs conj(e), e = g / |g| (the phase that makes the cross product real): G <- J^H G J, the row
+ * side with the conjugate coefficients. */
+struct RotRecC { double cs, sn, ar, ai, br, bi; };   /* sn == 0: no rotation */
+struct Cx { double re, im; };
+__device__ __forceinline__ Cx cmul(double ar, double ai, Cx b) { return Cx{ ar * b.re - ai * b.im, ar * b.im + ai * b.re }; }
+
+template <int ROWS, int BC, bool FULL, int THREADS>
+__global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t N, int32_t nb, int32_t r, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations) {
+  constexpr int NC = 2 * BC, NG = NC * (NC + 1) / 2, NT = NC * NC, WAVES = THREADS / 64, STEPS = FULL ? NC - 1 : BC, GS = NC + 1;
+  constexpr int CH = NT >= 32 ? 32 : NT;
+  static_assert(NT % CH == 0 && CH >= 4 && BC * BC <= 64, "whole chunks; one lane of the first wavefront per pair of pairs");
+  __shared__ double part[WAVES][NT];
+  __shared__ double Gre[NC * GS], Gim[NC * GS];
+  __shared__ RotRecC rot[STEPS][BC];
+  __shared__ double fixed[BC][2];
+  __shared__ int32_t pairCol[BC][2];
+  __shared__ int32_t appliedAll;
+  const int i = blockIdx.x; int P, Q;
+  if (i == 0) { P = nb - 1; Q = round; } else { P = (round + i) % (nb - 1); Q = (round - i + (nb - 1)) % (nb - 1); }
+  if (P > Q) { const int t = P; P = Q; Q = t; }
+  int col[NC]; bool live[NC];
+  #pragma unroll
+  for (int c = 0; c < NC; ++c) { col[c] = (c < BC ? P : Q) * BC + (c % BC); live[c] = col[c] < r; }
+  if (!live[0]) { return; }
+  double x[NC][ROWS][2];
+  #pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    #pragma unroll
+    for (int m = 0; m < ROWS; ++m) {
+      const int k = threadIdx.x + m * THREADS;
+      #pragma unroll
+      for (int w = 0; w < 2; ++w) { x[c][m][w] = (live[c] && k < N) ? B[((int64_t)col[c] * N + k) * 2 + w] : 0.; }
+    }
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  /* sum q < NG: real part of pair p = q; q >= NG: imaginary part of pair p = q - NG + NC (the diagonal has none); pairs
+   * numbered by diagonal as in the real kernel */
+  #pragma unroll
+  for (int chunk = 0; chunk < NT / CH; ++chunk) {
+    double v[CH];
+    #pragma unroll
+    for (int e = 0; e < CH; ++e) {
+      const int q = chunk * CH + e; const bool isIm = q >= NG; const int p = isIm ? q - NG + NC : q, c0 = p % NC, c1 = (c0 + p / NC) % NC;
+      double sum = 0.;
+      #pragma unroll
+      for (int m = 0; m < ROWS; ++m) {
+        if (isIm) { sum += x[c0][m][0] * x[c1][m][1] - x[c0][m][1] * x[c1][m][0]; }
+        else { sum += x[c0][m][0] * x[c1][m][0] + x[c0][m][1] * x[c1][m][1]; }
+      }
+      v[e] = sum;
+    }
+    const double tot = wave_sum_swap<CH>(v);
+    if ((lane & (64 / CH - 1)) == 0) { part[wave][chunk * CH + lane / (64 / CH)] = tot; }
+  }
+  __syncthreads();
+  if (wave == 0) {
+    for (int idx = lane; idx < NT; idx += 64) {
+      double tot = 0.;
+      #pragma unroll
+      for (int w = 0; w < WAVES; ++w) { tot += part[w][idx]; }
+      const bool isIm = idx >= NG; const int p = isIm ? idx - NG + NC : idx, c0 = p % NC, c1 = (c0 + p / NC) % NC;
+      if (isIm) { Gim[c0 * GS + c1] = tot; Gim[c1 * GS + c0] = -tot; }
+      else { Gre[c0 * GS + c1] = tot; Gre[c1 * GS + c0] = tot; if (c0 == c1) { Gim[c0 * GS + c0] = 0.; } }
+    }
+    wave_lds_sync();
+    int applied = 0; double worst = 0.;
+    for (int step = 0; step < STEPS; ++step) {
+      if (lane < BC) {
+        const int j = lane;
+        int c0, c1;
+        if constexpr (FULL) {
+          const int fa = (j == 0) ? NC - 1 : (step + j) % (NC - 1), fb = (j == 0) ? step : (step - j + (NC - 1)) % (NC - 1);
+          c0 = fa < fb ? fa : fb; c1 = fa < fb ? fb : fa;
+        } else { c0 = j; c1 = BC + (j + step) % BC; }
+        const double alpha = Gre[c0 * GS + c0], beta = Gre[c1 * GS + c1], gre = Gre[c0 * GS + c1], gim = Gim[c0 * GS + c1];
+        const bool pairLive = ((c0 < BC ? P : Q) * BC + (c0 % BC) < r) && ((c1 < BC ? P : Q) * BC + (c1 % BC) < r);
+        const double g2 = gre * gre + gim * gim;
+        if (pairLive) {
+          const double ab = alpha * beta;
+          if (ab > 0.) { if (g2 > worst * ab) { worst = g2 / ab; } } else if (g2 > 0.) { worst = fmax(worst, 1.); }
+        }
+        const bool rotate = pairLive && g2 > tol * tol * alpha * beta && g2 > 0.;
+        RotRecC rr = { 1., 0., 0., 0., 1., 0. }; double na = alpha, nbeta = beta;
+        if (rotate) {
+          const double gabs = sqrt(g2), inv = 1. / gabs, er = gre * inv, ei = gim * inv, d = beta - alpha, h = 2. * gabs;
+          const int e = __builtin_amdgcn_frexp_exp(fmax(fabs(d), h));
+          const double ds = ldexp(fabs(d), -e), hs = ldexp(h, -e);
+          const double t = copysign(hs / (ds + sqrt(ds * ds + hs * hs)), d);
+          const double cs = rsqrt(1. + t * t), sn = cs * t, shift = t * gabs;
+          rr.cs = cs; rr.sn = sn; rr.ar = sn * er; rr.ai = -sn * ei; rr.br = cs * er; rr.bi = -cs * ei;
+          na = alpha - shift; nbeta = beta + shift;
+          if (sn != 0.) { ++applied; }
+        }
+        rot[step][j] = rr; fixed[j][0] = na; fixed[j][1] = nbeta; pairCol[j][0] = c0; pairCol[j][1] = c1;
+      }
+      wave_lds_sync();
+      if (lane < BC * BC) {
+        const int jr = lane / BC, jc = lane % BC, r0 = pairCol[jr][0], r1 = pairCol[jr][1], k0 = pairCol[jc][0], k1 = pairCol[jc][1];
+        const RotRecC rw = rot[step][jr], cl = rot[step][jc];
+        const Cx g00 = { Gre[r0 * GS + k0], Gim[r0 * GS + k0] }, g01 = { Gre[r0 * GS + k1], Gim[r0 * GS + k1] };
+        const Cx g10 = { Gre[r1 * GS + k0], Gim[r1 * GS + k0] }, g11 = { Gre[r1 * GS + k1], Gim[r1 * GS + k1] };
+        /* columns: h_x0 = cs g_x0 - a g_x1, h_x1 = sn g_x0 + b g_x1 */
+        const Cx a01 = cmul(cl.ar, cl.ai, g01), a11 = cmul(cl.ar, cl.ai, g11), b01 = cmul(cl.br, cl.bi, g01), b11 = cmul(cl.br, cl.bi, g11);
+        const Cx h00 = { cl.cs * g00.re - a01.re, cl.cs * g00.im - a01.im }, h01 = { cl.sn * g00.re + b01.re, cl.sn * g00.im + b01.im };
+        const Cx h10 = { cl.cs * g10.re - a11.re, cl.cs * g10.im - a11.im }, h11 = { cl.sn * g10.re + b11.re, cl.sn * g10.im + b11.im };
+        /* rows: y_0k = cs h_0k - conj(a) h_1k, y_1k = sn h_0k + conj(b) h_1k */
+        const Cx c10 = cmul(rw.ar, -rw.ai, h10), c11 = cmul(rw.ar, -rw.ai, h11), d10 = cmul(rw.br, -rw.bi, h10), d11 = cmul(rw.br, -rw.bi, h11);
+        Cx y00 = { rw.cs * h00.re - c10.re, rw.cs * h00.im - c10.im }, y01 = { rw.cs * h01.re - c11.re, rw.cs * h01.im - c11.im };
+        Cx y10 = { rw.sn * h00.re + d10.re, rw.sn * h00.im + d10.im }, y11 = { rw.sn * h01.re + d11.re, rw.sn * h01.im + d11.im };
+        if (jr == jc && rw.sn != 0.) { y00 = Cx{ fixed[jr][0], 0. }; y11 = Cx{ fixed[jr][1], 0. }; y01 = Cx{ 0., 0. }; y10 = Cx{ 0., 0. }; }
+        Gre[r0 * GS + k0] = y00.re; Gim[r0 * GS + k0] = y00.im; Gre[r0 * GS + k1] = y01.re; Gim[r0 * GS + k1] = y01.im;
+        Gre[r1 * GS + k0] = y10.re; Gim[r1 * GS + k0] = y10.im; Gre[r1 * GS + k1] = y11.re; Gim[r1 * GS + k1] = y11.im;
+      }
+      wave_lds_sync();
+    }
+    #pragma unroll
+    for (int off = BC / 2; off > 0; off >>= 1) { worst = fmax(worst, __shfl_xor(worst, off, 64)); applied += __shfl_xor(applied, off, 64); }
+    if (lane == 0) { report_cosine(rotations, worst); appliedAll = applied; if (applied > 0) { atomicAdd(rotations, applied); } }
+  }
+  __syncthreads();
+  if (appliedAll == 0) { return; }
+  RotRecC cur = rot[0][0];
+  #pragma unroll
+  for (int n = 0; n < STEPS * BC; ++n) {
+    const int step = n / BC, j = n % BC;
+    const RotRecC rr = cur;
+    if (n + 1 < STEPS * BC) { cur = rot[(n + 1) / BC][(n + 1) % BC]; }
+    const int fa = (j == 0) ? NC - 1 : (step + j) % (NC - 1), fb = (j == 0) ? step : (step - j + (NC - 1)) % (NC - 1);
+    const int c0 = FULL ? (fa < fb ? fa : fb) : j, c1 = FULL ? (fa < fb ? fb : fa) : BC + (j + step) % BC;
+    if (rr.sn != 0.) {
+      #pragma unroll
+      for (int m = 0; m < ROWS; ++m) {
+        const double pr = x[c0][m][0], pi = x[c0][m][1]; const Cx q = { x[c1][m][0], x[c1][m][1] };
+        const Cx aq = cmul(rr.ar, rr.ai, q), bq = cmul(rr.br, rr.bi, q);
+        x[c0][m][0] = rr.cs * pr - aq.re; x[c0][m][1] = rr.cs * pi - aq.im; x[c1][m][0] = rr.sn * pr + bq.re; x[c1][m][1] = rr.sn * pi + bq.im;
+      }
+    }
+  }
+  #pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    #pragma unroll
+    for (int m = 0; m < ROWS; ++m) {
+      const int k = threadIdx.x + m * THREADS;
+      if (live[c] && k < N) { B[((int64_t)col[c] * N + k) * 2] = x[c][m][0]; B[((int64_t)col[c] * N + k) * 2 + 1] = x[c][m][1]; }
+    }
+  }
+}
+
 template <bool CPLX>
 __global__ __launch_bounds__(T_THREADS) void column_norm_kernel(int32_t N, const double* __restrict__ B, double* __restrict__ sigma) {
   __shared__ double scratch[T_THREADS / 64]; constexpr int W = CPLX ? 2 : 1;
@@ -654,13 +804,21 @@ extern "C" int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t
 }
 
 /* one sweep = every pair of the r columns of B (N x r, FP64, complex interleaved) once; rotations counts the rotations applied */
-static int g_jacobiVariant = 0;   /* 0: Gram-space rounds for real factors, 8-column blocks where they fit (default); 1: the step kernel everywhere; 2: Gram-space rounds, 4-column blocks */
+static int g_jacobiVariant = 0;   /* 0: Gram-space rounds, 8-column blocks for real factors where they fit (default); 1: the step kernel everywhere; 2: Gram-space rounds, 4-column blocks */
 
 template <int ROWS, int BC, int THREADS = T_THREADS>
 static int gram_sweep(hipStream_t stream, int32_t N, int32_t r, double* B, double tol, int32_t* rotations) {
   const int blocks = (r + BC - 1) / BC, nb = (blocks + 1) & ~1;
   jacobi_gram_round_kernel<ROWS, BC, true, THREADS><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations);
   for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations); }
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+template <int ROWS, int BC, int THREADS = T_THREADS>
+static int gram_sweep_cplx(hipStream_t stream, int32_t N, int32_t r, double* B, double tol, int32_t* rotations) {
+  const int blocks = (r + BC - 1) / BC, nb = (blocks + 1) & ~1;
+  jacobi_gram_round_cplx_kernel<ROWS, BC, true, THREADS><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations);
+  for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_cplx_kernel<ROWS, BC, false, THREADS><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations); }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
@@ -692,6 +850,11 @@ extern "C" int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, in
     if (N <= 4 * T_THREADS) { return blocked_sweep<false, 4, 4>(stream, N, r, B, tol, rotations); }
     if (N <= 8 * T_THREADS) { return blocked_sweep<false, 8, 4>(stream, N, r, B, tol, rotations); }
     if (N <= 8 * 512) { return blocked_sweep<false, 8, 4, 512>(stream, N, r, B, tol, rotations); }
+  }
+  if (Complex && r >= 16 && g_jacobiVariant != 1) {
+    if (N <= 4 * T_THREADS) { return gram_sweep_cplx<4, 4>(stream, N, r, B, tol, rotations); }
+    if (N <= 4 * 512) { return gram_sweep_cplx<4, 4, 512>(stream, N, r, B, tol, rotations); }
+    if (N <= 8 * 512) { return gram_sweep_cplx<8, 2, 512>(stream, N, r, B, tol, rotations); }
   }
   if (Complex && r >= 16) {
     if (N <= 4 * T_THREADS) { return blocked_sweep<true, 4, 4>(stream, N, r, B, tol, rotations); }

@@ -84,11 +84,11 @@ int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t Gtype, con
  * tol is rotated.  rotations: 16 bytes of device memory, zero before the call; afterwards rotations[0] = pairs rotated and
  * the double at rotations + 2 = the largest squared cosine the sweep met (rotated or not). */
 int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations);
-/* Which kernel a sweep over a real factor runs: 0 (default) one Gram matrix per round and workgroup, the steps of the round
- * taken on it by one wavefront, blocks of 8 columns where N <= 2048 and of 4 above; 1 one reduction and barrier per step
- * (what complex factors always run); 2 as 0 with blocks of 4 columns throughout.  All rotate by the same rule, 0 and 2
- * visit the pairs in the order of 1 for equal block sizes; kept selectable so that tests cover every kernel.  Process-wide,
- * not thread-safe. */
+/* Which kernel a sweep runs: 0 (default) one Gram matrix per round and workgroup, the steps of the round taken on it by
+ * one wavefront; real factors in blocks of 8 columns where N <= 2048 and of 4 above, complex ones in blocks of 4 and 2;
+ * 1 one reduction and barrier per step; 2 as 0 with blocks of 4 columns for real factors throughout.  All rotate by the
+ * same rule, and for equal block sizes they visit the pairs in the same order; kept selectable so that tests cover every
+ * kernel.  Process-wide, not thread-safe. */
 int hykJacobiSetVariant(int32_t variant);
 int hykColumnNorms(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, const double* B, double* sigma);
 int hykBasisOut(hipStream_t stream, int32_t N, int32_t rank, int32_t Atype, const double* B, const double* sigma, const int32_t* order, void* X, int64_t ldx);

@@ -418,7 +418,7 @@ def test_gemm_fp64(gl, cplx, opA, opB, M, N, K):
 
 
 @pytest.mark.parametrize("variant", [0, 1, 2])
-@pytest.mark.parametrize("cplx,N,r", [(0, 300, 40), (0, 1000, 130), (0, 2048, 96), (0, 2500, 70), (1, 600, 50), (0, 64, 64), (0, 700, 20)])
+@pytest.mark.parametrize("cplx,N,r", [(0, 300, 40), (0, 1000, 130), (0, 2048, 96), (0, 2500, 70), (1, 600, 50), (1, 2048, 40), (1, 3000, 24), (0, 64, 64), (0, 700, 20)])
 def test_jacobi_sweep_kernels(gl, variant, cplx, N, r):
     """One-sided Jacobi sweeps on a graded N x r factor: every kernel behind hykJacobiSweep (Gram-space rounds with blocks
     of 8 and of 4 columns, the step kernel, the pair kernel for few columns) must leave orthogonal columns whose norms are
