@@ -16,6 +16,7 @@
 #include <numeric>
 #include <cfloat>
 #include "common.hpp"
+#include "jacobi_stop.hpp"
 
 namespace {
 
@@ -82,21 +83,9 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
       HYH_KERNEL(hykJacobiSweep(s, Complex, N, rank, B.as<double>(), rotateAbove, counter.as<int32_t>())); ++used;
       struct { int32_t rotations, pad; double cosine2; } seen = { 0, 0, 0. };
       HYH_CHECK(hipMemcpyAsync(&seen, counter.p, sizeof(seen), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
-      /* Done when nothing was rotated, or when every cosine the sweep met was within 8 thresholds: rotating such pairs
-       * moves the other cosines by products of two of them, so the sweep has left all of them at the threshold's level
-       * and a further sweep would only confirm it. */
       if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: %d rotations, largest cosine %.2le\n", used, seen.rotations, std::sqrt(seen.cosine2)); }
-      if (seen.rotations == 0 || seen.cosine2 <= 64. * rotateAbove * rotateAbove) { break; }
-      /* Or when the sweeps have reached their quadratic phase and the next one could only confirm: the largest cosine
-       * c_k of this sweep against c_{k-1}^2 of the one before gives the constant of the contraction as it is here
-       * (clusters of singular values make it larger); if that constant is moderate and, applied once more, puts the
-       * cosines this sweep has left behind (constant x c_k^2) within the same 8 thresholds, the columns are there. */
-      const double c2 = seen.cosine2;
-      if (lastCosine2 > 0. && c2 > 0.) {
-        const double contraction = std::max(1., std::sqrt(c2) / lastCosine2);   /* c_k / c_{k-1}^2 */
-        if (contraction <= 16. && contraction * c2 <= 8. * rotateAbove) { break; }
-      }
-      lastCosine2 = c2;
+      if (hyh::jacobi_sweeps_done(seen.rotations, seen.cosine2, lastCosine2, rotateAbove)) { break; }
+      lastCosine2 = seen.cosine2;
     }
     HYH_KERNEL(hykColumnNorms(s, Complex, N, rank, B.as<double>(), sigma.as<double>()));
     std::vector<double> sig((size_t)rank); HYH_CHECK(hipMemcpyAsync(sig.data(), sigma.p, sizeof(double) * (size_t)rank, hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));

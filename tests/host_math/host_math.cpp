@@ -3,6 +3,7 @@
 #include <cstring>
 #include "hyk_common.h"
 #include "crt_tables.h"
+#include "host/jacobi_stop.hpp"
 
 using namespace hyk;
 
@@ -90,5 +91,8 @@ void hm_crt_lift(int cplxTable, int order, const uint32_t* residues, uint64_t* w
   if (!i192_is_neg(diff)) { i192_add(a, i192_neg(P)); }
   words[0] = a.w[0]; words[1] = a.w[1]; words[2] = a.w[2];
 }
+
+/* the host's rule for ending the Jacobi sweeps of the SVD tail */
+int hm_jacobi_done(int rotations, double cosine2, double lastCosine2, double rotateAbove) { return hyh::jacobi_sweeps_done(rotations, cosine2, lastCosine2, rotateAbove) ? 1 : 0; }
 
 }

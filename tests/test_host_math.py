@@ -16,11 +16,14 @@ LIB = os.path.join(ROOT, "tests", "host_math", "libhost_math.so")
 @pytest.fixture(scope="module")
 def hm():
     hdr = os.path.join(ROOT, "hyacinth_amd", "csrc", "hyk_common.h")
-    if not os.path.exists(LIB) or os.path.getmtime(LIB) < max(os.path.getmtime(SRC), os.path.getmtime(hdr)):
+    stop = os.path.join(ROOT, "hyacinth_amd", "csrc", "host", "jacobi_stop.hpp")
+    if not os.path.exists(LIB) or os.path.getmtime(LIB) < max(os.path.getmtime(SRC), os.path.getmtime(hdr), os.path.getmtime(stop)):
         subprocess.check_call(["g++", "-O2", "-std=c++17", "-shared", "-fPIC", "-I", os.path.join(ROOT, "hyacinth_amd", "csrc"), SRC, "-o", LIB])
     L = C.CDLL(LIB)
     L.hm_frexp.restype = C.c_int32
     L.hm_reduce_i32.restype = C.c_int32
+    L.hm_jacobi_done.argtypes = [C.c_int, C.c_double, C.c_double, C.c_double]
+    L.hm_jacobi_done.restype = C.c_int
     return L
 
 
@@ -169,3 +172,34 @@ def test_crt_lift(hm, table, moduli):
             got = sum(int(words[k]) << (64 * k) for k in range(3))
             got -= (1 << 192) if got >= (1 << 191) else 0
             assert got == v, (order, v)
+
+
+def test_jacobi_stop_rule(hm):
+    """When the host ends the Jacobi sweeps (host/jacobi_stop.hpp): sequences of (rotations, largest cosine) per sweep as
+    the kernels report them, with the sweep after which the iteration must end."""
+    def sweeps_run(cosines, rotations, tol):
+        last = 0.0
+        for k, (c, n) in enumerate(zip(cosines, rotations)):
+            if hm.hm_jacobi_done(n, c * c, last, tol):
+                return k + 1
+            last = c * c
+        return None
+    # real FP64 2048 columns, eps 1e-12 (threshold eps / 16): quadratic from the third sweep on, 2 x (3.27e-7)^2 = 2.1e-13 <= 8 thresholds
+    assert sweeps_run([1.17e-2, 4.24e-3, 4.08e-4, 3.27e-7, 6.25e-14], [2096107, 2094368, 1781819, 108880, 0], 6.25e-14) == 4
+    # FP32 storage, eps 1e-5
+    assert sweeps_run([1.58e-2, 2.38e-3, 4.54e-5, 6.25e-7], [184760, 116616, 1190, 0], 6.25e-7) == 3
+    # complex FP64, eps 1e-12
+    assert sweeps_run([8.70e-3, 2.62e-3, 9.31e-5, 5.59e-8, 6.25e-14], [2096128, 2095717, 1811563, 109586, 0], 6.25e-14) == 4
+    # not yet contracting quadratically (constant above 16): no early end, the confirming sweep runs
+    assert sweeps_run([1e-2, 5e-3, 1e-6, 1e-15], [1000, 900, 800, 0], 1e-14) == 4
+    # contraction fine but the predicted cosines still above 8 thresholds
+    assert hm.hm_jacobi_done(800, (1e-7) ** 2, (1e-4) ** 2, 1e-15) == 0        # constant 10, predicted 1e-13 > 8e-15
+    assert hm.hm_jacobi_done(800, (1e-7) ** 2, (1e-4) ** 2, 2e-14) == 1        # 1e-13 <= 1.6e-13
+    assert sweeps_run([1e-2, 1e-4, 1e-7, 1e-13, 1e-15], [1000, 900, 800, 10, 0], 1e-15) == 4
+    # a sweep that met nothing above 8 thresholds ends the iteration even though it rotated
+    assert hm.hm_jacobi_done(5, (7e-14) ** 2, 0.0, 1e-14) == 1
+    assert hm.hm_jacobi_done(5, (9e-14) ** 2, 0.0, 1e-14) == 0
+    # nothing rotated
+    assert hm.hm_jacobi_done(0, 0.25, 0.0, 1e-14) == 1
+    # first sweep never ends on the contraction rule (no sweep before it)
+    assert hm.hm_jacobi_done(10, 1e-20, 0.0, 1e-14) == 0
