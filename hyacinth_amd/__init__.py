@@ -31,7 +31,7 @@ API_SYMBOLS = [
 KERNEL_SYMBOLS = [
     "hykColumnExponents", "hykSliceRange", "hykQuantizeLimbs", "hykQuantizeCrt", "hykZeroRows",
     "hykGramWorkspaceBytes", "hykGramWorkspaceClear", "hykGramCrt", "hykGramLimbs", "hykGramSetSlab",
-    "hykGramProfile", "hykGramProfileRead", "hykMfmaCeiling", "hykGramRange", "hykDequantize", "hykPotrfpWorkspaceBytes", "hykPotrfp", "hykFactorToB", "hykJacobiSweep", "hykJacobiSetVariant",
+    "hykGramProfile", "hykGramProfileRead", "hykMfmaCeiling", "hykGramRange", "hykDequantize", "hykPotrfpWorkspaceBytes", "hykPotrfp", "hykFactorToB", "hykJacobiSweep", "hykJacobiSweepCarry", "hykJacobiCarryBytes", "hykJacobiSetVariant",
     "hykColumnNorms", "hykBasisOut", "hykValuesOut", "hykInterpSolve", "hykInterpOut", "hykMatcopy",
     "hykSumSquares", "hykMatmulCf16", "hykGemm", "hykOrthonormalize",
 ]
@@ -89,6 +89,8 @@ def lib():
         L.hykGramSetSlab.argtypes = [i32]
         L.hykJacobiSetVariant.argtypes = [i32]
         L.hykJacobiSweep.argtypes = [vp, i32, i32, i32, vp, dbl, vp]
+        L.hykJacobiSweepCarry.argtypes = [vp, i32, i32, i32, vp, dbl, vp, vp]
+        L.hykJacobiCarryBytes.argtypes = [i32]; L.hykJacobiCarryBytes.restype = C.c_size_t
         L.hykGramProfile.argtypes = [i32]
         L.hykGramProfileRead.argtypes = [C.POINTER(dbl), C.POINTER(i32)]
         L.hykMfmaCeiling.argtypes = [vp, i32, i32, i32, C.POINTER(dbl), C.POINTER(dbl)]

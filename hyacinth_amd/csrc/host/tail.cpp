@@ -69,7 +69,7 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
     rank = run_potrfp(handle, f, lrqr ? eps : 0., N, N, jpiv.as<int32_t>());
     if (rank <= 0) { return rank; }
     /* B = (R P^T)^H, N x rank, FP64 */
-    hyh::Scratch B(handle, (size_t)N * rank * 8 * (1 + Complex)), sigma(handle, sizeof(double) * (size_t)rank), counter(handle, 64);
+    hyh::Scratch B(handle, (size_t)N * rank * 8 * (1 + Complex)), sigma(handle, sizeof(double) * (size_t)rank), counter(handle, 64), carry(handle, hykJacobiCarryBytes(rank));
     HYH_KERNEL(hykFactorToB(s, N, rank, f.type, f.Rt.p, f.ldr, B.as<double>()));
     const int32_t maxSweeps = sweeps > 0 ? 5 * sweeps : 30; int32_t used = 0;
     /* A pair is rotated while its cosine exceeds the storage precision, but never below sqrt(N) FP64 roundings: that is
@@ -80,7 +80,7 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
     double lastCosine2 = 0.;
     for (int32_t sw = 0; sw < maxSweeps && rank > 1; ++sw) {
       HYH_KERNEL(hykGramWorkspaceClear(s, counter.p, 64));
-      HYH_KERNEL(hykJacobiSweep(s, Complex, N, rank, B.as<double>(), rotateAbove, counter.as<int32_t>())); ++used;
+      HYH_KERNEL(hykJacobiSweepCarry(s, Complex, N, rank, B.as<double>(), rotateAbove, counter.as<int32_t>(), carry.as<double>())); ++used;
       struct { int32_t rotations, pad; double cosine2; } seen = { 0, 0, 0. };
       HYH_CHECK(hipMemcpyAsync(&seen, counter.p, sizeof(seen), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
       if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: %d rotations, largest cosine %.2le\n", used, seen.rotations, std::sqrt(seen.cosine2)); }

@@ -397,12 +397,27 @@ __device__ __forceinline__ void wave_lds_sync() {   /* LDS operations of one wav
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
-template <int ROWS, int BC, bool FULL, int THREADS>
-__global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, int32_t nb, int32_t r, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations) {
+/* CARRY: the products inside a block (x_i . x_j, i < j in the same block of BC columns) travel with the block from round
+ * to round in `carry` (BC (BC - 1) / 2 doubles per block) instead of being summed again: the first round of a sweep (FULL)
+ * sums everything and writes them, the other rounds sum the norms and the BC^2 cross products only (80 of 136 products
+ * for BC = 8) and take the rest from the small matrix as the previous round's steps left it.  The norms and the cross
+ * products, which decide every rotation of the round, are always fresh; what is carried only feeds the update of cross
+ * products inside a round, multiplied by the sine of a rotation. */
+template <int BC> __device__ __forceinline__ void carried_pair(int t, int& i, int& j) { i = 0; while (t >= BC - 1 - i) { t -= BC - 1 - i; ++i; } j = i + 1 + t; }
+
+template <int ROWS, int BC, bool FULL, int THREADS, bool CARRY>
+__global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, int32_t nb, int32_t r, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations, double* __restrict__ carry) {
   constexpr int NC = 2 * BC, NG = NC * (NC + 1) / 2, WAVES = THREADS / 64, STEPS = FULL ? NC - 1 : BC, GS = NC + 1;
-  constexpr int CH = NG >= 32 ? 32 : NG, TAIL = NG % CH;
-  static_assert((TAIL & (TAIL - 1)) == 0 && BC * BC <= 64, "tail chunk a power of two; one lane of the first wavefront per pair of pairs");
-  __shared__ double part[WAVES][NG];
+  constexpr bool SLIM = CARRY && !FULL;                    /* norms and cross products only */
+  constexpr int NW = BC * (BC - 1) / 2, NP = SLIM ? NC + BC * BC : NG;
+  constexpr int CH = NP >= 32 ? 32 : 16, TAIL = NP % CH;
+  static_assert((TAIL & (TAIL - 1)) == 0 && (TAIL == 0 || TAIL >= 4) && BC * BC <= 64 && 2 * NW <= 64, "tail chunk a power of two; one lane of the first wavefront per pair of pairs and per carried product");
+  auto pair_of = [](int p, int& c0, int& c1) {
+    if (!SLIM) { c0 = p % NC; c1 = (c0 + p / NC) % NC; }
+    else if (p < NC) { c0 = p; c1 = p; }
+    else { c0 = (p - NC) / BC; c1 = BC + (p - NC) % BC; }
+  };
+  __shared__ double part[WAVES][NP];
   __shared__ double Gs[NC * GS];
   __shared__ RotRec rot[STEPS][BC];
   __shared__ FastRot fast[STEPS][BC];
@@ -417,21 +432,23 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
   #pragma unroll
   for (int c = 0; c < NC; ++c) { col[c] = (c < BC ? P : Q) * BC + (c % BC); live[c] = col[c] < r; }
   if (!live[0]) { return; }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  [[maybe_unused]] double carried = 0.;
+  if constexpr (SLIM) { if (wave == 0 && lane < 2 * NW) { carried = carry[(int64_t)(lane < NW ? P : Q) * NW + lane % NW]; } }
   double x[NC][ROWS];
   #pragma unroll
   for (int c = 0; c < NC; ++c) {
     #pragma unroll
     for (int m = 0; m < ROWS; ++m) { const int k = threadIdx.x + m * THREADS; x[c][m] = (live[c] && k < N) ? B[(int64_t)col[c] * N + k] : 0.; }
   }
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   /* products numbered by diagonal: p = d NC + c stands for (c, (c + d) % NC), d = 0 .. NC / 2 (the last diagonal only for
    * c < NC / 2): every unordered pair once, and p splits back into the pair by shifts.  Summed over the wavefront 32 at a time. */
   #pragma unroll
-  for (int chunk = 0; chunk < NG / CH; ++chunk) {
+  for (int chunk = 0; chunk < NP / CH; ++chunk) {
     double v[CH];
     #pragma unroll
     for (int q = 0; q < CH; ++q) {
-      const int p = chunk * CH + q, c0 = p % NC, c1 = (c0 + p / NC) % NC;
+      int c0 = 0, c1 = 0; pair_of(chunk * CH + q, c0, c1);
       double sum = 0.;
       #pragma unroll
       for (int m = 0; m < ROWS; ++m) { sum += x[c0][m] * x[c1][m]; }
@@ -444,23 +461,26 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
     double v[TAIL];
     #pragma unroll
     for (int q = 0; q < TAIL; ++q) {
-      const int p = (NG / CH) * CH + q, c0 = p % NC, c1 = (c0 + p / NC) % NC;
+      int c0 = 0, c1 = 0; pair_of((NP / CH) * CH + q, c0, c1);
       double sum = 0.;
       #pragma unroll
       for (int m = 0; m < ROWS; ++m) { sum += x[c0][m] * x[c1][m]; }
       v[q] = sum;
     }
     const double tot = wave_sum_swap<TAIL>(v);
-    if ((lane & (64 / TAIL - 1)) == 0) { part[wave][(NG / CH) * CH + lane / (64 / TAIL)] = tot; }
+    if ((lane & (64 / TAIL - 1)) == 0) { part[wave][(NP / CH) * CH + lane / (64 / TAIL)] = tot; }
   }
   __syncthreads();
   if (wave == 0) {
-    for (int idx = lane; idx < NG; idx += 64) {
+    for (int idx = lane; idx < NP; idx += 64) {
       double tot = 0.;
       #pragma unroll
       for (int w = 0; w < WAVES; ++w) { tot += part[w][idx]; }
-      const int c0 = idx % NC, c1 = (c0 + idx / NC) % NC;
+      int c0 = 0, c1 = 0; pair_of(idx, c0, c1);
       Gs[c0 * GS + c1] = tot; Gs[c1 * GS + c0] = tot;
+    }
+    if constexpr (SLIM) {
+      if (lane < 2 * NW) { int ci, cj; carried_pair<BC>(lane % NW, ci, cj); const int base = lane < NW ? 0 : BC; Gs[(base + ci) * GS + base + cj] = carried; Gs[(base + cj) * GS + base + ci] = carried; }
     }
     if (lane < NC) { scale[lane] = 1.; }
     wave_lds_sync();
@@ -517,6 +537,9 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
     #pragma unroll
     for (int off = BC / 2; off > 0; off >>= 1) { worst = fmax(worst, __shfl_xor(worst, off, 64)); applied += __shfl_xor(applied, off, 64); }
     if (lane == 0) { report_cosine(rotations, worst); appliedAll = applied; if (applied > 0) { atomicAdd(rotations, applied); } }
+    if constexpr (CARRY) {   /* the products inside the two blocks as the steps have left them */
+      if (lane < 2 * NW) { int ci, cj; carried_pair<BC>(lane % NW, ci, cj); const int base = lane < NW ? 0 : BC; carry[(int64_t)(lane < NW ? P : Q) * NW + lane % NW] = Gs[(base + ci) * GS + base + cj]; }
+    }
   }
   __syncthreads();
   if (appliedAll == 0) { return; }
@@ -807,10 +830,15 @@ extern "C" int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t
 static int g_jacobiVariant = 0;   /* 0: Gram-space rounds, 8-column blocks for real factors where they fit (default); 1: the step kernel everywhere; 2: Gram-space rounds, 4-column blocks */
 
 template <int ROWS, int BC, int THREADS = T_THREADS>
-static int gram_sweep(hipStream_t stream, int32_t N, int32_t r, double* B, double tol, int32_t* rotations) {
+static int gram_sweep(hipStream_t stream, int32_t N, int32_t r, double* B, double tol, int32_t* rotations, double* carry) {
   const int blocks = (r + BC - 1) / BC, nb = (blocks + 1) & ~1;
-  jacobi_gram_round_kernel<ROWS, BC, true, THREADS><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations);
-  for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations); }
+  if (carry) {
+    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, true><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations, carry);
+    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, true><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations, carry); }
+  } else {
+    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, false><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations, nullptr);
+    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, false><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations, nullptr); }
+  }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
@@ -832,19 +860,23 @@ static int blocked_sweep(hipStream_t stream, int32_t N, int32_t r, double* B, do
 
 extern "C" int hykJacobiSetVariant(int32_t variant) { if (variant < 0 || variant > 2) { return -1; } g_jacobiVariant = variant; return 0; }
 
-extern "C" int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations) {
+extern "C" size_t hykJacobiCarryBytes(int32_t r) { return r <= 0 ? 0 : ((size_t)r / 4 + 2) * 28 * sizeof(double); }
+
+extern "C" int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations) { return hykJacobiSweepCarry(stream, Complex, N, r, B, tol, rotations, nullptr); }
+
+extern "C" int hykJacobiSweepCarry(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations, double* carry) {
   if (N <= 0 || r <= 1) { return 0; }
   /* blocked kernel when the rows of two column blocks fit the registers of a workgroup */
   /* real factors: Gram-space rounds; blocks of 8 columns where the rows of 16 columns fit the registers of 512 threads
    * (half as many rounds, each 1.4 times as long at N = 2048), blocks of 4 otherwise */
   if (!Complex && r >= 32 && g_jacobiVariant == 0) {
-    if (N <= 2 * 512) { return gram_sweep<2, 8, 512>(stream, N, r, B, tol, rotations); }
-    if (N <= 4 * 512) { return gram_sweep<4, 8, 512>(stream, N, r, B, tol, rotations); }
+    if (N <= 2 * 512) { return gram_sweep<2, 8, 512>(stream, N, r, B, tol, rotations, carry); }
+    if (N <= 4 * 512) { return gram_sweep<4, 8, 512>(stream, N, r, B, tol, rotations, carry); }
   }
   if (!Complex && r >= 16 && g_jacobiVariant != 1) {
-    if (N <= 4 * T_THREADS) { return gram_sweep<4, 4>(stream, N, r, B, tol, rotations); }
-    if (N <= 8 * T_THREADS) { return gram_sweep<8, 4>(stream, N, r, B, tol, rotations); }
-    if (N <= 8 * 512) { return gram_sweep<8, 4, 512>(stream, N, r, B, tol, rotations); }
+    if (N <= 4 * T_THREADS) { return gram_sweep<4, 4>(stream, N, r, B, tol, rotations, carry); }
+    if (N <= 8 * T_THREADS) { return gram_sweep<8, 4>(stream, N, r, B, tol, rotations, carry); }
+    if (N <= 8 * 512) { return gram_sweep<8, 4, 512>(stream, N, r, B, tol, rotations, carry); }
   }
   if (!Complex && r >= 16) {
     if (N <= 4 * T_THREADS) { return blocked_sweep<false, 4, 4>(stream, N, r, B, tol, rotations); }

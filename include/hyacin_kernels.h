@@ -84,6 +84,11 @@ int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t Gtype, con
  * tol is rotated.  rotations: 16 bytes of device memory, zero before the call; afterwards rotations[0] = pairs rotated and
  * the double at rotations + 2 = the largest squared cosine the sweep met (rotated or not). */
 int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations);
+/* The same sweep with hykJacobiCarryBytes(r) bytes of device memory that its rounds use to hand the products inside a
+ * column block from one round to the next instead of summing them again (real factors; ignored for complex ones and by
+ * the kernels of variant 1).  The memory needs no initialisation and holds nothing a later sweep relies on. */
+size_t hykJacobiCarryBytes(int32_t r);
+int hykJacobiSweepCarry(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations, double* carry);
 /* Which kernel a sweep runs: 0 (default) one Gram matrix per round and workgroup, the steps of the round taken on it by
  * one wavefront; real factors in blocks of 8 columns where N <= 2048 and of 4 above, complex ones in blocks of 4 and 2;
  * 1 one reduction and barrier per step; 2 as 0 with blocks of 4 columns for real factors throughout.  All rotate by the

@@ -417,11 +417,12 @@ def test_gemm_fp64(gl, cplx, opA, opB, M, N, K):
     assert np.abs(got - want).max() <= 1e-13 * np.abs(want).max() * max(1, K) ** 0.5
 
 
-@pytest.mark.parametrize("variant", [0, 1, 2])
+@pytest.mark.parametrize("variant,carry", [(0, 0), (0, 1), (1, 0), (2, 0), (2, 1)])
 @pytest.mark.parametrize("cplx,N,r", [(0, 300, 40), (0, 1000, 130), (0, 2048, 96), (0, 2500, 70), (1, 600, 50), (1, 2048, 40), (1, 3000, 24), (0, 64, 64), (0, 700, 20)])
-def test_jacobi_sweep_kernels(gl, variant, cplx, N, r):
-    """One-sided Jacobi sweeps on a graded N x r factor: every kernel behind hykJacobiSweep (Gram-space rounds with blocks
-    of 8 and of 4 columns, the step kernel, the pair kernel for few columns) must leave orthogonal columns whose norms are
+def test_jacobi_sweep_kernels(gl, variant, carry, cplx, N, r):
+    """One-sided Jacobi sweeps on a graded N x r factor: every kernel behind hykJacobiSweep / hykJacobiSweepCarry (Gram-space
+    rounds with blocks of 8 and of 4 columns, with and without the products inside a block carried from round to round in
+    memory that starts as NaN, the step kernel, the pair kernel for few columns) must leave orthogonal columns whose norms are
     the singular values numpy finds, to 32 sqrt(r) eps of the largest (a column takes part in a few hundred rotations), and
     whose span is unchanged."""
     from gpu_util import dev, host, ptr, stream, sync, zeros
@@ -431,6 +432,7 @@ def test_jacobi_sweep_kernels(gl, variant, cplx, N, r):
     B = (B @ mix) * 10.0 ** (-6.0 * np.arange(r) / r)                       # graded like a pivoted Cholesky factor
     want = np.linalg.svd(B, compute_uv=False)
     dB = dev(np.ascontiguousarray(B.T)); counter = zeros(64)
+    carried = zeros(gl.L.hykJacobiCarryBytes(r)); carried.fill_(255)       # all-ones bytes: NaN, must never be read before written
     tol = float(2.220446049250313e-16 * np.sqrt(N))
     assert gl.L.hykJacobiSetVariant(variant) == 0
     try:
@@ -438,7 +440,10 @@ def test_jacobi_sweep_kernels(gl, variant, cplx, N, r):
         while True:
             counter.zero_()
             print("jacobi", variant, cplx, N, r, "sweep", sweeps, flush=True)
-            assert gl.L.hykJacobiSweep(stream(), cplx, N, r, ptr(dB), tol, ptr(counter)) == 0
+            if carry:
+                assert gl.L.hykJacobiSweepCarry(stream(), cplx, N, r, ptr(dB), tol, ptr(counter), ptr(carried)) == 0
+            else:
+                assert gl.L.hykJacobiSweep(stream(), cplx, N, r, ptr(dB), tol, ptr(counter)) == 0
             sync(); sweeps += 1
             rotations = int(host(counter, np.int32)[0]); cos2 = float(host(counter, np.float64)[1])
             if rotations == 0:
