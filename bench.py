@@ -38,6 +38,23 @@ WORKLOADS = {
 }
 
 
+def synth_low_rank(torch, M, N, rank, noise, seed):
+    """Configuration 4's own recipe: a rank-`rank` product L R with entries complex N(0, 1 / 256) plus complex Gaussian
+    noise of size `noise`, cast to half; column-major M x N (the tensor is [N][M][re, im])."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    s = (1.0 / 512.0) ** 0.5                                   # real and imaginary part: variance 1 / 512 each
+    Lt = torch.view_as_complex(torch.randn((rank, M, 2), generator=g, device="cuda", dtype=torch.float32) * s)   # L^T
+    Rt = torch.view_as_complex(torch.randn((N, rank, 2), generator=g, device="cuda", dtype=torch.float32) * s)   # R^T
+    out = torch.empty((N, M, 2), device="cuda", dtype=torch.float16)
+    step = 512                                                  # columns per slab: keeps the FP32 product at 1 GB
+    for j in range(0, N, step):
+        P = torch.view_as_real(Rt[j:j + step] @ Lt)             # (L R)^T, rows j .. j + step
+        P.add_(torch.randn(P.shape, generator=g, device="cuda", dtype=torch.float32), alpha=noise * 0.5 ** 0.5)
+        out[j:j + step] = P.half()
+    return out
+
+
 def synth(torch, at, M, N, seed):
     """Column-scaled Gaussian test matrix generated on the device, column-major M x N."""
     g = torch.Generator(device="cuda")
@@ -127,7 +144,7 @@ def main():
     stream = torch.cuda.current_stream().cuda_stream
     h = ha.create_handle(stream=stream, GramMatrixAlgorithm=alg)
     cplx = at & 1
-    A = synth(torch, at, M, N, 0x4859)          # stored column-major M x N; opA='T' workloads are benchmarked on the transposed copy the fit makes
+    A = synth_low_rank(torch, M, N, 256, 1e-4, 0x4859) if a.workload == "cfg4" else synth(torch, at, M, N, 0x4859)          # stored column-major M x N; opA='T' workloads are benchmarked on the transposed copy the fit makes
     lda = M
     u, cP, lP, stride = ha.herk_batch_init(h, eps, M, N, at)
     seg = min(h.GramSegmentK, M) if h.GramSegmentK > 0 else M
