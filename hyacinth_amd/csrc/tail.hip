@@ -405,7 +405,10 @@ __device__ __forceinline__ void wave_lds_sync() {   /* LDS operations of one wav
  * products inside a round, multiplied by the sine of a rotation. */
 template <int BC> __device__ __forceinline__ void carried_pair(int t, int& i, int& j) { i = 0; while (t >= BC - 1 - i) { t -= BC - 1 - i; ++i; } j = i + 1 + t; }
 
-template <int ROWS, int BC, bool FULL, int THREADS, bool CARRY>
+/* PASSES = 2: factors with twice the rows that fit the registers.  The rows are taken in two halves: the sums of the first
+ * half, then of the second (which stays in registers), the steps, and the replay on the second half and then on the first,
+ * loaded again: three loads and two stores of half the rows instead of one each of all, for blocks twice as wide. */
+template <int ROWS, int BC, bool FULL, int THREADS, bool CARRY, int PASSES>
 __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, int32_t nb, int32_t r, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations, double* __restrict__ carry) {
   constexpr int NC = 2 * BC, NG = NC * (NC + 1) / 2, WAVES = THREADS / 64, STEPS = FULL ? NC - 1 : BC, GS = NC + 1;
   constexpr bool SLIM = CARRY && !FULL;                    /* norms and cross products only */
@@ -435,12 +438,18 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   [[maybe_unused]] double carried = 0.;
   if constexpr (SLIM) { if (wave == 0 && lane < 2 * NW) { carried = carry[(int64_t)(lane < NW ? P : Q) * NW + lane % NW]; } }
+  static_assert(PASSES == 1 || PASSES == 2, "all rows at once or in two halves");
   double x[NC][ROWS];
-  #pragma unroll
-  for (int c = 0; c < NC; ++c) {
+  auto load_rows = [&](int pass) {
     #pragma unroll
-    for (int m = 0; m < ROWS; ++m) { const int k = threadIdx.x + m * THREADS; x[c][m] = (live[c] && k < N) ? B[(int64_t)col[c] * N + k] : 0.; }
-  }
+    for (int c = 0; c < NC; ++c) {
+      #pragma unroll
+      for (int m = 0; m < ROWS; ++m) { const int k = threadIdx.x + (pass * ROWS + m) * THREADS; x[c][m] = (live[c] && k < N) ? B[(int64_t)col[c] * N + k] : 0.; }
+    }
+  };
+  #pragma unroll
+  for (int pass = 0; pass < PASSES; ++pass) {
+  load_rows(pass);
   /* products numbered by diagonal: p = d NC + c stands for (c, (c + d) % NC), d = 0 .. NC / 2 (the last diagonal only for
    * c < NC / 2): every unordered pair once, and p splits back into the pair by shifts.  Summed over the wavefront 32 at a time. */
   #pragma unroll
@@ -455,7 +464,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
       v[q] = sum;
     }
     const double tot = wave_sum_swap<CH>(v);
-    if ((lane & (64 / CH - 1)) == 0) { part[wave][chunk * CH + lane / (64 / CH)] = tot; }
+    if ((lane & (64 / CH - 1)) == 0) { double* slot = &part[wave][chunk * CH + lane / (64 / CH)]; *slot = pass == 0 ? tot : *slot + tot; }
   }
   if constexpr (TAIL > 0) {
     double v[TAIL];
@@ -468,8 +477,9 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
       v[q] = sum;
     }
     const double tot = wave_sum_swap<TAIL>(v);
-    if ((lane & (64 / TAIL - 1)) == 0) { part[wave][(NP / CH) * CH + lane / (64 / TAIL)] = tot; }
+    if ((lane & (64 / TAIL - 1)) == 0) { double* slot = &part[wave][(NP / CH) * CH + lane / (64 / TAIL)]; *slot = pass == 0 ? tot : *slot + tot; }
   }
+  }   /* passes */
   __syncthreads();
   if (wave == 0) {
     for (int idx = lane; idx < NP; idx += 64) {
@@ -543,7 +553,10 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
   }
   __syncthreads();
   if (appliedAll == 0) { return; }
-  /* replay the rotations on the rows of this thread (records fetched one ahead) */
+  /* replay the rotations on the rows of this thread (records fetched one ahead); the half in registers first */
+  #pragma unroll
+  for (int pass = PASSES - 1; pass >= 0; --pass) {
+  if (pass != PASSES - 1) { load_rows(pass); }
   FastRot cur = fast[0][0];
   #pragma unroll
   for (int n = 0; n < STEPS * BC; ++n) {
@@ -569,8 +582,9 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
   #pragma unroll
   for (int c = 0; c < NC; ++c) {
     #pragma unroll
-    for (int m = 0; m < ROWS; ++m) { const int k = threadIdx.x + m * THREADS; if (live[c] && k < N) { B[(int64_t)col[c] * N + k] = x[c][m]; } }
+    for (int m = 0; m < ROWS; ++m) { const int k = threadIdx.x + (pass * ROWS + m) * THREADS; if (live[c] && k < N) { B[(int64_t)col[c] * N + k] = x[c][m]; } }
   }
+  }   /* passes */
 }
 
 /* The same round for complex factors.  The Gram matrix is Hermitian, G[c0][c1] = x_c0^H x_c1: NC (NC + 1) / 2 real parts
@@ -829,15 +843,15 @@ extern "C" int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t
 /* one sweep = every pair of the r columns of B (N x r, FP64, complex interleaved) once; rotations counts the rotations applied */
 static int g_jacobiVariant = 0;   /* 0: Gram-space rounds, 8-column blocks for real factors where they fit (default); 1: the step kernel everywhere; 2: Gram-space rounds, 4-column blocks */
 
-template <int ROWS, int BC, int THREADS = T_THREADS>
+template <int ROWS, int BC, int THREADS = T_THREADS, int PASSES = 1>
 static int gram_sweep(hipStream_t stream, int32_t N, int32_t r, double* B, double tol, int32_t* rotations, double* carry) {
   const int blocks = (r + BC - 1) / BC, nb = (blocks + 1) & ~1;
   if (carry) {
-    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, true><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations, carry);
-    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, true><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations, carry); }
+    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations, carry);
+    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations, carry); }
   } else {
-    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, false><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations, nullptr);
-    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, false><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations, nullptr); }
+    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, false, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations, nullptr);
+    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, false, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations, nullptr); }
   }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
@@ -868,10 +882,11 @@ extern "C" int hykJacobiSweepCarry(hipStream_t stream, int32_t Complex, int32_t 
   if (N <= 0 || r <= 1) { return 0; }
   /* blocked kernel when the rows of two column blocks fit the registers of a workgroup */
   /* real factors: Gram-space rounds; blocks of 8 columns where the rows of 16 columns fit the registers of 512 threads
-   * (half as many rounds, each 1.4 times as long at N = 2048), blocks of 4 otherwise */
+   * (half as many rounds, each 1.4 times as long at N = 2048; up to 4096 rows in two halves), blocks of 4 otherwise */
   if (!Complex && r >= 32 && g_jacobiVariant == 0) {
     if (N <= 2 * 512) { return gram_sweep<2, 8, 512>(stream, N, r, B, tol, rotations, carry); }
     if (N <= 4 * 512) { return gram_sweep<4, 8, 512>(stream, N, r, B, tol, rotations, carry); }
+    if (N <= 8 * 512) { return gram_sweep<4, 8, 512, 2>(stream, N, r, B, tol, rotations, carry); }
   }
   if (!Complex && r >= 16 && g_jacobiVariant != 1) {
     if (N <= 4 * T_THREADS) { return gram_sweep<4, 4>(stream, N, r, B, tol, rotations, carry); }
