@@ -595,7 +595,7 @@ struct RotRecC { double cs, sn, ar, ai, br, bi; };   /* sn == 0: no rotation */
 struct Cx { double re, im; };
 __device__ __forceinline__ Cx cmul(double ar, double ai, Cx b) { return Cx{ ar * b.re - ai * b.im, ar * b.im + ai * b.re }; }
 
-template <int ROWS, int BC, bool FULL, int THREADS>
+template <int ROWS, int BC, bool FULL, int THREADS, int PASSES>
 __global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t N, int32_t nb, int32_t r, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations) {
   constexpr int NC = 2 * BC, NG = NC * (NC + 1) / 2, NT = NC * NC, WAVES = THREADS / 64, STEPS = FULL ? NC - 1 : BC, GS = NC + 1;
   constexpr int CH = NT >= 32 ? 32 : NT;
@@ -613,19 +613,26 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t
   #pragma unroll
   for (int c = 0; c < NC; ++c) { col[c] = (c < BC ? P : Q) * BC + (c % BC); live[c] = col[c] < r; }
   if (!live[0]) { return; }
+  static_assert(PASSES == 1 || PASSES == 2, "all rows at once or in two halves (as in the real kernel)");
   double x[NC][ROWS][2];
-  #pragma unroll
-  for (int c = 0; c < NC; ++c) {
+  auto load_rows = [&](int pass) {
     #pragma unroll
-    for (int m = 0; m < ROWS; ++m) {
-      const int k = threadIdx.x + m * THREADS;
+    for (int c = 0; c < NC; ++c) {
       #pragma unroll
-      for (int w = 0; w < 2; ++w) { x[c][m][w] = (live[c] && k < N) ? B[((int64_t)col[c] * N + k) * 2 + w] : 0.; }
+      for (int m = 0; m < ROWS; ++m) {
+        const int k = threadIdx.x + (pass * ROWS + m) * THREADS;
+        #pragma unroll
+        for (int w = 0; w < 2; ++w) { x[c][m][w] = (live[c] && k < N) ? B[((int64_t)col[c] * N + k) * 2 + w] : 0.; }
+      }
     }
-  }
+  };
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   /* sum q < NG: real part of pair p = q; q >= NG: imaginary part of pair p = q - NG + NC (the diagonal has none); pairs
    * numbered by diagonal as in the real kernel */
+  #pragma unroll
+  for (int pass = 0; pass < PASSES; ++pass) {
+  if (pass > 0) { asm volatile("" ::: "memory"); }   /* the second half is loaded when the first is done with, not before */
+  load_rows(pass);
   #pragma unroll
   for (int chunk = 0; chunk < NT / CH; ++chunk) {
     double v[CH];
@@ -641,8 +648,9 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t
       v[e] = sum;
     }
     const double tot = wave_sum_swap<CH>(v);
-    if ((lane & (64 / CH - 1)) == 0) { part[wave][chunk * CH + lane / (64 / CH)] = tot; }
+    if ((lane & (64 / CH - 1)) == 0) { double* slot = &part[wave][chunk * CH + lane / (64 / CH)]; *slot = pass == 0 ? tot : *slot + tot; }
   }
+  }   /* passes */
   __syncthreads();
   if (wave == 0) {
     for (int idx = lane; idx < NT; idx += 64) {
@@ -710,6 +718,9 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t
   }
   __syncthreads();
   if (appliedAll == 0) { return; }
+  #pragma unroll
+  for (int pass = PASSES - 1; pass >= 0; --pass) {   /* the half in registers first */
+  if (pass != PASSES - 1) { asm volatile("" ::: "memory"); load_rows(pass); }
   RotRecC cur = rot[0][0];
   #pragma unroll
   for (int n = 0; n < STEPS * BC; ++n) {
@@ -731,10 +742,11 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t
   for (int c = 0; c < NC; ++c) {
     #pragma unroll
     for (int m = 0; m < ROWS; ++m) {
-      const int k = threadIdx.x + m * THREADS;
+      const int k = threadIdx.x + (pass * ROWS + m) * THREADS;
       if (live[c] && k < N) { B[((int64_t)col[c] * N + k) * 2] = x[c][m][0]; B[((int64_t)col[c] * N + k) * 2 + 1] = x[c][m][1]; }
     }
   }
+  }   /* passes */
 }
 
 template <bool CPLX>
@@ -856,11 +868,11 @@ static int gram_sweep(hipStream_t stream, int32_t N, int32_t r, double* B, doubl
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
-template <int ROWS, int BC, int THREADS = T_THREADS>
+template <int ROWS, int BC, int THREADS = T_THREADS, int PASSES = 1>
 static int gram_sweep_cplx(hipStream_t stream, int32_t N, int32_t r, double* B, double tol, int32_t* rotations) {
   const int blocks = (r + BC - 1) / BC, nb = (blocks + 1) & ~1;
-  jacobi_gram_round_cplx_kernel<ROWS, BC, true, THREADS><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations);
-  for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_cplx_kernel<ROWS, BC, false, THREADS><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations); }
+  jacobi_gram_round_cplx_kernel<ROWS, BC, true, THREADS, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations);
+  for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_cplx_kernel<ROWS, BC, false, THREADS, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations); }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
@@ -901,7 +913,7 @@ extern "C" int hykJacobiSweepCarry(hipStream_t stream, int32_t Complex, int32_t 
   if (Complex && r >= 16 && g_jacobiVariant != 1) {
     if (N <= 4 * T_THREADS) { return gram_sweep_cplx<4, 4>(stream, N, r, B, tol, rotations); }
     if (N <= 4 * 512) { return gram_sweep_cplx<4, 4, 512>(stream, N, r, B, tol, rotations); }
-    if (N <= 8 * 512) { return gram_sweep_cplx<8, 2, 512>(stream, N, r, B, tol, rotations); }
+    if (N <= 8 * 512) { return g_jacobiVariant == 0 ? gram_sweep_cplx<4, 4, 512, 2>(stream, N, r, B, tol, rotations) : gram_sweep_cplx<8, 2, 512>(stream, N, r, B, tol, rotations); }
   }
   if (Complex && r >= 16) {
     if (N <= 4 * T_THREADS) { return blocked_sweep<true, 4, 4>(stream, N, r, B, tol, rotations); }

@@ -418,7 +418,7 @@ def test_gemm_fp64(gl, cplx, opA, opB, M, N, K):
 
 
 @pytest.mark.parametrize("variant,carry", [(0, 0), (0, 1), (1, 0), (2, 0), (2, 1)])
-@pytest.mark.parametrize("cplx,N,r", [(0, 300, 40), (0, 1000, 130), (0, 2048, 96), (0, 2500, 70), (0, 4096, 40), (1, 600, 50), (1, 2048, 40), (1, 3000, 24), (0, 64, 64), (0, 700, 20)])
+@pytest.mark.parametrize("cplx,N,r", [(0, 300, 40), (0, 1000, 130), (0, 2048, 96), (0, 2500, 70), (0, 4096, 40), (1, 600, 50), (1, 2048, 40), (1, 3000, 24), (1, 4096, 36), (0, 64, 64), (0, 700, 20)])
 def test_jacobi_sweep_kernels(gl, variant, carry, cplx, N, r):
     """One-sided Jacobi sweeps on a graded N x r factor: every kernel behind hykJacobiSweep / hykJacobiSweepCarry (Gram-space
     rounds with blocks of 8 and of 4 columns, with and without the products inside a block carried from round to round in
