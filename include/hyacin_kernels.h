@@ -90,10 +90,10 @@ int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, do
 size_t hykJacobiCarryBytes(int32_t r);
 int hykJacobiSweepCarry(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations, double* carry);
 /* Which kernel a sweep runs: 0 (default) one Gram matrix per round and workgroup, the steps of the round taken on it by
- * one wavefront; real factors in blocks of 8 columns where N <= 2048 and of 4 above, complex ones in blocks of 4 and 2;
- * 1 one reduction and barrier per step; 2 as 0 with blocks of 4 columns for real factors throughout.  All rotate by the
- * same rule, and for equal block sizes they visit the pairs in the same order; kept selectable so that tests cover every
- * kernel.  Process-wide, not thread-safe. */
+ * one wavefront; real factors in blocks of 8 columns, complex ones in blocks of 4, the rows in two halves where N > 2048;
+ * 1 one reduction and barrier per step; 2 as 0 with the narrower blocks that hold all rows at once (4 columns for real
+ * factors, 2 for complex ones above 2048 rows).  All rotate by the same rule, and for equal block sizes they visit the
+ * pairs in the same order; kept selectable so that tests cover every kernel.  Process-wide, not thread-safe. */
 int hykJacobiSetVariant(int32_t variant);
 int hykColumnNorms(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, const double* B, double* sigma);
 int hykBasisOut(hipStream_t stream, int32_t N, int32_t rank, int32_t Atype, const double* B, const double* sigma, const int32_t* order, void* X, int64_t ldx);
