@@ -595,12 +595,22 @@ struct RotRecC { double cs, sn, ar, ai, br, bi; };   /* sn == 0: no rotation */
 struct Cx { double re, im; };
 __device__ __forceinline__ Cx cmul(double ar, double ai, Cx b) { return Cx{ ar * b.re - ai * b.im, ar * b.im + ai * b.re }; }
 
-template <int ROWS, int BC, bool FULL, int THREADS, int PASSES>
-__global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t N, int32_t nb, int32_t r, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations) {
+template <int ROWS, int BC, bool FULL, int THREADS, int PASSES, bool CARRY>
+__global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t N, int32_t nb, int32_t r, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations, double* __restrict__ carry) {
   constexpr int NC = 2 * BC, NG = NC * (NC + 1) / 2, NT = NC * NC, WAVES = THREADS / 64, STEPS = FULL ? NC - 1 : BC, GS = NC + 1;
-  constexpr int CH = NT >= 32 ? 32 : NT;
-  static_assert(NT % CH == 0 && CH >= 4 && BC * BC <= 64, "whole chunks; one lane of the first wavefront per pair of pairs");
-  __shared__ double part[WAVES][NT];
+  /* CARRY as in the real kernel: the products inside a block (real and imaginary part, 2 NW doubles per block) come from
+   * the round before; summed are the NC norms and the BC^2 cross products (real parts, then imaginary parts) */
+  constexpr bool SLIM = CARRY && !FULL;
+  constexpr int NW = BC * (BC - 1) / 2, NP = SLIM ? NC + 2 * BC * BC : NT;
+  constexpr int CH = SLIM ? 2 * BC : (NP >= 32 ? 32 : NP), TAIL = NP % CH;   /* 40 sums: five times 8; 12: three times 4 */
+  static_assert(TAIL == 0 && CH >= 4 && BC * BC <= 64 && 4 * NW <= 64, "whole chunks and a power-of-two tail; one lane of the first wavefront per pair of pairs and per carried value");
+  /* which sum number q is: real or imaginary part of the product of columns (c0, c1) */
+  auto sum_of = [](int q, bool& isIm, int& c0, int& c1) {
+    if (!SLIM) { isIm = q >= NG; const int p = isIm ? q - NG + NC : q; c0 = p % NC; c1 = (c0 + p / NC) % NC; }
+    else if (q < NC) { isIm = false; c0 = q; c1 = q; }
+    else { const int e = q - NC; isIm = e >= BC * BC; const int f = e % (BC * BC); c0 = f / BC; c1 = BC + f % BC; }
+  };
+  __shared__ double part[WAVES][NP];
   __shared__ double Gre[NC * GS], Gim[NC * GS];
   __shared__ RotRecC rot[STEPS][BC];
   __shared__ double fixed[BC][2];
@@ -627,6 +637,8 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t
     }
   };
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  [[maybe_unused]] double carried = 0.;
+  if constexpr (SLIM) { if (wave == 0 && lane < 4 * NW) { carried = carry[(int64_t)(lane < 2 * NW ? P : Q) * 2 * NW + lane % (2 * NW)]; } }
   /* sum q < NG: real part of pair p = q; q >= NG: imaginary part of pair p = q - NG + NC (the diagonal has none); pairs
    * numbered by diagonal as in the real kernel */
   #pragma unroll
@@ -634,11 +646,12 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t
   if (pass > 0) { asm volatile("" ::: "memory"); }   /* the second half is loaded when the first is done with, not before */
   load_rows(pass);
   #pragma unroll
-  for (int chunk = 0; chunk < NT / CH; ++chunk) {
+  for (int chunk = 0; chunk < NP / CH + (TAIL > 0 ? 1 : 0); ++chunk) {
+    constexpr int dummy = 0; (void)dummy;
     double v[CH];
     #pragma unroll
     for (int e = 0; e < CH; ++e) {
-      const int q = chunk * CH + e; const bool isIm = q >= NG; const int p = isIm ? q - NG + NC : q, c0 = p % NC, c1 = (c0 + p / NC) % NC;
+      bool isIm = false; int c0 = 0, c1 = 0; if (chunk * CH + e < NP) { sum_of(chunk * CH + e, isIm, c0, c1); }
       double sum = 0.;
       #pragma unroll
       for (int m = 0; m < ROWS; ++m) {
@@ -648,18 +661,25 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t
       v[e] = sum;
     }
     const double tot = wave_sum_swap<CH>(v);
-    if ((lane & (64 / CH - 1)) == 0) { double* slot = &part[wave][chunk * CH + lane / (64 / CH)]; *slot = pass == 0 ? tot : *slot + tot; }
+    if ((lane & (64 / CH - 1)) == 0 && chunk * CH + lane / (64 / CH) < NP) { double* slot = &part[wave][chunk * CH + lane / (64 / CH)]; *slot = pass == 0 ? tot : *slot + tot; }
   }
   }   /* passes */
   __syncthreads();
   if (wave == 0) {
-    for (int idx = lane; idx < NT; idx += 64) {
+    for (int idx = lane; idx < NP; idx += 64) {
       double tot = 0.;
       #pragma unroll
       for (int w = 0; w < WAVES; ++w) { tot += part[w][idx]; }
-      const bool isIm = idx >= NG; const int p = isIm ? idx - NG + NC : idx, c0 = p % NC, c1 = (c0 + p / NC) % NC;
+      bool isIm = false; int c0 = 0, c1 = 0; sum_of(idx, isIm, c0, c1);
       if (isIm) { Gim[c0 * GS + c1] = tot; Gim[c1 * GS + c0] = -tot; }
       else { Gre[c0 * GS + c1] = tot; Gre[c1 * GS + c0] = tot; if (c0 == c1) { Gim[c0 * GS + c0] = 0.; } }
+    }
+    if constexpr (SLIM) {
+      if (lane < 4 * NW) {
+        int ci, cj; carried_pair<BC>((lane % (2 * NW)) % NW, ci, cj); const int base = lane < 2 * NW ? 0 : BC; const bool im = lane % (2 * NW) >= NW;
+        if (im) { Gim[(base + ci) * GS + base + cj] = carried; Gim[(base + cj) * GS + base + ci] = -carried; }
+        else { Gre[(base + ci) * GS + base + cj] = carried; Gre[(base + cj) * GS + base + ci] = carried; }
+      }
     }
     wave_lds_sync();
     int applied = 0; double worst = 0.;
@@ -715,6 +735,12 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t
     #pragma unroll
     for (int off = BC / 2; off > 0; off >>= 1) { worst = fmax(worst, __shfl_xor(worst, off, 64)); applied += __shfl_xor(applied, off, 64); }
     if (lane == 0) { report_cosine(rotations, worst); appliedAll = applied; if (applied > 0) { atomicAdd(rotations, applied); } }
+    if constexpr (CARRY) {
+      if (lane < 4 * NW) {
+        int ci, cj; carried_pair<BC>((lane % (2 * NW)) % NW, ci, cj); const int base = lane < 2 * NW ? 0 : BC; const bool im = lane % (2 * NW) >= NW;
+        carry[(int64_t)(lane < 2 * NW ? P : Q) * 2 * NW + lane % (2 * NW)] = im ? Gim[(base + ci) * GS + base + cj] : Gre[(base + ci) * GS + base + cj];
+      }
+    }
   }
   __syncthreads();
   if (appliedAll == 0) { return; }
@@ -869,10 +895,15 @@ static int gram_sweep(hipStream_t stream, int32_t N, int32_t r, double* B, doubl
 }
 
 template <int ROWS, int BC, int THREADS = T_THREADS, int PASSES = 1>
-static int gram_sweep_cplx(hipStream_t stream, int32_t N, int32_t r, double* B, double tol, int32_t* rotations) {
+static int gram_sweep_cplx(hipStream_t stream, int32_t N, int32_t r, double* B, double tol, int32_t* rotations, double* carry) {
   const int blocks = (r + BC - 1) / BC, nb = (blocks + 1) & ~1;
-  jacobi_gram_round_cplx_kernel<ROWS, BC, true, THREADS, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations);
-  for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_cplx_kernel<ROWS, BC, false, THREADS, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations); }
+  if (carry) {
+    jacobi_gram_round_cplx_kernel<ROWS, BC, true, THREADS, PASSES, true><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations, carry);
+    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_cplx_kernel<ROWS, BC, false, THREADS, PASSES, true><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations, carry); }
+  } else {
+    jacobi_gram_round_cplx_kernel<ROWS, BC, true, THREADS, PASSES, false><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations, nullptr);
+    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_cplx_kernel<ROWS, BC, false, THREADS, PASSES, false><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations, nullptr); }
+  }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
@@ -911,9 +942,9 @@ extern "C" int hykJacobiSweepCarry(hipStream_t stream, int32_t Complex, int32_t 
     if (N <= 8 * 512) { return blocked_sweep<false, 8, 4, 512>(stream, N, r, B, tol, rotations); }
   }
   if (Complex && r >= 16 && g_jacobiVariant != 1) {
-    if (N <= 4 * T_THREADS) { return gram_sweep_cplx<4, 4>(stream, N, r, B, tol, rotations); }
-    if (N <= 4 * 512) { return gram_sweep_cplx<4, 4, 512>(stream, N, r, B, tol, rotations); }
-    if (N <= 8 * 512) { return g_jacobiVariant == 0 ? gram_sweep_cplx<4, 4, 512, 2>(stream, N, r, B, tol, rotations) : gram_sweep_cplx<8, 2, 512>(stream, N, r, B, tol, rotations); }
+    if (N <= 4 * T_THREADS) { return gram_sweep_cplx<4, 4>(stream, N, r, B, tol, rotations, carry); }
+    if (N <= 4 * 512) { return gram_sweep_cplx<4, 4, 512>(stream, N, r, B, tol, rotations, carry); }
+    if (N <= 8 * 512) { return g_jacobiVariant == 0 ? gram_sweep_cplx<4, 4, 512, 2>(stream, N, r, B, tol, rotations, carry) : gram_sweep_cplx<8, 2, 512>(stream, N, r, B, tol, rotations, carry); }
   }
   if (Complex && r >= 16) {
     if (N <= 4 * T_THREADS) { return blocked_sweep<true, 4, 4>(stream, N, r, B, tol, rotations); }

@@ -85,8 +85,7 @@ int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t Gtype, con
  * the double at rotations + 2 = the largest squared cosine the sweep met (rotated or not). */
 int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations);
 /* The same sweep with hykJacobiCarryBytes(r) bytes of device memory that its rounds use to hand the products inside a
- * column block from one round to the next instead of summing them again (real factors; ignored for complex ones and by
- * the kernels of variant 1).  The memory needs no initialisation and holds nothing a later sweep relies on. */
+ * column block from one round to the next instead of summing them again (ignored by the kernels of variant 1).  The memory needs no initialisation and holds nothing a later sweep relies on. */
 size_t hykJacobiCarryBytes(int32_t r);
 int hykJacobiSweepCarry(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations, double* carry);
 /* Which kernel a sweep runs: 0 (default) one Gram matrix per round and workgroup, the steps of the round taken on it by
