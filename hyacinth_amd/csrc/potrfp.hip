@@ -28,6 +28,8 @@
  * Cooperative launch: at most one workgroup per compute unit, all resident.
  */
 #include <hip/hip_runtime.h>
+#include <atomic>
+#include <cstdio>
 #include "hyk_common.h"
 #include "hyk_dd.h"
 #include "hyacin_kernels.h"
@@ -293,6 +295,7 @@ extern "C" size_t hykPotrfpWorkspaceBytes(int32_t N, int32_t Gtype) {
 
 extern "C" int hykPotrfp(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, int32_t N, int32_t Gtype, const void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, void* workspace, int32_t* rankOut) {
   if (N <= 0) { return 0; }
+  if (!workspace) { return -1; }
   if (K <= 0 || K > N) { K = N; }
   if (ldg < N || ldr < (K < N ? K + 1 : N) || computeUnits < 1) { return -1; }
   const bool dd = (Gtype & ~1) == HYK_DD, cplx = Gtype & 1;
@@ -303,4 +306,40 @@ extern "C" int hykPotrfp(hipStream_t stream, int32_t computeUnits, double eps, i
   clear_records_kernel<<<1, 2 * MAX_WORKGROUPS, 0, stream>>>(a.records);
   if (dd) { return cplx ? launch<true, true>(stream, a, computeUnits) : launch<true, false>(stream, a, computeUnits); }
   return cplx ? launch<false, true>(stream, a, computeUnits) : launch<false, false>(stream, a, computeUnits);
+}
+
+/* ---- the same factorisation for callers that cannot allocate device memory ----
+ * The diagonal, the position table and the exchange records live in a file-scope device array instead of a workspace
+ * argument.  Every device holds its own copy of the array at its own address; the address is looked up once per device
+ * (with that device current) and only that pointer is ever handed to kernels. */
+constexpr int32_t STATIC_MAX_N = 8192;
+constexpr size_t STATIC_BYTES = (size_t)STATIC_MAX_N * 16 + (size_t)STATIC_MAX_N * 4 + 2 * MAX_WORKGROUPS * sizeof(Record) + 256;
+static __device__ __align__(256) unsigned char scratch[STATIC_BYTES];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::atomic<void*> g_scratchPtr[MAX_DEVICES];
+
+/* device address of `scratch` on the current device; nullptr (and a message) when the runtime refuses */
+void* static_scratch() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) { return nullptr; }
+  void* p = g_scratchPtr[dev].load(std::memory_order_acquire);
+  if (p) { return p; }
+  const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+  if (e != hipSuccess || !p) { std::fprintf(stderr, "hyacin: hipGetSymbolAddress(scratch) failed on device %d: %s\n", dev, hipGetErrorString(e)); return nullptr; }
+  g_scratchPtr[dev].store(p, std::memory_order_release);   /* two threads racing here store the same address */
+  return p;
+}
+}  // namespace
+
+extern "C" int32_t hykPotrfpStaticMaxN(void) { return STATIC_MAX_N; }
+
+extern "C" int hykPotrfpStatic(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, int32_t N, int32_t Gtype, const void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, int32_t* rankOut) {
+  if (N <= 0) { return 0; }
+  if (N > STATIC_MAX_N) { std::fprintf(stderr, "hyacin: hykPotrfpStatic: N = %d exceeds the built-in scratch (N <= %d); use hykPotrfp with a workspace\n", N, STATIC_MAX_N); return -2; }
+  if (hykPotrfpWorkspaceBytes(N, Gtype) > STATIC_BYTES) { return -2; }
+  void* ws = static_scratch();
+  if (!ws) { return -3; }
+  return hykPotrfp(stream, computeUnits, eps, K, N, Gtype, G, ldg, Rt, ldr, jpiv, ws, rankOut);
 }

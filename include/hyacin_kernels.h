@@ -78,6 +78,14 @@ int hykDequantize(hipStream_t stream, int32_t N, int32_t orderC, const uint64_t*
 size_t hykPotrfpWorkspaceBytes(int32_t N, int32_t Gtype);
 int hykPotrfp(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, int32_t N, int32_t Gtype, const void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, void* workspace, int32_t* rankOut);
 
+/* hykPotrfp for callers that cannot allocate device memory (code under HIP graph capture, serving loops, harnesses that
+ * forbid hipMalloc).  No counterpart in the reference.  The workspace of hykPotrfp (diagonal, position table, exchange
+ * records; 192 KB) is a device array built into the library, one copy per device, so the call allocates nothing; inputs
+ * and outputs are the caller's as in hykPotrfp.  N <= hykPotrfpStaticMaxN() (8192), larger N returns -2 with a message on
+ * stderr.  All calls on one device share the array: calls that overlap on one device (two streams, two threads) race. */
+int32_t hykPotrfpStaticMaxN(void);
+int hykPotrfpStatic(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, int32_t N, int32_t Gtype, const void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, int32_t* rankOut);
+
 /* SVD tail.  Replaces the cuSOLVER gesvdj call and the copies around it, src/gram_evd.cu:110-137. */
 int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t Gtype, const void* Rt, int32_t ldr, double* B);
 /* One sweep of one-sided Jacobi over the r columns of B (N x r, FP64, complex interleaved): every pair whose cosine exceeds
