@@ -105,6 +105,12 @@ def lib():
         L.hykMatmulCf16.argtypes = [vp, ch, i32, i32, i32, vp, i64, vp, i64, vp, i64]
         L.hykSumSquares.argtypes = [vp, i64, i64, vp, i64, vp]
         L.hykOrthonormalize.argtypes = [vp, i32, i32, i32, vp, i64, vp]
+        L.hykFactorToB.argtypes = [vp, i32, i32, i32, vp, i32, vp]
+        L.hykColumnNorms.argtypes = [vp, i32, i32, i32, vp, vp]
+        L.hykBasisOut.argtypes = [vp, i32, i32, i32, vp, vp, vp, vp, i64]
+        L.hykValuesOut.argtypes = [vp, i32, i32, vp, vp]
+        L.hykInterpSolve.argtypes = [vp, i32, i32, i32, vp, i32, vp, vp, vp]
+        L.hykInterpOut.argtypes = [vp, i32, i32, i32, vp, vp, vp, i64]
         _lib = L
     return _lib
 

@@ -99,8 +99,6 @@ GRAM_SHAPES = [(7, 128, 128), (130, 384, 300), (300, 1152, 1100), (513, 256, 256
 @pytest.mark.parametrize("N,K,rows", GRAM_SHAPES)
 @pytest.mark.parametrize("cplx,order", [(0, 1), (0, 14), (1, 2), (1, 15), (1, 22)])
 def test_gram_crt_bit_exact(gl, oracle, N, K, rows, cplx, order):
-    if N > 300 and order > 15:
-        pytest.skip("covered at the smaller sizes")
     rng = np.random.default_rng(34)
     panels = random_panels(rng, oracle.n_panels("crt", order, cplx), N, K, rows, -125, 126)
     orderC = 3
@@ -114,10 +112,10 @@ def test_gram_crt_bit_exact(gl, oracle, N, K, rows, cplx, order):
 
 
 @pytest.mark.parametrize("N,K,rows", GRAM_SHAPES)
-@pytest.mark.parametrize("cplx,order", [(0, 1), (0, 6), (1, 3), (0, 11), (1, 6)])
+@pytest.mark.parametrize("cplx,order", [(0, 1), (0, 6), (1, 3), (0, 11), (1, 6), (1, 9), (1, 11)])
 def test_gram_limbs_bit_exact(gl, oracle, N, K, rows, cplx, order):
-    if N > 300 and order > 6:
-        pytest.skip("covered at the smaller sizes")
+    """Complex orders 9 and 11 make 3 o^2 > 192 panel pairs in 3 (2 o - 1) > 48 groups: the plan no longer fits one launch's
+    tables and is cut between groups, also between the three groups of one level."""
     rng = np.random.default_rng(35)
     panels = random_panels(rng, oracle.n_panels("limbs", order, cplx), N, K, rows)
     orderC = 3 if order > 6 else 2

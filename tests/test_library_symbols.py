@@ -32,3 +32,12 @@ def test_handle_layout_and_host_planner():
         assert ha.herk_batch_init(h, eps, M, 300, at) == ho.herk_batch_init(eps, M, 300, at, 7)
     # precision enum values are ABI
     assert (ha.F64, ha.F64C, ha.F32, ha.F32C, ha.F16, ha.F16C, ha.DD, ha.DDC, ha.TF, ha.TFC, ha.QF, ha.QFC) == tuple(range(12))
+
+
+def test_every_kernel_entry_has_argument_types():
+    """A ctypes call without argtypes passes Python ints as 32-bit C ints: a 64-bit leading dimension would arrive with
+    undefined upper bits.  Every kernel-layer function therefore declares its arguments."""
+    import hyacinth_amd as ha
+    L = ha.lib()
+    for name in ha.KERNEL_SYMBOLS:
+        assert getattr(L, name).argtypes is not None, name
