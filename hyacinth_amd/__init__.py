@@ -31,7 +31,7 @@ API_SYMBOLS = [
 KERNEL_SYMBOLS = [
     "hykColumnExponents", "hykSliceRange", "hykQuantizeLimbs", "hykQuantizeCrt", "hykZeroRows",
     "hykGramWorkspaceBytes", "hykGramWorkspaceClear", "hykGramCrt", "hykGramLimbs", "hykGramSetSlab",
-    "hykGramProfile", "hykGramProfileRead", "hykMfmaCeiling", "hykGramRange", "hykDequantize", "hykPotrfpWorkspaceBytes", "hykPotrfp", "hykPotrfpStaticMaxN", "hykPotrfpStatic", "hykFactorToB", "hykJacobiSweep", "hykJacobiSweepCarry", "hykJacobiCarryBytes", "hykJacobiSetVariant",
+    "hykGramProfile", "hykGramProfileRead", "hykMfmaCeiling", "hykGramRange", "hykDequantize", "hykPotrfpWorkspaceBytes", "hykPotrfp", "hykPotrfpLeftLooking", "hykPotrfpStaticMaxN", "hykPotrfpStatic", "hykFactorToB", "hykJacobiSweep", "hykJacobiSweepCarry", "hykJacobiCarryBytes", "hykJacobiSetVariant",
     "hykColumnNorms", "hykBasisOut", "hykValuesOut", "hykInterpSolve", "hykInterpOut", "hykMatcopy",
     "hykSumSquares", "hykMatmulCf16", "hykGemm", "hykOrthonormalize",
 ]
@@ -98,6 +98,7 @@ def lib():
         L.hykDequantize.argtypes = [vp, i32, i32, vp, vp, i32, vp, i64]
         L.hykPotrfpWorkspaceBytes.argtypes = [i32, i32]; L.hykPotrfpWorkspaceBytes.restype = C.c_size_t
         L.hykPotrfp.argtypes = [vp, i32, dbl, i32, i32, i32, vp, i64, vp, i32, vp, vp, vp]
+        L.hykPotrfpLeftLooking.argtypes = [vp, i32, dbl, i32, i32, i32, vp, i64, vp, i32, vp, vp, vp]
         L.hykPotrfpStaticMaxN.argtypes = []; L.hykPotrfpStaticMaxN.restype = i32
         L.hykPotrfpStatic.argtypes = [vp, i32, dbl, i32, i32, i32, vp, i64, vp, i32, vp, vp]
         L.hykMatcopy.argtypes = [vp, ch, i64, i64, i32, vp, i64, i32, vp, i64]

@@ -11,7 +11,8 @@
  *    contraction measured over the last two sweeps puts within 8 thresholds; a sweep here is one plain round-robin pass over all
  *    column pairs, which does less work than a sweep of the vendor's blocked solver, so the cap is 5 x |JacobiSVDSweeps|
  *    plain sweeps (15 by default); JacobiSVDSweeps == 0 (the reference's "bidiagonalization backend") caps at 30.
- * G is left untouched (the reference overwrites it with the factor).
+ * G is working storage, as in the reference (which overwrites it with the factor): the Cholesky keeps the trailing matrix
+ * in its strict upper triangle.  An FP32 Gram is factored from a widened copy and stays as it was.
  */
 #include <numeric>
 #include <cfloat>
@@ -24,8 +25,8 @@ double storage_eps(int Atype) { return (Atype == HYACIN_F64 || Atype == HYACIN_F
 int factor_type(int Gtype) { const int c = Gtype & 1; return ((Gtype & ~1) == HYACIN_DD ? HYACIN_DD : HYACIN_F64) + c; }
 
 struct Factor {
-  hyh::Scratch widened, Rt, work; const void* G; int64_t ldg; int type; int32_t ldr; size_t rtBytes;
-  Factor(const hyacinHandle_t* h, int32_t N, int32_t Kmax, int Gtype, const void* Gin, int64_t ldgIn)
+  hyh::Scratch widened, Rt, work; void* G; int64_t ldg; int type; int32_t ldr; size_t rtBytes;
+  Factor(const hyacinHandle_t* h, int32_t N, int32_t Kmax, int Gtype, void* Gin, int64_t ldgIn)
     : widened(h, ((Gtype & ~1) == HYACIN_F32) ? (size_t)N * N * 8 * (1 + (Gtype & 1)) : 0),
       Rt(h, (size_t)N * (size_t)std::min(N, Kmax + 1) * (size_t)hyh::elem_bytes(factor_type(Gtype))),
       work(h, hykPotrfpWorkspaceBytes(N, factor_type(Gtype))) {

@@ -72,19 +72,25 @@ int hykGramRange(hipStream_t stream, int32_t N, int32_t orderC, const uint64_t* 
 int hykDequantize(hipStream_t stream, int32_t N, int32_t orderC, const uint64_t* C, const int32_t* vexp, int32_t Gtype, void* G, int64_t ldg);
 
 /* Pivoted Cholesky.  Replaces internal::Cholesky::potrfp, src/hyacin_potrfp.cu:119-343.
- * G: N x N (FP64 / FP64 complex / double-double / double-double complex), read only.
+ * G: N x N (FP64 / FP64 complex / double-double / double-double complex), Hermitian with both triangles filled; it is
+ * working storage: the strict upper triangle is overwritten (the reference overwrites G with the factor).
  * Rt: zero-initialised, column-wise factor Rt[c * ldr + k] = R[k, c] in the type of G, ldr >= min(N, K + 1).
- * jpiv: N 1-based pivots in the reference's swap order.  rankOut: device-visible int32 (pinned host memory). */
+ * jpiv: N 1-based pivots in the reference's swap order.  rankOut: device-visible int32 (pinned host memory); -1 when the
+ * workgroups of the run lost each other (a bounded wait inside the kernel gave up).
+ * hykPotrfp runs the blocked right-looking kernel (panels of 16 columns, one rank-16 update of the trailing matrix per
+ * panel) for N <= 8192 when computeUnits >= ceil(N / 64), else the left-looking kernel, which hykPotrfpLeftLooking
+ * always runs (it leaves G untouched).  Same pivots, same rank; factor entries equal to rounding. */
 size_t hykPotrfpWorkspaceBytes(int32_t N, int32_t Gtype);
-int hykPotrfp(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, int32_t N, int32_t Gtype, const void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, void* workspace, int32_t* rankOut);
+int hykPotrfp(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, int32_t N, int32_t Gtype, void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, void* workspace, int32_t* rankOut);
+int hykPotrfpLeftLooking(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, int32_t N, int32_t Gtype, void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, void* workspace, int32_t* rankOut);
 
 /* hykPotrfp for callers that cannot allocate device memory (code under HIP graph capture, serving loops, harnesses that
  * forbid hipMalloc).  No counterpart in the reference.  The workspace of hykPotrfp (diagonal, position table, exchange
- * records; 192 KB) is a device array built into the library, one copy per device, so the call allocates nothing; inputs
+ * records; 194 KB) is a device array built into the library, one copy per device, so the call allocates nothing; inputs
  * and outputs are the caller's as in hykPotrfp.  N <= hykPotrfpStaticMaxN() (8192), larger N returns -2 with a message on
  * stderr.  All calls on one device share the array: calls that overlap on one device (two streams, two threads) race. */
 int32_t hykPotrfpStaticMaxN(void);
-int hykPotrfpStatic(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, int32_t N, int32_t Gtype, const void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, int32_t* rankOut);
+int hykPotrfpStatic(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, int32_t N, int32_t Gtype, void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, int32_t* rankOut);
 
 /* SVD tail.  Replaces the cuSOLVER gesvdj call and the copies around it, src/gram_evd.cu:110-137. */
 int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t Gtype, const void* Rt, int32_t ldr, double* B);

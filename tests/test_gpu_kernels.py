@@ -256,14 +256,16 @@ def spd_exact_dd(rng, N, r, cplx):
 
 # (N, leading values, K, eps for FP64, eps for double-double, floor, compute units offered)
 POTRFP_CASES = [(24, 9, 24, 1e-6, 1e-6, 1e-9, 256), (150, 40, 150, 1e-6, 1e-10, 1e-13, 256), (150, 15, 150, 0.0, 0.0, 1e-5, 3),
-                (150, 60, 17, 1e-12, 1e-12, 1e-15, 256), (700, 64, 700, 1e-6, 1e-9, 1e-12, 256)]
+                (150, 60, 17, 1e-12, 1e-12, 1e-15, 256), (700, 64, 700, 1e-6, 1e-9, 1e-12, 256), (700, 64, 16, 1e-12, 1e-12, 1e-12, 11),
+                (130, 50, 18, 1e-12, 1e-12, 1e-12, 2)]
 
 
+@pytest.mark.parametrize("entry", ["hykPotrfp", "hykPotrfpLeftLooking"])
 @pytest.mark.parametrize("gbase", [0, 6])        # FP64, double-double
 @pytest.mark.parametrize("cplx", [0, 1])
 @pytest.mark.parametrize("N,r,K,eps64,epsdd,floor,units", POTRFP_CASES)
-def test_potrfp_kernel(gl, oracle, gbase, cplx, N, r, K, eps64, epsdd, floor, units):
-    """hykPotrfp against the oracle's pivoted Cholesky (src/hyacin_potrfp.cu:119-318): same rank, same pivots, factor rows equal
+def test_potrfp_kernel(gl, oracle, entry, gbase, cplx, N, r, K, eps64, epsdd, floor, units):
+    """Both kernels (blocked right-looking, left-looking) against the oracle's pivoted Cholesky (src/hyacin_potrfp.cu:119-318): same rank, same pivots, factor rows equal
     to rounding (the two sum in different orders, and row t carries the rounding of the Schur complement it came from, so
     the bound grows with d_0 / d_t).  The cut-off sits well above the rounding level of the arithmetic and well above the
     floor of the spectrum, so the rank is not decided by rounding.  `units` limits the workgroups, so that wavefronts
@@ -285,7 +287,8 @@ def test_potrfp_kernel(gl, oracle, gbase, cplx, N, r, K, eps64, epsdd, floor, un
     rk = zeros(4)
     ws = zeros(gl.L.hykPotrfpWorkspaceBytes(N, gtype))
     dG = dev(raw)
-    assert gl.L.hykPotrfp(stream(), units, eps, K, N, gtype, ptr(dG), N, ptr(Rt), ldr, ptr(jp), ptr(ws), ptr(rk)) == 0
+    print(entry, "N", N, "K", K, "gtype", gtype, "units", units, flush=True)
+    assert getattr(gl.L, entry)(stream(), units, eps, K, N, gtype, ptr(dG), N, ptr(Rt), ldr, ptr(jp), ptr(ws), ptr(rk)) == 0
     sync()
     rank = int(host(rk, np.int32)[0])
     piv = host(jp, np.int32)
