@@ -285,129 +285,255 @@ template <bool DD, bool CPLX> int launch(hipStream_t stream, PotrfArgs& args, in
 /* ====================================================================================================================
  * Blocked, right-looking form (N <= 8192): the factorization advances in panels of PB columns.
  *
- *  - Panel.  One wavefront per 64 columns is an *agent* (wavefront 0 of workgroup a < agents); a lane owns one column
- *    for the whole run: its remaining diagonal entry lives in a register, its entries of the current panel's rows in
- *    LDS.  The trailing matrix G' is kept up to date by the update phase, so a step needs, per lane, G'[l, c] and the
- *    dot product of at most PB - 1 factor entries.  Per step an agent publishes ONE 128-byte record (arg-max and trace
- *    of its columns and the candidate's newest factor entry, every 32-bit piece in a 64-bit word tagged with the step
- *    number) and every agent polls all records, one lane per record, and reduces them inside the wavefront: no
- *    workgroup barrier and no LDS on the chain from one pivot to the next.  The factor entries of a step are stored
- *    after its record (the one entry another agent can need before they are visible travels in the record).
+ *  - Panel.  One wavefront per 64 columns is an *agent* (wavefront 0 of workgroup a < agents; column l belongs to agent
+ *    l % agents); a lane owns one column for the whole run: its remaining diagonal entry lives in a register, its entries of the current panel's rows in
+ *    LDS.  The trailing matrix G' is kept up to date by the update phase, so a step needs, per lane, G'[l, c] and a
+ *    dot product of at most PB - 1 factor entries.  Per step an agent publishes ONE record (arg-max and trace of its
+ *    columns and the candidate's newest factor entry; every 32-bit piece in a 64-bit word tagged with the step number,
+ *    word j of all agents side by side so that a poll of all records touches two or three cache lines per word) and
+ *    every agent polls all records, one lane per record, and reduces them inside the wavefront with data-parallel
+ *    lane exchanges: no workgroup barrier and no LDS on the chain from one pivot to the next.  The factor entries of a
+ *    step are stored after its record (the one entry another agent can need before they are visible travels in the
+ *    record).  While a step runs, the agents fetch what the next step needs if the runner-up of the last arg-max
+ *    becomes the pivot (its column of G' and its factor entries); when it does, the step starts without waiting for
+ *    memory.
  *  - Update.  After a panel every workgroup drops the new pivots from its sorted list of remaining columns and all
  *    workgroups apply the rank-PB update G'[l, m] -= sum_t conj(R[t, l]) R[t, m] to the pairs l < m of remaining
  *    columns, in 64 x 64 tiles (operands in LDS, a 4 x 4 block per lane).  Only the strict upper triangle of G' is kept;
  *    the panel reads G'[l, c] as conj(G'[c, l]) where l > c.  G is overwritten (as in the reference).
- *  - What crosses workgroups (records, factor entries, G', pivots) is stored write-through and loaded past the
- *    non-coherent cache levels; a counter that every workgroup bumps after its update tiles is the one grid-wide
+ *  - What crosses workgroups (records, factor entries, G', the panel summary) is stored write-through and loaded past
+ *    the non-coherent cache levels; a counter that every workgroup bumps after its update tiles is the one grid-wide
  *    rendezvous per panel.  Every wait is bounded and gives up for the whole grid.
  * ==================================================================================================================== */
 namespace blk {
 
 constexpr int THREADS = 256;        /* four wavefronts: the first leads (agent or waiter), all four update */
-constexpr int PB = 16;              /* columns per panel */
+constexpr int MAX_PB = 32;          /* columns per panel: 32 for real matrices, 16 for complex ones */
 constexpr int MAX_AGENTS = 128;     /* 64 columns each */
 constexpr int MAX_N = MAX_AGENTS * 64;
-constexpr int REC_WORDS = 16;       /* 128 bytes per record */
+constexpr int REC_WORDS = 16;       /* at most 15 tagged words per record */
 constexpr int TILE = 64;
 constexpr int SPIN = 1 << 21;
-constexpr int CTL_WORDS = 32;       /* control block: [0], [1] tagged panel summary; [8] update counter */
+constexpr int CTL_WORDS = 64;       /* control block: [0 .. 2 + PB/2) tagged panel summary; [32] update counter; [40 .. 50) timing sums */
+constexpr int CTL_COUNTER = 32, CTL_TIMING = 40;
 
 struct Args {
   int32_t N, K, ldr, agents; double eps2;
-  double* G; int64_t ldg; double* Rt; int32_t* jpiv; int32_t* pos; uint64_t* records; uint64_t* ctl; int32_t* rankOut;
+  double* G; int64_t ldg; double* Rt; int32_t* jpiv; uint64_t* records; uint64_t* ctl; int32_t* rankOut;
 };
 
 __device__ __forceinline__ uint64_t ld_shared_u64(const uint64_t* p) { return __hip_atomic_load(const_cast<uint64_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void st_shared_u64(uint64_t* p, uint64_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-__device__ __forceinline__ int32_t ld_shared_i32(const int32_t* p) { return __hip_atomic_load(const_cast<int32_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-__device__ __forceinline__ void st_shared_i32(int32_t* p, int32_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 
-/* what an agent publishes per step, all wavefront-uniform */
-struct Msg { double bx, by, tr, n[4]; int32_t bi; };
-
-/* lane j < 15 stores word j = epoch << 32 | piece j; pieces: the halves of bx, by, tr, n[0..3], then the index */
-__device__ __forceinline__ void publish(uint64_t* rec, const Msg& m, uint32_t epoch) {
-  const int j = threadIdx.x & 63, q = j >> 1;
-  double v = m.bx; v = q == 1 ? m.by : v; v = q == 2 ? m.tr : v; v = q == 3 ? m.n[0] : v; v = q == 4 ? m.n[1] : v; v = q == 5 ? m.n[2] : v; v = q == 6 ? m.n[3] : v;
-  const uint64_t bits = (uint64_t)__double_as_longlong(v);
-  const uint32_t piece = j == 14 ? (uint32_t)m.bi : (uint32_t)(bits >> (32 * (j & 1)));
-  if (j < 15) { st_shared_u64(&rec[j], ((uint64_t)epoch << 32) | piece); }
+/* ---- wavefront-wide arg-max / sum without LDS: six exchange steps, after which every lane holds the result.
+ * Steps 0..3 stay inside a row of 16 lanes (quad permutations, then the two mirror patterns: any pairing that joins
+ * two groups holding equal values does), steps 4 and 5 swap rows / halves between two registers. */
+template <int STEP> __device__ __forceinline__ void pair_u32(uint32_t v, uint32_t& x, uint32_t& y) {
+  if constexpr (STEP == 0) { x = v; y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xf, 0xf, false); }
+  else if constexpr (STEP == 1) { x = v; y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xf, 0xf, false); }
+  else if constexpr (STEP == 2) { x = v; y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xf, 0xf, false); }
+  else if constexpr (STEP == 3) { x = v; y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xf, 0xf, false); }
+  else if constexpr (STEP == 4) { const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false); x = r[0]; y = r[1]; }
+  else { const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false); x = r[0]; y = r[1]; }
+}
+template <int STEP> __device__ __forceinline__ void pair_f64(double v, double& x, double& y) {
+  const uint64_t b = (uint64_t)__double_as_longlong(v); uint32_t xl, yl, xh, yh;
+  pair_u32<STEP>((uint32_t)b, xl, yl); pair_u32<STEP>((uint32_t)(b >> 32), xh, yh);
+  x = __longlong_as_double((long long)(((uint64_t)xh << 32) | xl)); y = __longlong_as_double((long long)(((uint64_t)yh << 32) | yl));
+}
+template <bool DD, int STEP> __device__ __forceinline__ void reduce_step(double& bx, double& by, int32_t& bi, double& tr) {
+  double x0, x1, y0 = 0., y1 = 0., t0, t1; uint32_t i0, i1;
+  pair_f64<STEP>(bx, x0, x1); if constexpr (DD) { pair_f64<STEP>(by, y0, y1); } pair_u32<STEP>((uint32_t)bi, i0, i1); pair_f64<STEP>(tr, t0, t1);
+  bx = x0; by = y0; bi = (int32_t)i0; better(DD, bx, by, bi, x1, y1, (int32_t)i1); tr = t0 + t1;
+}
+template <bool DD> __device__ __forceinline__ void reduce_wave_full(double& bx, double& by, int32_t& bi, double& tr) {
+  reduce_step<DD, 0>(bx, by, bi, tr); reduce_step<DD, 1>(bx, by, bi, tr); reduce_step<DD, 2>(bx, by, bi, tr);
+  reduce_step<DD, 3>(bx, by, bi, tr); reduce_step<DD, 4>(bx, by, bi, tr); reduce_step<DD, 5>(bx, by, bi, tr);
+}
+template <int STEP> __device__ __forceinline__ void max_sum_step(double& bx, double& tr) {
+  double x0, x1, t0, t1; pair_f64<STEP>(bx, x0, x1); pair_f64<STEP>(tr, t0, t1); bx = x0 < x1 ? x1 : x0; tr = t0 + t1;
+}
+/* The usual case has one largest high word: then only that maximum and the trace go through the six exchange steps, and
+ * the low word and the index are read from the one lane that holds the maximum.  Candidates have bx > 0, lanes without
+ * one bx = 0 and bi = -1.  Equal high words (or no candidate) take the full reduction; both give the same result. */
+template <bool DD> __device__ __forceinline__ void reduce_wave(double& bx, double& by, int32_t& bi, double& tr) {
+  double mx = bx, t = tr;
+  max_sum_step<0>(mx, t); max_sum_step<1>(mx, t); max_sum_step<2>(mx, t); max_sum_step<3>(mx, t); max_sum_step<4>(mx, t); max_sum_step<5>(mx, t);
+  const uint64_t holders = __ballot(bi >= 0 && bx == mx);
+  if (__popcll(holders) == 1) {
+    const int src = __builtin_amdgcn_readfirstlane((int)__ffsll((long long)holders) - 1);
+    bx = mx; tr = t; bi = __builtin_amdgcn_readlane(bi, src);
+    if constexpr (DD) {
+      const uint64_t b = (uint64_t)__double_as_longlong(by);
+      const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)b, src), hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(b >> 32), src);
+      by = __longlong_as_double((long long)(((uint64_t)hi << 32) | lo));
+    } else { by = 0.; }
+  } else { reduce_wave_full<DD>(bx, by, bi, tr); }
 }
 
-/* waits for record `r` of `epoch` (bounded); false when the wait gave up */
-__device__ __forceinline__ bool read_record(const uint64_t* rec, uint32_t epoch, Msg& m) {
-  uint64_t v[15];
+/* acc -= a b without renormalising acc (its low word collects the error terms; renorm() once at the end) */
+template <bool DD> __device__ __forceinline__ void fnma_acc(const Real<DD>& a, const Real<DD>& b, Real<DD>& acc) {
+  if constexpr (DD) {
+    const double p = a.v.x * b.v.x; double e = fma(a.v.x, b.v.x, -p); e = fma(a.v.x, b.v.y, e); e = fma(a.v.y, b.v.x, e);
+    const double s = acc.v.x - p, bb = s - acc.v.x, err = (acc.v.x - (s - bb)) + (-p - bb);
+    acc.v.x = s; acc.v.y = (acc.v.y + err) - e;
+  } else { acc.v.x = fma(-a.v.x, b.v.x, acc.v.x); }
+}
+template <bool DD> __device__ __forceinline__ Real<DD> renorm(Real<DD> a) {
+  if constexpr (DD) { double s, e; hyk::two_sum(a.v.x, a.v.y, s, e); return Real<DD>{ dd_t{ s, e } }; } else { return a; }
+}
+
+/* what an agent publishes per step (wavefront-uniform): doubles bx, tr, n[0 .. WE), by (double-double only), then the index */
+template <bool DD, bool CPLX> struct Rec {
+  static constexpr int WE = Width<DD, CPLX>::elem, ND = 2 + WE + (DD ? 1 : 0), NW = 2 * ND + 1;
+  double bx, by, tr, n[4]; int32_t bi;
+  __device__ __forceinline__ void clear() { bx = by = tr = 0.; bi = -1; n[0] = n[1] = n[2] = n[3] = 0.; }
+};
+
+/* word j of agent i for the step parity: recs[(parity * REC_WORDS + j) * MAX_AGENTS + i] */
+template <bool DD, bool CPLX>
+__device__ __forceinline__ void publish(uint64_t* recs, int agent, const Rec<DD, CPLX>& m, uint32_t epoch) {
+  using RC = Rec<DD, CPLX>; const int j = threadIdx.x & 63, q = j >> 1;
+  double v = m.bx; v = q == 1 ? m.tr : v;
+  #pragma unroll
+  for (int w = 0; w < RC::WE; ++w) { v = q == 2 + w ? m.n[w] : v; }
+  if constexpr (DD) { v = q == 2 + RC::WE ? m.by : v; }
+  const uint64_t bits = (uint64_t)__double_as_longlong(v);
+  const uint32_t piece = j == RC::NW - 1 ? (uint32_t)m.bi : (uint32_t)(bits >> (32 * (j & 1)));
+  if (j < RC::NW) { st_shared_u64(&recs[((size_t)(epoch & 1) * REC_WORDS + j) * MAX_AGENTS + agent], ((uint64_t)epoch << 32) | piece); }
+}
+
+/* waits for the record of agent i (bounded); false when the wait gave up.  Two polls are kept in flight, so that a record
+ * is seen at most half a memory latency after it has become visible. */
+template <bool DD, bool CPLX>
+__device__ __forceinline__ bool read_record(const uint64_t* recs, int i, uint32_t epoch, Rec<DD, CPLX>& m) {
+  using RC = Rec<DD, CPLX>; uint64_t va[RC::NW], vb[RC::NW], v[RC::NW]; const uint64_t* base = &recs[(size_t)(epoch & 1) * REC_WORDS * MAX_AGENTS + i];
+  auto poll = [&](uint64_t (&w)[RC::NW]) {
+    #pragma unroll
+    for (int j = 0; j < RC::NW; ++j) { w[j] = ld_shared_u64(base + (size_t)j * MAX_AGENTS); }
+  };
+  auto complete = [&](const uint64_t (&w)[RC::NW]) {
+    bool all = true;
+    #pragma unroll
+    for (int j = 0; j < RC::NW; ++j) { all = all && (uint32_t)(w[j] >> 32) == epoch; }
+    return all;
+  };
+  poll(va);
   for (int spins = 0;; ++spins) {
-    bool complete = true;
-    #pragma unroll
-    for (int j = 0; j < 15; ++j) { v[j] = ld_shared_u64(&rec[j]); }
-    #pragma unroll
-    for (int j = 0; j < 15; ++j) { complete = complete && (uint32_t)(v[j] >> 32) == epoch; }
-    if (complete) { break; }
+    poll(vb);
+    if (complete(va)) {
+      #pragma unroll
+      for (int j = 0; j < RC::NW; ++j) { v[j] = va[j]; }
+      break;
+    }
+    poll(va);
+    if (complete(vb)) {
+      #pragma unroll
+      for (int j = 0; j < RC::NW; ++j) { v[j] = vb[j]; }
+      break;
+    }
     if (spins > SPIN) { return false; }
-    __builtin_amdgcn_s_sleep(1);
   }
   auto dbl = [&](int q) { return __longlong_as_double((long long)((v[2 * q] & 0xffffffffull) | (v[2 * q + 1] << 32))); };
-  m.bx = dbl(0); m.by = dbl(1); m.tr = dbl(2); m.n[0] = dbl(3); m.n[1] = dbl(4); m.n[2] = dbl(5); m.n[3] = dbl(6); m.bi = (int32_t)(uint32_t)v[14];
+  m.bx = dbl(0); m.tr = dbl(1); m.by = 0.; m.n[0] = m.n[1] = m.n[2] = m.n[3] = 0.;
+  #pragma unroll
+  for (int w = 0; w < RC::WE; ++w) { m.n[w] = dbl(2 + w); }
+  if constexpr (DD) { m.by = dbl(2 + RC::WE); }
+  m.bi = (int32_t)(uint32_t)v[RC::NW - 1];
   return true;
 }
 
-/* All records of `epoch` -> in every lane: the best column over all agents (its value, its newest factor entry) and the
- * total trace.  Lane i reads records i and i + 64.  Every agent runs the same instructions on the same data, so all
- * agents take the same decisions.  Returns false when a wait gave up. */
-template <bool DD>
-__device__ __forceinline__ bool collect(const uint64_t* recs, int agents, uint32_t epoch, Msg& out) {
-  const int lane = threadIdx.x & 63; bool ok = true;
-  Msg m; m.bx = m.by = m.tr = 0.; m.bi = -1; m.n[0] = m.n[1] = m.n[2] = m.n[3] = 0.;
-  if (lane < agents) { ok = read_record(&recs[(size_t)lane * REC_WORDS], epoch, m); if (!ok) { m.bi = -1; m.tr = 0.; } }
+/* value of a wavefront-uniform lane's register in every lane */
+__device__ __forceinline__ double lane_f64(double v, int src) {
+  const int s = __builtin_amdgcn_readfirstlane(src); const uint64_t b = (uint64_t)__double_as_longlong(v);
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)b, s), hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(b >> 32), s);
+  return __longlong_as_double((long long)(((uint64_t)hi << 32) | lo));
+}
+
+/* All records of `epoch` -> in every lane: the best column over all agents (value, newest factor entry) and the total
+ * trace; m / m2 keep what this lane read (records i and i + 64: the better one, the other one) for runner_up().  Column l
+ * belongs to agent l % agents.  Every agent runs the same instructions on the same data, so all agents take the same
+ * decisions. */
+template <bool DD, bool CPLX>
+__device__ __forceinline__ bool collect(const uint64_t* recs, int agents, uint32_t epoch, Rec<DD, CPLX>& out, Rec<DD, CPLX>& m, Rec<DD, CPLX>& m2) {
+  using RC = Rec<DD, CPLX>; const int lane = threadIdx.x & 63; bool ok = true;
+  m.clear(); m2.clear();
+  if (lane < agents) { ok = read_record<DD, CPLX>(recs, lane, epoch, m); if (!ok) { m.clear(); } }
   if (lane + 64 < agents) {
-    Msg o; const bool ok2 = read_record(&recs[(size_t)(lane + 64) * REC_WORDS], epoch, o); ok = ok && ok2;
+    RC o; const bool ok2 = read_record<DD, CPLX>(recs, lane + 64, epoch, o); ok = ok && ok2;
     if (ok2) {
-      const int before = m.bi; better(DD, m.bx, m.by, m.bi, o.bx, o.by, o.bi); m.tr += o.tr;
-      if (m.bi != before) { m.n[0] = o.n[0]; m.n[1] = o.n[1]; m.n[2] = o.n[2]; m.n[3] = o.n[3]; }
+      const double t = m.tr + o.tr; double bx = m.bx, by = m.by; int32_t bi = m.bi; better(DD, bx, by, bi, o.bx, o.by, o.bi);
+      if (bi != m.bi) { m2 = m; m = o; } else { m2 = o; }
+      m.tr = t;
     }
   }
   out.bx = m.bx; out.by = m.by; out.bi = m.bi; out.tr = m.tr;
-  wave_reduce<DD, 6>(out.bx, out.by, out.bi, out.tr);
-  /* the winner's newest entry sits in the lane that read its record */
-  const int src = out.bi >= 0 ? ((out.bi >> 6) & 63) : 0;
+  reduce_wave<DD>(out.bx, out.by, out.bi, out.tr);
+  const int src = out.bi >= 0 ? ((out.bi % agents) & 63) : 0;   /* the winner's newest entry sits in the lane that read its record */
   #pragma unroll
-  for (int q = 0; q < 4; ++q) { out.n[q] = __shfl(m.n[q], src, 64); }
+  for (int q = 0; q < 4; ++q) { out.n[q] = q < RC::WE ? lane_f64(m.n[q], src) : 0.; }
   return __all(ok);
 }
+/* the best column of the agents other than the winner's, with its newest entry: the same reduction with the winner's record left out */
+template <bool DD, bool CPLX>
+__device__ __forceinline__ void runner_up(int agents, int winner, const Rec<DD, CPLX>& m, const Rec<DD, CPLX>& m2, Rec<DD, CPLX>& second) {
+  using RC = Rec<DD, CPLX>; const RC& r = (winner >= 0 && m.bi == winner) ? m2 : m; double dummy = 0.;
+  second.bx = r.bx; second.by = r.by; second.bi = r.bi; second.tr = 0.;
+  reduce_wave<DD>(second.bx, second.by, second.bi, dummy);
+  const int src = second.bi >= 0 ? ((second.bi % agents) & 63) : 0;
+  #pragma unroll
+  for (int q = 0; q < 4; ++q) { second.n[q] = q < RC::WE ? lane_f64(r.n[q], src) : 0.; }
+}
+
+/* -DHYK_POTRFP_TIMING: the first agent adds up, in wall-clock ticks of 10 ns, where its steps spend their time, and leaves
+ * the sums in the control words CTL_TIMING .. of the workspace (a measuring build; the stamps themselves cost time) */
+#ifdef HYK_POTRFP_TIMING
+#define HYK_STAMP(slot) do { const long long now_ = wall_clock64(); tsum[slot] += now_ - tlast; tlast = now_; } while (0)
+#define HYK_COUNT(slot) do { tsum[slot] += 1; } while (0)
+#else
+#define HYK_STAMP(slot) do { } while (0)
+#define HYK_COUNT(slot) do { } while (0)
+#endif
 
 template <bool DD, bool CPLX>
 __global__ __launch_bounds__(THREADS) void potrfp_blocked_kernel(const Args a) {
-  using R = Real<DD>; constexpr int WR = Width<DD, CPLX>::real, WE = Width<DD, CPLX>::elem;
+#ifdef HYK_POTRFP_TIMING
+  long long tsum[10] = { 0, 0, 0, 0, 0, 0, 0, 0, 0, 0 }, tlast = wall_clock64();
+#endif
+  using R = Real<DD>; using RC = Rec<DD, CPLX>; constexpr int WR = Width<DD, CPLX>::real, WE = Width<DD, CPLX>::elem, PB = CPLX ? 16 : 32;
   extern __shared__ __attribute__((aligned(16))) double lds[];
-  /* LDS: [operands / own rows: 2 * TILE * PB * WE doubles][pivot rows: PB * WE doubles][remaining columns: N uint16] */
+  /* LDS: [operands / own rows: 2 * TILE * PB * WE doubles][pivot rows: PB * WE doubles][remaining columns, pivot order, positions: N uint16 each] */
   double* const own = lds;                              /* agent: own[(t * 64 + lane) * WE + w]; update: operand A */
   double* const opB = lds + TILE * PB * WE;             /* update: operand B */
   double* const prow = lds + 2 * TILE * PB * WE;        /* agent: factor entries of the pivot column in this panel */
   uint16_t* const list = reinterpret_cast<uint16_t*>(prow + PB * WE);
+  uint16_t* const order = list + a.N;                   /* first workgroup: column at each position of the reference's swap order */
+  uint16_t* const where = order + a.N;                  /* ... and the position of each column */
   __shared__ int32_t info[4];                           /* panel end, finished, failed */
-  __shared__ int32_t piv[PB];
+  __shared__ int32_t piv[MAX_PB];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wg = blockIdx.x, nwg = gridDim.x;
   const int N = a.N, P = a.agents; const bool agent = wave == 0 && wg < P;
-  const int l = wg * 64 + lane; const bool mine = agent && l < N;
+  const int l = lane * P + wg; const bool mine = agent && l < N;   /* columns dealt round-robin to the agents: neighbouring columns (often neighbours in size) sit with different agents */
 
-  for (int i = tid; i < N; i += THREADS) { list[i] = (uint16_t)i; }
-  if (wg == 0) { for (int i = tid; i < N; i += THREADS) { st_shared_i32(&a.jpiv[i], i + 1); st_shared_i32(&a.pos[i], i); } }
+  for (int i = tid; i < N; i += THREADS) { list[i] = (uint16_t)i; order[i] = (uint16_t)i; where[i] = (uint16_t)i; }
   if (tid == 0) { info[0] = 0; info[1] = 0; info[2] = 0; }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   int na = N;
 
   /* agent state */
-  R d = R::zero(); bool dead = !mine; uint32_t epoch = 0; Msg cur; cur.bi = -1; cur.bx = cur.by = cur.tr = 0.; cur.n[0] = cur.n[1] = cur.n[2] = cur.n[3] = 0.;
-  double thresh = 0.; int k = 0; bool failed = false, stop = false;
+  R d = R::zero(); bool dead = !mine; uint32_t epoch = 0; RC cur, nxt, seen, seen2; cur.clear(); nxt.clear(); seen.clear(); seen2.clear();
+  double thresh = 0.; int k = 0; bool failed = false, stop = false; int mypiv = 0;
+  /* what was fetched for the runner-up: its column of G' and (lane t) its factor entry t of this panel */
+  int specCol = -1; R specGre = R::zero(), specGim = R::zero(); double specRow[WE], specNew[WE];
+  #pragma unroll
+  for (int w = 0; w < WE; ++w) { specRow[w] = 0.; specNew[w] = 0.; }
   const int Kstop = a.K >= N ? N - 1 : a.K;
   if (agent) {
-    Msg m; m.bx = m.by = m.tr = 0.; m.bi = -1; m.n[0] = m.n[1] = m.n[2] = m.n[3] = 0.;
+    RC m; m.clear();
     if (mine) { d = R::load_shared(&a.G[((int64_t)l + (int64_t)l * a.ldg) * WE]); m.tr = d.v.x; if (d.v.x > 0.) { m.bx = d.v.x; m.by = d.v.y; m.bi = l; } }
-    wave_reduce<DD, 6>(m.bx, m.by, m.bi, m.tr);
-    ++epoch; publish(&a.records[((size_t)(epoch & 1) * MAX_AGENTS + wg) * REC_WORDS], m, epoch);
-    failed = !collect<DD>(&a.records[(size_t)(epoch & 1) * MAX_AGENTS * REC_WORDS], P, epoch, cur);
+    reduce_wave<DD>(m.bx, m.by, m.bi, m.tr);
+    ++epoch; publish<DD, CPLX>(a.records, wg, m, epoch);
+    failed = !collect<DD, CPLX>(a.records, P, epoch, cur, seen, seen2);
     thresh = a.eps2 * cur.tr;
     stop = failed || cur.bi < 0 || k >= Kstop;
   }
@@ -415,130 +541,191 @@ __global__ __launch_bounds__(THREADS) void potrfp_blocked_kernel(const Args a) {
   for (int kb = 0, panel = 0;; kb += PB, ++panel) {
     if (wave == 0) {
       if (agent && !failed) {
+        HYK_STAMP(7);
         if (panel > 0) {   /* every workgroup has applied the previous panel to G' */
           const uint32_t want = (uint32_t)nwg * (uint32_t)panel; int spins = 0;
-          while (__hip_atomic_load(reinterpret_cast<uint32_t*>(&a.ctl[8]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < want) { if (++spins > SPIN) { failed = true; break; } __builtin_amdgcn_s_sleep(1); }
+          while (__hip_atomic_load(reinterpret_cast<uint32_t*>(&a.ctl[CTL_COUNTER]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < want) { if (++spins > SPIN) { failed = true; break; } }
         }
+        specCol = -1;
+        HYK_STAMP(0);
         while (!failed && !stop && k < kb + PB) {
+          HYK_COUNT(9);
           const int c = cur.bi, j = k - kb; R dc{ dd_t{ cur.bx, cur.by } }, sq, rho; sqrt_rsqrt<DD>(dc, sq, rho);
-          /* factor entries R[kb .. k, c] of the pivot column: lane t fetches entry t, the newest one came with the record */
-          if (lane < j - 1) {
-            const double* src = &a.Rt[((int64_t)c * a.ldr + kb + lane) * WE];
-            #pragma unroll
-            for (int w = 0; w < WE; ++w) { prow[lane * WE + w] = __hip_atomic_load(const_cast<double*>(src) + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+          const bool hit = specCol == c; const bool work = !dead && l != c;
+          if (lane == j) { mypiv = c; }
+          /* factor entries R[kb .. k, c] of the pivot column: entry t from lane t (fetched ahead on a hit: entries 0 .. j-3;
+           * else 0 .. j-2 now), the newer ones came with the records */
+          R gre = specGre, gim = specGim;
+          if (hit) {
+            HYK_COUNT(8);
+            if (lane < j - 2) {
+              #pragma unroll
+              for (int w = 0; w < WE; ++w) { prow[lane * WE + w] = specRow[w]; }
+            }
+            if (lane == 0 && j > 1) {
+              #pragma unroll
+              for (int w = 0; w < WE; ++w) { prow[(j - 2) * WE + w] = specNew[w]; }
+            }
+          } else {
+            if (lane < j - 1) {
+              const double* src = &a.Rt[((int64_t)c * a.ldr + kb + lane) * WE];
+              #pragma unroll
+              for (int w = 0; w < WE; ++w) { prow[lane * WE + w] = __hip_atomic_load(const_cast<double*>(src) + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+            }
+            if (work) {
+              if (l < c) { const double* g = &a.G[((int64_t)l + (int64_t)c * a.ldg) * WE]; gre = R::load_shared(g); if constexpr (CPLX) { gim = R::load_shared(g + WR); } }
+              else { const double* g = &a.G[((int64_t)c + (int64_t)l * a.ldg) * WE]; gre = R::load_shared(g); if constexpr (CPLX) { gim = R::load_shared(g + WR).neg(); } }
+            }
           }
           if (lane == 0 && j > 0) {
             #pragma unroll
             for (int w = 0; w < WE; ++w) { prow[(j - 1) * WE + w] = cur.n[w]; }
           }
           R rr = R::zero(), ri = R::zero();
-          const bool work = !dead && l != c;
           if (work) {
-            R gre, gim = R::zero();
-            if (l < c) { const double* g = &a.G[((int64_t)l + (int64_t)c * a.ldg) * WE]; gre = R::load_shared(g); if constexpr (CPLX) { gim = R::load_shared(g + WR); } }
-            else { const double* g = &a.G[((int64_t)c + (int64_t)l * a.ldg) * WE]; gre = R::load_shared(g); if constexpr (CPLX) { gim = R::load_shared(g + WR).neg(); } }
             R sre = gre, sim = gim;
-            for (int t = 0; t < j; ++t) {
+            #pragma unroll 4
+            for (int t = 0; t < j; ++t) {   /* unrolled so that the LDS reads of several entries are in flight together */
               const double* o = &own[(t * 64 + lane) * WE]; const double* b = &prow[t * WE];
               if constexpr (CPLX) {
                 const R ar = R::load(o), ai = R::load(o + WR), br = R::load(b), bim = R::load(b + WR);
                 /* S -= conj(a) b:  re -= ar br + ai bi;  im -= ar bi - ai br */
-                sre = R::fnma(ar, br, sre); sre = R::fnma(ai, bim, sre); sim = R::fnma(ar, bim, sim); sim = R::fnma(ai.neg(), br, sim);
-              } else { sre = R::fnma(R::load(o), R::load(b), sre); }
+                fnma_acc<DD>(ar, br, sre); fnma_acc<DD>(ai, bim, sre); fnma_acc<DD>(ar, bim, sim); fnma_acc<DD>(ai.neg(), br, sim);
+              } else { fnma_acc<DD>(R::load(o), R::load(b), sre); }
             }
-            rr = rho * sre; if constexpr (CPLX) { ri = (rho * sim).neg(); }
+            sre = renorm<DD>(sre); rr = rho * sre; if constexpr (CPLX) { sim = renorm<DD>(sim); ri = (rho * sim).neg(); }
             if constexpr (CPLX) { d = d - (rr * rr + ri * ri); } else { d = d - rr * rr; }
           }
           if (!dead && l == c) { rr = sq; ri = R::zero(); dead = true; }
           const bool wrote = work || (mine && l == c);
           if (wrote) { double* o = &own[(j * 64 + lane) * WE]; rr.store(o); if constexpr (CPLX) { ri.store(o + WR); } }
+          HYK_STAMP(1);
           /* arg-max and trace of the columns this agent still has, and the candidate's newest entry */
-          Msg m; m.bx = m.by = m.tr = 0.; m.bi = -1;
+          RC m; m.clear();
           if (!dead) { m.tr = d.v.x; if (d.v.x > 0.) { m.bx = d.v.x; m.by = d.v.y; m.bi = l; } }
-          wave_reduce<DD, 6>(m.bx, m.by, m.bi, m.tr);
-          { const int src = m.bi >= 0 ? (m.bi & 63) : 0;
-            m.n[0] = __shfl(rr.v.x, src, 64); m.n[1] = m.n[2] = m.n[3] = 0.;
-            if constexpr (DD) { m.n[1] = __shfl(rr.v.y, src, 64); }
-            if constexpr (CPLX) { m.n[WR] = __shfl(ri.v.x, src, 64); if constexpr (DD) { m.n[WR + 1] = __shfl(ri.v.y, src, 64); } } }
+          reduce_wave<DD>(m.bx, m.by, m.bi, m.tr);
+          { const int src = m.bi >= 0 ? m.bi / P : 0;
+            m.n[0] = lane_f64(rr.v.x, src);
+            if constexpr (DD) { m.n[1] = lane_f64(rr.v.y, src); }
+            if constexpr (CPLX) { m.n[WR] = lane_f64(ri.v.x, src); if constexpr (DD) { m.n[WR + 1] = lane_f64(ri.v.y, src); } } }
+          HYK_STAMP(2);
           ++k; ++epoch;
           const bool last = (k == kb + PB) || (k >= Kstop);   /* the update (or the host) reads this panel's factor entries next */
           double* out = &a.Rt[((int64_t)l * a.ldr + (k - 1)) * WE];
           if (last) { if (wrote) { rr.store_shared(out); if constexpr (CPLX) { ri.store_shared(out + WR); } } asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-          publish(&a.records[((size_t)(epoch & 1) * MAX_AGENTS + wg) * REC_WORDS], m, epoch);
+          publish<DD, CPLX>(a.records, wg, m, epoch);
           if (!last && wrote) { rr.store_shared(out); if constexpr (CPLX) { ri.store_shared(out + WR); } }
-          if (wg == 0 && lane == 0) {   /* pivot bookkeeping in the reference's swap order */
-            const int p = ld_shared_i32(&a.pos[c]), c0 = ld_shared_i32(&a.jpiv[k - 1]) - 1;
-            st_shared_i32(&a.jpiv[k - 1], c + 1); st_shared_i32(&a.jpiv[p], c0 + 1); st_shared_i32(&a.pos[c], k - 1); st_shared_i32(&a.pos[c0], p);
+          /* fetch ahead for the runner-up c2 of the arg-max that chose this step's pivot: G'[l, c2] and its factor entries
+           * 0 .. j-2 (what is certainly in memory by now); not across a panel end, where G' changes.  Issued after the
+           * record, so that nothing on the way to the record waits for these loads. */
+          runner_up<DD, CPLX>(P, c, seen, seen2, nxt);
+          const int c2 = nxt.bi; const bool ahead = c2 >= 0 && j + 1 < PB && k < Kstop;
+          if (ahead) {
+            if (lane < j - 1) {
+              const double* src = &a.Rt[((int64_t)c2 * a.ldr + kb + lane) * WE];
+              #pragma unroll
+              for (int w = 0; w < WE; ++w) { specRow[w] = __hip_atomic_load(const_cast<double*>(src) + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+            }
+            if (!dead && l != c2) {
+              if (l < c2) { const double* g = &a.G[((int64_t)l + (int64_t)c2 * a.ldg) * WE]; specGre = R::load_shared(g); if constexpr (CPLX) { specGim = R::load_shared(g + WR); } }
+              else { const double* g = &a.G[((int64_t)c2 + (int64_t)l * a.ldg) * WE]; specGre = R::load_shared(g); if constexpr (CPLX) { specGim = R::load_shared(g + WR).neg(); } }
+            }
+            #pragma unroll
+            for (int w = 0; w < WE; ++w) { specNew[w] = nxt.n[w]; }
           }
-          failed = !collect<DD>(&a.records[(size_t)(epoch & 1) * MAX_AGENTS * REC_WORDS], P, epoch, cur);
+          specCol = ahead ? c2 : -1;
+          if (wg == 0 && lane == 0) {   /* pivot bookkeeping in the reference's swap order */
+            const int p = where[c], c0 = order[k - 1]; order[k - 1] = (uint16_t)c; order[p] = (uint16_t)c0; where[c] = (uint16_t)(k - 1); where[c0] = (uint16_t)p;
+          }
+          HYK_STAMP(3);
+          failed = !collect<DD, CPLX>(a.records, P, epoch, cur, seen, seen2);
+          HYK_STAMP(4);
           if (!(thresh < cur.tr)) { cur.bi = -1; }
           stop = failed || cur.bi < 0 || k >= Kstop;
         }
-        if (wg == 0) {   /* panel summary for every workgroup: columns done, and whether the factorization ends here */
-          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-          const uint32_t seq = (uint32_t)panel + 1u;
-          if (lane == 0) { st_shared_u64(&a.ctl[0], ((uint64_t)seq << 32) | (uint32_t)k); st_shared_u64(&a.ctl[1], ((uint64_t)seq << 32) | (uint32_t)((stop ? 1 : 0) | (failed ? 2 : 0))); }
+        if (wg == 0) {   /* panel summary for every workgroup: columns done, whether the factorization ends here, the new pivots */
+          const uint32_t seq = (uint32_t)panel + 1u; const int pl = lane >= 2 ? lane - 2 : 0;
+          const int q0 = __shfl(mypiv, (2 * pl) & 63, 64), q1 = __shfl(mypiv, (2 * pl + 1) & 63, 64);   /* lane t holds the pivot of step t of this panel */
+          uint32_t payload = (uint32_t)q0 | ((uint32_t)q1 << 16); payload = lane == 0 ? (uint32_t)k : payload; payload = lane == 1 ? (uint32_t)((stop ? 1 : 0) | (failed ? 2 : 0)) : payload;
+          if (lane < 2 + PB / 2) { st_shared_u64(&a.ctl[lane], ((uint64_t)seq << 32) | payload); }
         }
       }
       /* every leader waits for the summary */
-      { const uint32_t seq = (uint32_t)panel + 1u; uint64_t s0 = 0, s1 = 0; int spins = 0; bool got = false;
+      { const uint32_t seq = (uint32_t)panel + 1u; uint64_t s = 0; int spins = 0; bool got = false;
         while (!failed) {
-          s0 = ld_shared_u64(&a.ctl[0]); s1 = ld_shared_u64(&a.ctl[1]);
-          if ((uint32_t)(s0 >> 32) == seq && (uint32_t)(s1 >> 32) == seq) { got = true; break; }
+          if (lane < 2 + PB / 2) { s = ld_shared_u64(&a.ctl[lane]); }
+          if (__all(lane >= 2 + PB / 2 || (uint32_t)(s >> 32) == seq)) { got = true; break; }
           if (++spins > SPIN) { failed = true; break; }
-          __builtin_amdgcn_s_sleep(4);
+          __builtin_amdgcn_s_sleep(2);
         }
-        if (lane == 0) { info[0] = got ? (int32_t)(uint32_t)s0 : 0; info[1] = got ? (int32_t)((uint32_t)s1 & 1u) : 1; info[2] = (failed || (got && ((uint32_t)s1 & 2u))) ? 1 : 0; }
+        const uint32_t w0 = (uint32_t)__shfl((int)(uint32_t)s, 0, 64), w1 = (uint32_t)__shfl((int)(uint32_t)s, 1, 64);
+        if (lane == 0) { info[0] = got ? (int32_t)w0 : 0; info[1] = got ? (int32_t)(w1 & 1u) : 1; info[2] = (failed || (got && (w1 & 2u))) ? 1 : 0; }
+        if (got && lane >= 2 && lane < 2 + PB / 2) { piv[2 * (lane - 2)] = (int32_t)((uint32_t)s & 0xffffu); piv[2 * (lane - 2) + 1] = (int32_t)(((uint32_t)s >> 16) & 0xffffu); }
       }
     }
     __syncthreads();
+    HYK_STAMP(5);
     const int ke = info[0], fin = info[1], bad = info[2];
-    __syncthreads();   /* info is rewritten in the next round */
     if (bad) { failed = true; break; }
     if (fin) { break; }
     const int nbk = ke - kb;
 
     /* ---- update phase ---- */
-    if (tid < nbk) { piv[tid] = ld_shared_i32(&a.jpiv[kb + tid]) - 1; }
-    __syncthreads();
-    { /* drop the new pivots from the sorted list of remaining columns */
-      constexpr int PER = MAX_N / THREADS; uint16_t keep[PER]; int16_t to[PER];
-      #pragma unroll
-      for (int e = 0; e < PER; ++e) {
-        const int idx = tid + e * THREADS; to[e] = -1;
-        if (idx < na) { const int v = list[idx]; int shift = 0; bool gone = false; for (int i = 0; i < nbk; ++i) { shift += piv[i] < v ? 1 : 0; gone = gone || piv[i] == v; } keep[e] = (uint16_t)v; if (!gone) { to[e] = (int16_t)(idx - shift); } }
-      }
+    /* drop the new pivots from the sorted list of remaining columns: an entry moves down by the number of pivots below it */
+    for (int base = 0; base < na; base += THREADS) {
+      const int idx = base + tid; int v = 0, to = -1;
+      if (idx < na) { v = list[idx]; int shift = 0; bool gone = false; for (int i = 0; i < nbk; ++i) { shift += piv[i] < v ? 1 : 0; gone = gone || piv[i] == v; } if (!gone) { to = idx - shift; } }
       __syncthreads();
-      #pragma unroll
-      for (int e = 0; e < PER; ++e) { if (to[e] >= 0) { list[to[e]] = keep[e]; } }
-      na -= nbk;
+      if (to >= 0) { list[to] = (uint16_t)v; }
       __syncthreads();
     }
+    na -= nbk;
     const int nT = (na + TILE - 1) / TILE, tiles = nT * (nT + 1) / 2;
     for (int tile = wg; tile < tiles; tile += nwg) {
       int J = (int)((sqrtf(8.f * (float)tile + 1.f) - 1.f) * 0.5f); while ((J + 1) * (J + 2) / 2 <= tile) { ++J; } while (J * (J + 1) / 2 > tile) { --J; }
       const int I = tile - J * (J + 1) / 2;
-      /* operands: the panel's factor entries of 64 remaining columns each, op[(t * 64 + col) * WE + w] */
-      for (int e = tid; e < 2 * TILE * PB; e += THREADS) {
-        const int which = e / (TILE * PB), r = e % (TILE * PB), col = r / PB, t = r % PB; if (which == 1 && I == J) { break; }
-        const int li = (which ? J : I) * TILE + col; double* dst = &(which ? opB : own)[(t * 64 + col) * WE];
-        if (li < na && t < nbk) {
-          const double* src = &a.Rt[((int64_t)list[li] * a.ldr + kb + t) * WE];
+      /* operands: the panel's factor entries of 64 remaining columns each, op[(t * 64 + col) * WE + w]; all loads of a
+       * thread are issued before the first is stored, so that their latencies overlap */
+      { constexpr int PER = TILE * PB / THREADS;
+        #pragma unroll
+        for (int which = 0; which < 2; ++which) {
+          if (which == 1 && I == J) { break; }
+          double v[PER][WE];
           #pragma unroll
-          for (int w = 0; w < WE; ++w) { dst[w] = __hip_atomic_load(const_cast<double*>(src) + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-        } else {
+          for (int e = 0; e < PER; ++e) {
+            const int r = tid + e * THREADS, col = r / PB, t = r % PB, li = (which ? J : I) * TILE + col;
+            #pragma unroll
+            for (int w = 0; w < WE; ++w) { v[e][w] = 0.; }
+            if (li < na && t < nbk) {
+              const double* src = &a.Rt[((int64_t)list[li] * a.ldr + kb + t) * WE];
+              #pragma unroll
+              for (int w = 0; w < WE; ++w) { v[e][w] = __hip_atomic_load(const_cast<double*>(src) + w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+            }
+          }
           #pragma unroll
-          for (int w = 0; w < WE; ++w) { dst[w] = 0.; }
+          for (int e = 0; e < PER; ++e) {
+            const int r = tid + e * THREADS, col = r / PB, t = r % PB; double* dst = &(which ? opB : own)[(t * 64 + col) * WE];
+            #pragma unroll
+            for (int w = 0; w < WE; ++w) { dst[w] = v[e][w]; }
+          }
         }
       }
       __syncthreads();
       const double* A = own; const double* B = I == J ? own : opB;
       const int ry = (wave >> 1) * 32 + (lane & 7), cx = (wave & 1) * 32 + (lane >> 3);
-      R sre[4][4], sim[4][4];
+      /* G'[l, m] for the 16 pairs of this lane: requested now, needed after the products */
+      R gre[4][4], gim[4][4]; double* gp[4][4];
       #pragma unroll
       for (int i = 0; i < 4; ++i) {
+        const int li = I * TILE + ry + 8 * i; const int lcol = li < na ? list[li] : 0;
         #pragma unroll
-        for (int jj = 0; jj < 4; ++jj) { sre[i][jj] = R::zero(); sim[i][jj] = R::zero(); }
+        for (int jj = 0; jj < 4; ++jj) {
+          const int mi = J * TILE + cx + 8 * jj; gp[i][jj] = nullptr; gre[i][jj] = R::zero(); gim[i][jj] = R::zero();
+          if (li < na && mi < na && li < mi) {
+            double* g = &a.G[((int64_t)lcol + (int64_t)list[mi] * a.ldg) * WE]; gp[i][jj] = g;
+            gre[i][jj] = R::load_shared(g); if constexpr (CPLX) { gim[i][jj] = R::load_shared(g + WR); }
+          }
+        }
       }
       for (int t = 0; t < nbk; ++t) {
         R ar[4], ai[4], br[4], bi[4];
@@ -552,40 +739,46 @@ __global__ __launch_bounds__(THREADS) void potrfp_blocked_kernel(const Args a) {
           #pragma unroll
           for (int jj = 0; jj < 4; ++jj) {
             /* G'[l, m] -= conj(R[t, l]) R[t, m] */
-            sre[i][jj] = R::fnma(ar[i], br[jj], sre[i][jj]);
-            if constexpr (CPLX) { sre[i][jj] = R::fnma(ai[i], bi[jj], sre[i][jj]); sim[i][jj] = R::fnma(ar[i], bi[jj], sim[i][jj]); sim[i][jj] = R::fnma(ai[i].neg(), br[jj], sim[i][jj]); }
+            fnma_acc<DD>(ar[i], br[jj], gre[i][jj]);
+            if constexpr (CPLX) { fnma_acc<DD>(ai[i], bi[jj], gre[i][jj]); fnma_acc<DD>(ar[i], bi[jj], gim[i][jj]); fnma_acc<DD>(ai[i].neg(), br[jj], gim[i][jj]); }
           }
         }
       }
       #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int li = I * TILE + ry + 8 * i; if (li >= na) { continue; } const int lcol = list[li];
         #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
-          const int mi = J * TILE + cx + 8 * jj; if (mi >= na || li >= mi) { continue; } const int mcol = list[mi];
-          double* g = &a.G[((int64_t)lcol + (int64_t)mcol * a.ldg) * WE];
-          (R::load_shared(g) + sre[i][jj]).store_shared(g);
-          if constexpr (CPLX) { (R::load_shared(g + WR) + sim[i][jj]).store_shared(g + WR); }
+          if (gp[i][jj]) { renorm<DD>(gre[i][jj]).store_shared(gp[i][jj]); if constexpr (CPLX) { renorm<DD>(gim[i][jj]).store_shared(gp[i][jj] + WR); } }
         }
       }
       __syncthreads();
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (tid == 0) { __hip_atomic_fetch_add(reinterpret_cast<uint32_t*>(&a.ctl[8]), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+    if (tid == 0) { __hip_atomic_fetch_add(reinterpret_cast<uint32_t*>(&a.ctl[CTL_COUNTER]), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+    HYK_STAMP(6);
   }
+#ifdef HYK_POTRFP_TIMING
+  if (wg == 0 && tid == 0) { for (int i = 0; i < 10; ++i) { a.ctl[CTL_TIMING + i] = (uint64_t)tsum[i]; } }
+#endif
 
   /* reference quirk (src/hyacin_potrfp.cu:271): when exactly one column is left it is counted and its diagonal written */
   if (agent && !failed && N - k == 1 && !dead) {
     R sq = R::zero(), rho; if (d.v.x > 0.) { sqrt_rsqrt<DD>(d, sq, rho); }
     double* rc = &a.Rt[((int64_t)l * a.ldr + k) * WE]; sq.store(rc); if constexpr (CPLX) { R::zero().store(rc + WR); }
   }
-  if (wg == 0 && tid == 0) { *a.rankOut = failed ? -1 : ((N - k == 1) ? k + 1 : k); }
+  __syncthreads();
+  if (wg == 0) {
+    if (tid == 0) { info[3] = k; }   /* the agent's count of columns done */
+    __syncthreads();
+    for (int i = tid; i < N; i += THREADS) { a.jpiv[i] = (int32_t)order[i] + 1; }
+    if (tid == 0) { *a.rankOut = failed ? -1 : ((N - info[3] == 1) ? info[3] + 1 : info[3]); }
+  }
 }
 
 template <bool DD, bool CPLX> int launch(hipStream_t stream, Args& args, int cus) {
-  constexpr int WE = Width<DD, CPLX>::elem;
-  const size_t ldsBytes = (size_t)(2 * TILE * PB * WE + PB * WE) * 8 + (size_t)args.N * 2 + 16;
+  constexpr int WE = Width<DD, CPLX>::elem, PB = CPLX ? 16 : 32;
+  const size_t ldsBytes = (size_t)(2 * TILE * PB * WE + PB * WE) * 8 + (size_t)args.N * 6 + 16;
   const void* fn = reinterpret_cast<const void*>(&potrfp_blocked_kernel<DD, CPLX>);
   if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes) != hipSuccess) { return -3; }
   int perCu = 0; if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, potrfp_blocked_kernel<DD, CPLX>, THREADS, ldsBytes) != hipSuccess || perCu < 1) { return -3; }
@@ -602,7 +795,7 @@ __global__ void clear_kernel(uint64_t* p, int words) { for (int i = threadIdx.x;
 
 namespace {
 /* workspace: [pos: N int32][exchange area: records / control words of either kernel][D: N reals (left-looking kernel)] */
-constexpr size_t EXCHANGE_BYTES = 2 * blk::MAX_AGENTS * blk::REC_WORDS * 8 + blk::CTL_WORDS * 8;
+constexpr size_t EXCHANGE_BYTES = 2 * blk::MAX_AGENTS * blk::REC_WORDS * 8 + blk::CTL_WORDS * 8;   /* 33 280 bytes */
 static_assert(EXCHANGE_BYTES >= 2 * MAX_WORKGROUPS * sizeof(Record), "the exchange area holds the records of either kernel");
 size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 
@@ -617,7 +810,7 @@ int run_potrfp(hipStream_t stream, bool blocked, int32_t computeUnits, double ep
   blk::clear_kernel<<<1, 256, 0, stream>>>(exchange, (int)(EXCHANGE_BYTES / 8));
   const int agents = (N + 63) / 64, grid = computeUnits < 256 ? computeUnits : 256;
   if (blocked && N <= blk::MAX_N && agents <= grid) {
-    blk::Args b; b.N = N; b.K = K; b.ldr = ldr; b.agents = agents; b.eps2 = eps * eps; b.G = (double*)G; b.ldg = ldg; b.Rt = (double*)Rt; b.jpiv = jpiv; b.pos = pos;
+    blk::Args b; b.N = N; b.K = K; b.ldr = ldr; b.agents = agents; b.eps2 = eps * eps; b.G = (double*)G; b.ldg = ldg; b.Rt = (double*)Rt; b.jpiv = jpiv;
     b.records = exchange; b.ctl = exchange + 2 * blk::MAX_AGENTS * blk::REC_WORDS; b.rankOut = rankOut;
     if (dd) { return cplx ? blk::launch<true, true>(stream, b, computeUnits) : blk::launch<true, false>(stream, b, computeUnits); }
     return cplx ? blk::launch<false, true>(stream, b, computeUnits) : blk::launch<false, false>(stream, b, computeUnits);
