@@ -33,7 +33,7 @@ KERNEL_SYMBOLS = [
     "hykGramWorkspaceBytes", "hykGramWorkspaceClear", "hykGramCrt", "hykGramLimbs", "hykGramSetSlab",
     "hykGramProfile", "hykGramProfileRead", "hykMfmaCeiling", "hykGramRange", "hykDequantize", "hykPotrfpWorkspaceBytes", "hykPotrfp", "hykPotrfpLeftLooking", "hykPotrfpStaticMaxN", "hykPotrfpStatic", "hykFactorToB", "hykJacobiSweep", "hykJacobiSweepCarry", "hykJacobiCarryBytes", "hykJacobiSetVariant",
     "hykColumnNorms", "hykBasisOut", "hykValuesOut", "hykInterpSolve", "hykInterpOut", "hykMatcopy",
-    "hykSumSquares", "hykMatmulCf16", "hykGemm", "hykOrthonormalize",
+    "hykSumSquares", "hykMatmulCf16", "hykGemm", "hykOrthonormalize", "hykLastStatus", "hykTestFailAllocation",
 ]
 
 
@@ -106,6 +106,8 @@ def lib():
         L.hykMatmulCf16.argtypes = [vp, ch, i32, i32, i32, vp, i64, vp, i64, vp, i64]
         L.hykSumSquares.argtypes = [vp, i64, i64, vp, i64, vp]
         L.hykOrthonormalize.argtypes = [vp, i32, i32, i32, vp, i64, vp]
+        L.hykLastStatus.argtypes = []
+        L.hykTestFailAllocation.argtypes = [i32]
         L.hykFactorToB.argtypes = [vp, i32, i32, i32, vp, i32, vp]
         L.hykColumnNorms.argtypes = [vp, i32, i32, i32, vp, vp]
         L.hykBasisOut.argtypes = [vp, i32, i32, i32, vp, vp, vp, vp, i64]

@@ -41,6 +41,7 @@
  */
 #include <vector>
 #include <type_traits>
+#include <atomic>
 #include <hip/hip_runtime.h>
 #include "hyk_common.h"
 #include "crt_tables.h"
@@ -768,16 +769,18 @@ __global__ void fill_zero_kernel(uint4* __restrict__ p, int64_t n16) {
 /* ------------------------------------------------------------------ host-side planning */
 struct Launch { GramArgs args; int epi; };
 
-int g_bk = 0;   /* 0: direct-to-LDS ring of 128-byte rows (default); 2: direct-to-LDS ring of 64-byte rows; 64 / 128: register-staged kernel with that K slab (hykGramSetSlab) */
+/* Tuning and measuring state is per host thread: a setting made on one thread never changes what another thread's calls
+ * launch, and nothing here is shared between threads. */
+thread_local int g_bk = 0;   /* 0: direct-to-LDS ring of 128-byte rows (default); 2: direct-to-LDS ring of 64-byte rows; 64 / 128: register-staged kernel with that K slab (hykGramSetSlab) */
 
 /* optional per-launch timing of the contraction kernel with HIP events on its own stream */
 struct Timed { hipEvent_t start, stop; };
-bool g_profile = false; std::vector<Timed> g_timed;
+thread_local bool g_profile = false; thread_local std::vector<Timed> g_timed;
 
 template <int BK, int EPI> hipError_t launch_one(hipStream_t stream, const GramArgs& a) {
   const int ldsBytes = 2 * 2 * Slab<BK>::TILE_BYTES;
-  static bool attr = false;
-  if (!attr) { hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gram_kernel<BK, EPI>), hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes); if (e != hipSuccess) { return e; } attr = true; }
+  static std::atomic<bool> attr{ false };   /* two threads arriving together both set the attribute: harmless */
+  if (!attr.load(std::memory_order_acquire)) { hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gram_kernel<BK, EPI>), hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes); if (e != hipSuccess) { return e; } attr.store(true, std::memory_order_release); }
   const int blocks = a.itemsPerXcd * XCDS;
   Timed t{ nullptr, nullptr };
   if (g_profile) { if (hipEventCreate(&t.start) != hipSuccess || hipEventCreate(&t.stop) != hipSuccess) { return hipErrorUnknown; } (void)hipEventRecord(t.start, stream); }
@@ -788,8 +791,8 @@ template <int BK, int EPI> hipError_t launch_one(hipStream_t stream, const GramA
 
 template <int EPI, bool EXCL> hipError_t launch_dma(hipStream_t stream, const GramArgs& a) {
   const int ldsBytes = DMA_STAGES * DMA_STAGE_BYTES;
-  static bool attr = false;
-  if (!attr) { hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gram_dma_kernel<EPI, EXCL>), hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes); if (e != hipSuccess) { return e; } attr = true; }
+  static std::atomic<bool> attr{ false };   /* two threads arriving together both set the attribute: harmless */
+  if (!attr.load(std::memory_order_acquire)) { hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gram_dma_kernel<EPI, EXCL>), hipFuncAttributeMaxDynamicSharedMemorySize, ldsBytes); if (e != hipSuccess) { return e; } attr.store(true, std::memory_order_release); }
   const int blocks = a.itemsPerXcd * XCDS;
   Timed t{ nullptr, nullptr };
   if (g_profile) { if (hipEventCreate(&t.start) != hipSuccess || hipEventCreate(&t.stop) != hipSuccess) { return hipErrorUnknown; } (void)hipEventRecord(t.start, stream); }
@@ -799,8 +802,8 @@ template <int EPI, bool EXCL> hipError_t launch_dma(hipStream_t stream, const Gr
 }
 
 template <int EPI, bool EXCL> hipError_t launch_ring(hipStream_t stream, const GramArgs& a) {
-  static bool attr = false;
-  if (!attr) { hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gram_ring_kernel<EPI, EXCL>), hipFuncAttributeMaxDynamicSharedMemorySize, RING_BYTES); if (e != hipSuccess) { return e; } attr = true; }
+  static std::atomic<bool> attr{ false };   /* two threads arriving together both set the attribute: harmless */
+  if (!attr.load(std::memory_order_acquire)) { hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gram_ring_kernel<EPI, EXCL>), hipFuncAttributeMaxDynamicSharedMemorySize, RING_BYTES); if (e != hipSuccess) { return e; } attr.store(true, std::memory_order_release); }
   const int blocks = XCDS * a.roundsPerXcd * (1 << a.slotShift);
   Timed t{ nullptr, nullptr };
   if (g_profile) { if (hipEventCreate(&t.start) != hipSuccess || hipEventCreate(&t.stop) != hipSuccess) { return hipErrorUnknown; } (void)hipEventRecord(t.start, stream); }
@@ -809,10 +812,10 @@ template <int EPI, bool EXCL> hipError_t launch_ring(hipStream_t stream, const G
   return hipGetLastError();
 }
 
-int compute_units() {
-  static int units = 0;
-  if (units == 0) { int dev = 0, n = 0; if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) { units = n; } else { units = 256; } }
-  return units;
+int compute_units() {   /* of the device current on this thread */
+  int dev = 0, n = 0;
+  if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) { return n; }
+  return 256;
 }
 
 hipError_t launch_gram(hipStream_t stream, GramArgs& a, int epi, int maxProducts, bool unshared, bool paired) {

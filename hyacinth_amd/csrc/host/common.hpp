@@ -13,10 +13,21 @@
 
 namespace hyh {
 
-/* A failed runtime call or kernel launch is reported on stderr once per call site and the call chain carries on,
- * like the reference's release build; silent wrong answers are worse than noise. */
-#define HYH_CHECK(call) do { hipError_t hyh_e_ = (call); if (hyh_e_ != hipSuccess) { std::fprintf(stderr, "hyacin: %s failed: %s (%s:%d)\n", #call, hipGetErrorString(hyh_e_), __FILE__, __LINE__); } } while (0)
-#define HYH_KERNEL(call) do { int hyh_r_ = (call); if (hyh_r_ != 0) { std::fprintf(stderr, "hyacin: %s returned %d (%s:%d)\n", #call, hyh_r_, __FILE__, __LINE__); } } while (0)
+/* Failure handling.  A failed runtime call, allocation or kernel-layer call is reported on stderr and recorded as the
+ * status of the hyacin.h call that is running on this thread; from then on that call launches nothing more (HYH_KERNEL
+ * skips its argument), frees what it holds and returns 0 / leaves its outputs as they are.  The status of the last
+ * outermost call stays readable through hykLastStatus() until the thread's next hyacin.h call. */
+struct CallStatus { int code = 0; int depth = 0; };
+CallStatus& call_status();
+inline bool ok() { return call_status().code == 0; }
+void fail(int code, const char* what, const char* detail, const char* file, int line);
+struct ApiScope {   /* first statement of every hyacin.h function: the outermost one starts with a clean status */
+  ApiScope() { CallStatus& s = call_status(); if (s.depth++ == 0) { s.code = 0; } }
+  ~ApiScope() { --call_status().depth; }
+  ApiScope(const ApiScope&) = delete; ApiScope& operator=(const ApiScope&) = delete;
+};
+#define HYH_CHECK(call) do { hipError_t hyh_e_ = (call); if (hyh_e_ != hipSuccess) { hyh::fail((int)hyh_e_, #call, hipGetErrorString(hyh_e_), __FILE__, __LINE__); } } while (0)
+#define HYH_KERNEL(call) do { if (hyh::ok()) { int hyh_r_ = (call); if (hyh_r_ != 0) { hyh::fail(hyh_r_, #call, "kernel layer refused or failed to launch", __FILE__, __LINE__); } } } while (0)
 
 inline bool is_complex(int t) { return (t & 1) != 0; }
 inline int elem_bytes(int t) { static const int b[12] = { 8, 16, 4, 8, 2, 4, 16, 32, 12, 24, 16, 32 }; return (t >= 0 && t < 12) ? b[t] : 0; }
@@ -30,7 +41,9 @@ void scratch_release(const hyacinHandle_t* h, void* p, bool kept);
 void scratch_drop_all(const hyacinHandle_t* h);
 struct Scratch {
   const hyacinHandle_t* h; void* p = nullptr; bool kept = false;
-  Scratch(const hyacinHandle_t* h_, size_t bytes) : h(h_) { if (bytes) { p = scratch_acquire(h, bytes, &kept); } }
+  Scratch(const hyacinHandle_t* h_, size_t bytes) : h(h_) {
+    if (bytes && ok()) { p = scratch_acquire(h, bytes, &kept); if (!p) { fail(-4, "scratch allocation", "the memory pool returned no block", __FILE__, __LINE__); } }
+  }
   ~Scratch() { if (p) { scratch_release(h, p, kept); } }
   Scratch(const Scratch&) = delete; Scratch& operator=(const Scratch&) = delete;
   template <typename T> T* as() const { return reinterpret_cast<T*>(p); }

@@ -10,6 +10,7 @@
 #include <string>
 #include <map>
 #include <mutex>
+#include <atomic>
 #include "common.hpp"
 
 namespace {
@@ -22,12 +23,15 @@ struct EventTimer { std::vector<std::pair<hyh::Segment, hipEvent_t>> events; hyh
 struct Block { void* p; size_t bytes; bool busy; };
 std::mutex g_keptMutex; std::map<hipMemPool_t, std::vector<Block>> g_kept;
 
+std::atomic<int> g_failAllocation{ 0 };   /* test hook: the n-th scratch acquisition from now on fails */
+
 bool env_get(const char* key, std::string& out) { const char* v = std::getenv(key); if (!v) { return false; } out = v; return true; }
 bool env_true(const std::string& s) { return s == "1" || s == "true" || s == "True"; }
 
 }  // namespace
 
 extern "C" void hyacinCreate(hyacinHandle_t* handle) {
+  hyh::ApiScope scope;
   if (!handle) { return; }
   HYH_CHECK(hipGetDevice(&handle->DeviceID));
   HYH_CHECK(hipDeviceGetAttribute(&handle->DeviceSMs, hipDeviceAttributeMultiprocessorCount, handle->DeviceID));
@@ -59,8 +63,19 @@ extern "C" void hyacinCreate(hyacinHandle_t* handle) {
   if (verbose && handle->logger == nullptr) { handle->logger = stdout; }
 }
 
+hyh::CallStatus& hyh::call_status() { static thread_local CallStatus s; return s; }
+
+void hyh::fail(int code, const char* what, const char* detail, const char* file, int line) {
+  std::fprintf(stderr, "hyacin: %s failed (%d: %s) at %s:%d\n", what, code, detail, file, line);
+  CallStatus& s = call_status(); if (s.code == 0) { s.code = code ? code : -1; }
+}
+
+extern "C" int hykLastStatus(void) { return hyh::call_status().code; }
+extern "C" int hykTestFailAllocation(int32_t nth) { g_failAllocation.store(nth > 0 ? nth : 0); return 0; }
+
 void* hyh::scratch_acquire(const hyacinHandle_t* h, size_t bytes, bool* kept) {
   void* p = nullptr; *kept = false;
+  if (g_failAllocation.load(std::memory_order_relaxed) > 0 && g_failAllocation.fetch_sub(1) == 1) { return nullptr; }
   if ((h->HandleOwnedResource & OWNS_MEMPOOL) && h->mempool) {
     std::lock_guard<std::mutex> lock(g_keptMutex);
     std::vector<Block>& blocks = g_kept[h->mempool]; Block* best = nullptr;
@@ -93,6 +108,7 @@ void hyh::scratch_drop_all(const hyacinHandle_t* h) {
 }
 
 extern "C" void hyacinDestroy(hyacinHandle_t* handle) {
+  hyh::ApiScope scope;
   if (!handle) { return; }
   if ((handle->HandleOwnedResource & OWNS_MEMPOOL) && handle->mempool) { hyh::scratch_drop_all(handle); }
   HYH_CHECK(hipDeviceSynchronize());
@@ -110,6 +126,7 @@ void hyh::timer_mark(const hyacinHandle_t* h, hyh::Segment seg) {
 }
 
 extern "C" void hyacinSync_TimerSegments(const hyacinHandle_t* handle, double* eventMs, int32_t lenMs) {
+  hyh::ApiScope scope;
   if (handle->timer == nullptr) { HYH_CHECK(hipStreamSynchronize(handle->hipStream)); return; }
   EventTimer* t = (EventTimer*)handle->timer; const int len = (int)t->events.size();
   hipEvent_t e; HYH_CHECK(hipEventCreate(&e)); HYH_CHECK(hipEventRecord(e, handle->hipStream)); HYH_CHECK(hipEventSynchronize(e));

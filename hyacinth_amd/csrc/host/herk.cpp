@@ -48,6 +48,7 @@ hyh::GramPlan hyh::gram_algorithm(char alg, int32_t K, int32_t u, int32_t Comple
 }
 
 extern "C" void hyacinXherkBatchInit(const hyacinHandle_t* handle, double eps, uint64_t M, int32_t N, hyacinPrecision_t Atype, int32_t* uA, int32_t* cPanels, int32_t* lPanels, uint64_t* stride) {
+  hyh::ApiScope scope;
   if (stride) { const uint64_t n = (uint64_t)std::max(0, N); *stride = (n * n + n) >> 1; }
   if (!uA && !cPanels && !lPanels) { return; }
   static const int32_t mantissa[12] = { 52, 52, 23, 23, 10, 10, 105, 105, 71, 71, 95, 95 };
@@ -61,6 +62,7 @@ extern "C" void hyacinXherkBatchInit(const hyacinHandle_t* handle, double eps, u
 }
 
 extern "C" void hyacinXquantizeScaleBatch(const hyacinHandle_t* handle, int32_t batches, int32_t segM, int32_t lastM, int32_t N, hyacinPrecision_t Atype, const void* A, int32_t lda, int32_t uA, int32_t* vexp) {
+  hyh::ApiScope scope;
   if (N <= 0 || (int)Atype > HYACIN_F16_COMPLEX) { return; }
   hyh::timer_mark(handle, hyh::Segment::dist_kernel);
   HYH_KERNEL(hykColumnExponents(handle->hipStream, batches, segM, lastM, N, (int32_t)Atype, A, lda, uA, vexp));
@@ -93,6 +95,7 @@ void limb_bucket(Ctx& c, const std::vector<Run>& runs, int32_t order) {
   const size_t wsBytes = hykGramWorkspaceBytes(HYK_GRAM_LIMBS, c.Complex, c.N, order);
   const int64_t ld = panel_ld(cap);
   hyh::Scratch W(c.h, (size_t)ld * (size_t)rowBytes), ws(c.h, wsBytes);
+  if (!hyh::ok()) { return; }
   HYH_KERNEL(hykGramWorkspaceClear(c.s, ws.p, wsBytes));
   int32_t filled = 0;
   auto flush = [&]() {
@@ -119,6 +122,7 @@ void crt_bucket(Ctx& c, const std::vector<Run>& runs, int32_t order, int32_t chu
   const size_t wsBytes = hykGramWorkspaceBytes(HYK_GRAM_CRT, c.Complex, c.N, order);
   const int64_t ld = panel_ld(cap);
   hyh::Scratch W(c.h, (size_t)ld * (size_t)rowBytes), ws(c.h, wsBytes);
+  if (!hyh::ok()) { return; }
   HYH_KERNEL(hykGramWorkspaceClear(c.s, ws.p, wsBytes));
   int32_t filled = 0;
   auto flush = [&]() {
@@ -156,7 +160,8 @@ void herk_sliced(Ctx& c, int32_t batches, int32_t segM, int32_t lastM) {
   std::vector<int32_t> segU((size_t)batches);
   { hyh::Scratch d(c.h, sizeof(int32_t) * (size_t)batches);
     HYH_KERNEL(hykSliceRange(c.s, batches, c.N, c.u + c.Complex, c.vexp, d.as<int32_t>()));
-    HYH_CHECK(hipMemcpyAsync(segU.data(), d.p, sizeof(int32_t) * (size_t)batches, hipMemcpyDeviceToHost, c.s)); HYH_CHECK(hipStreamSynchronize(c.s)); }
+    if (hyh::ok()) { HYH_CHECK(hipMemcpyAsync(segU.data(), d.p, sizeof(int32_t) * (size_t)batches, hipMemcpyDeviceToHost, c.s)); } HYH_CHECK(hipStreamSynchronize(c.s)); }
+  if (!hyh::ok()) { return; }
   /* precision levels at which the limb path wins: slices whose own bit range fits level i are contracted with that few limbs */
   std::vector<hyh::GramPlan> limbLevels; int32_t uFloor = c.Complex;
   while (uFloor <= uCeil) {
@@ -191,6 +196,7 @@ void herk_sliced(Ctx& c, int32_t batches, int32_t segM, int32_t lastM) {
 }  // namespace
 
 extern "C" void hyacinXherkBatch(const hyacinHandle_t* handle, int32_t batches, int32_t segM, int32_t lastM, int32_t N, hyacinPrecision_t Atype, const void* A, int32_t lda, int32_t u, const int32_t* vexp, int32_t beta, int32_t orderC, uint64_t* C) {
+  hyh::ApiScope scope;
   if (N <= 0 || orderC <= 0 || (int)Atype < 0 || (int)Atype > HYACIN_F16_COMPLEX) { return; }
   hyh::timer_mark(handle, hyh::Segment::dist_kernel);
   Ctx c{ handle, handle->hipStream, N, (int32_t)Atype, (int32_t)Atype & 1, u, (const char*)A, lda, vexp, beta, orderC, C };
@@ -198,9 +204,10 @@ extern "C" void hyacinXherkBatch(const hyacinHandle_t* handle, int32_t batches, 
 }
 
 extern "C" void hyacinXdequantizeInit(const hyacinHandle_t* handle, int32_t N, int32_t orderC, const uint64_t* C, const int32_t* vexp, hyacinPrecision_t Atype, hyacinPrecision_t* Gtype, int32_t* gElemBytes) {
+  hyh::ApiScope scope;
   if (N <= 0 && (Gtype != nullptr || gElemBytes != nullptr)) { return; }
   hyh::timer_mark(handle, hyh::Segment::rep_kernel);
-  int32_t* word = (int32_t*)handle->pinnedWorkspace; *word = 0;
+  int32_t* word = (int32_t*)handle->pinnedWorkspace; if (!word) { hyh::fail(-1, "hyacinXdequantizeInit", "the handle has no pinned word (hyacinCreate not called?)", __FILE__, __LINE__); return; } *word = 0;
   if (N > 0 && orderC >= 1 && orderC <= 3) { HYH_KERNEL(hykGramRange(handle->hipStream, N, orderC, C, vexp, word)); }
   HYH_CHECK(hipStreamSynchronize(handle->hipStream));
   /* significant bits of the Gram = bit length of the dominant diagonal entry minus the 2 x correction bits of head-room */
@@ -211,6 +218,7 @@ extern "C" void hyacinXdequantizeInit(const hyacinHandle_t* handle, int32_t N, i
 }
 
 extern "C" void hyacinXdequantize(const hyacinHandle_t* handle, int32_t N, int32_t orderC, const uint64_t* C, const int32_t* vexp, hyacinPrecision_t Gtype, void* G, int32_t ldg) {
+  hyh::ApiScope scope;
   if (N <= 0) { return; }
   hyh::timer_mark(handle, hyh::Segment::rep_kernel);
   HYH_KERNEL(hykDequantize(handle->hipStream, N, orderC, C, vexp, (int32_t)Gtype, G, ldg));

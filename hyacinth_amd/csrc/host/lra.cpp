@@ -29,8 +29,10 @@ int32_t fit_common(const hyacinHandle_t* h, double eps, char opA, int32_t M, int
   int32_t u = 0, cPanels = 1, lPanels = 1; uint64_t strideC = 0;
   hyacinXherkBatchInit(h, eps, (uint64_t)globalM, N, (hyacinPrecision_t)Atype, &u, &cPanels, &lPanels, &strideC);
   hyh::Scratch vexp(h, sizeof(int32_t) * (size_t)(sl.batches + 1) * (size_t)N), C(h, sizeof(uint64_t) * (size_t)cPanels * (size_t)std::max(1, lPanels) * (size_t)strideC);
+  if (!hyh::ok()) { return 0; }
   if (opA == 'T' || opA == 'C') {
     hyh::Scratch AH(h, (size_t)M * (size_t)N * (size_t)hyh::elem_bytes(Atype));
+    if (!hyh::ok()) { return 0; }
     HYH_KERNEL(hykMatcopy(s, opA, M, N, Atype, A, lda, Atype, AH.p, M));
     hyacinXquantizeScaleBatch(h, sl.batches, sl.batchIter, sl.lastM, N, (hyacinPrecision_t)Atype, AH.p, M, u, vexp.as<int32_t>());
     hyacinAllReduceVExp(h, (uint64_t)N, vexp.as<int32_t>());
@@ -41,12 +43,16 @@ int32_t fit_common(const hyacinHandle_t* h, double eps, char opA, int32_t M, int
     hyacinXherkBatch(h, sl.batches, sl.batchIter, sl.lastM, N, (hyacinPrecision_t)Atype, A, lda, u, vexp.as<int32_t>(), 0, lPanels, C.as<uint64_t>());
   }
   hyacinAllReduce1Drow(h, cPanels, lPanels, strideC, C.as<uint64_t>());
-  if (lPanels <= 0) { return 0; }   /* u < 0: nothing was quantized */
+  if (lPanels <= 0 || !hyh::ok()) { return 0; }   /* u < 0: nothing was quantized */
   hyacinPrecision_t Gtype = HYACIN_F64; int32_t gBytes = 8;
   hyacinXdequantizeInit(h, N, lPanels, C.as<uint64_t>(), vexp.as<int32_t>(), (hyacinPrecision_t)Atype, &Gtype, &gBytes);
+  if (!hyh::ok()) { return 0; }
   hyh::Scratch G(h, (size_t)N * (size_t)N * (size_t)gBytes);
+  if (!hyh::ok()) { return 0; }
   hyacinXdequantize(h, N, lPanels, C.as<uint64_t>(), vexp.as<int32_t>(), Gtype, G.p, N);
-  return tail(Gtype, G.p);
+  if (!hyh::ok()) { return 0; }
+  const int32_t rank = tail(Gtype, G.p);
+  return hyh::ok() ? rank : 0;
 }
 
 int32_t svd_fit(const hyacinHandle_t* h, double eps, char opA, int32_t M, int32_t N, int32_t K, int Atype, const void* A, int32_t lda, void* S, void* V, int32_t ldv, int64_t globalM) {
@@ -71,16 +77,19 @@ int32_t svd_fit_segmented(const hyacinHandle_t* h, double eps, char opA, int32_t
   const int32_t q = N / segments, r = N % segments, N1 = q + (0 < r ? 1 : 0); const size_t eb = (size_t)hyh::elem_bytes(Atype), v1Stride = (size_t)N1 * N1;
   const size_t sBytes = (size_t)(eb / (1 + (Atype & 1)));
   hyh::Scratch V1(h, v1Stride * segments * eb), S1(h, (size_t)N1 * sBytes);
+  if (!hyh::ok()) { return 0; }
   std::vector<int32_t> ranks; int64_t locA = 0;
   for (int32_t i = 0; i < segments; ++i) {
     const int32_t cols = q + (i < r ? 1 : 0);
     ranks.push_back(svd_fit(h, eps, opA, M, cols, cols, Atype, at(A, locA, Atype), lda, S1.p, at(V1.p, (int64_t)(i * v1Stride), Atype), N1, globalM));
     locA += transA ? cols : (int64_t)cols * lda;
+    if (!hyh::ok()) { return 0; }
   }
   const int32_t N2 = std::accumulate(ranks.begin(), ranks.end(), 0); if (N2 <= 0) { return 0; }
   int32_t rank;
   hyh::Scratch V2(h, (size_t)N2 * std::min(N2, K) * eb);
   { hyh::Scratch A2(h, (size_t)M * N2 * eb); locA = 0; int64_t locA2 = 0;
+    if (!hyh::ok()) { return 0; }
     hyh::timer_mark(h, hyh::Segment::dist_kernel);
     if (0 < M) for (int32_t i = 0; i < segments; ++i) {
       const int32_t cols = q + (i < r ? 1 : 0);
@@ -98,7 +107,7 @@ int32_t svd_fit_segmented(const hyacinHandle_t* h, double eps, char opA, int32_t
     else if (rank > 0) { HYH_KERNEL(hykGemm(s, 'N', 'N', cols, rank, 0, 0.0, Atype, V1.p, N1, V2.p, N2, 0.0, at(V, row, Atype), ldv)); }
     row += cols; rowV += ranks[i];
   }
-  return rank;
+  return hyh::ok() ? rank : 0;
 }
 
 /* reference: check_answer, src/lra.cpp:158-208 */
@@ -107,9 +116,10 @@ double check_norm(const hyacinHandle_t* h, char opA, int32_t M, int32_t N, int32
   hyh::timer_mark(h, hyh::Segment::untimed);
   opA = norm_op(opA); const bool transA = opA == 'T' || opA == 'C'; const int Complex = Atype & 1, wide = HYACIN_F64 + Complex; const int32_t block = 2048;
   const size_t eb = (size_t)8 * (1 + Complex); hipStream_t s = h->hipStream; const char mode = transA ? opA : 'A';
-  hyh::Scratch acc(h, 64); HYH_KERNEL(hykGramWorkspaceClear(s, acc.p, 64));
+  hyh::Scratch acc(h, 64); if (!hyh::ok()) { return 0.; } HYH_KERNEL(hykGramWorkspaceClear(s, acc.p, 64));
   if (rank <= 0) {
     hyh::Scratch matA(h, (size_t)block * block * eb);
+    if (!hyh::ok()) { return 0.; }
     for (int32_t i = 0; i < M; i += block) { const int32_t rows = std::min(M - i, block);
       for (int32_t j = 0; j < N; j += block) { const int32_t cols = std::min(N - j, block);
         const void* src = transA ? at(A, (int64_t)j + (int64_t)i * lda, Atype) : at(A, (int64_t)i + (int64_t)j * lda, Atype);
@@ -119,9 +129,11 @@ double check_norm(const hyacinHandle_t* h, char opA, int32_t M, int32_t N, int32
   } else {
     rank = std::min(rank, N);
     hyh::Scratch Q(h, (size_t)N * rank * eb), work(h, (size_t)rank * 16 + 64);
+    if (!hyh::ok()) { return 0.; }
     HYH_KERNEL(hykMatcopy(s, 'A', N, rank, Atype, V, ldv, wide, Q.p, N));
     HYH_KERNEL(hykOrthonormalize(s, Complex, N, rank, Q.as<double>(), N, work.as<double>()));
     hyh::Scratch matA(h, (size_t)block * N * eb), matU(h, (size_t)block * rank * eb);
+    if (!hyh::ok()) { return 0.; }
     for (int32_t i = 0; i < M; i += block) { const int32_t rows = std::min(M - i, block);
       const void* src = transA ? at(A, (int64_t)i * lda, Atype) : at(A, (int64_t)i, Atype);
       HYH_KERNEL(hykMatcopy(s, mode, rows, N, Atype, src, lda, wide, matA.p, rows));
@@ -131,27 +143,31 @@ double check_norm(const hyacinHandle_t* h, char opA, int32_t M, int32_t N, int32
     }
   }
   double err = 0.; HYH_CHECK(hipMemcpyAsync(&err, acc.p, sizeof(double), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
-  return err;
+  return hyh::ok() ? err : 0.;
 }
 
 }  // namespace
 
 extern "C" int32_t hyacinInterpolateFit(const hyacinHandle_t* handle, double eps, char opA, int32_t M, int32_t N, int32_t K, const void* A, int32_t lda, int32_t* jpvt, void* V, int32_t ldv, int64_t globalM, hyacinPrecision_t ComputeType) {
+  hyh::ApiScope scope;
   if ((int)ComputeType < 0 || (int)ComputeType > HYACIN_F16_COMPLEX) { return 0; }
   return interp_fit(handle, eps, opA, M, N, K, (int)ComputeType, A, lda, jpvt, V, ldv, globalM <= 0 ? (int64_t)M : globalM);
 }
 
 extern "C" int32_t hyacinTsvdFit(const hyacinHandle_t* handle, double eps, char opA, int32_t M, int32_t N, int32_t K, const void* A, int32_t lda, void* S, void* V, int32_t ldv, int64_t globalM, hyacinPrecision_t ComputeType) {
+  hyh::ApiScope scope;
   if ((int)ComputeType < 0 || (int)ComputeType > HYACIN_F16_COMPLEX) { return 0; }
   return svd_fit(handle, eps, opA, M, N, K, (int)ComputeType, A, lda, S, V, ldv, globalM <= 0 ? (int64_t)M : globalM);
 }
 
 extern "C" int32_t hyacinTsvdFitSegmentN(const hyacinHandle_t* handle, double eps, char opA, int32_t M, int32_t N, int32_t K, const void* A, int32_t lda, void* S, void* V, int32_t ldv, int64_t globalM, hyacinPrecision_t ComputeType) {
+  hyh::ApiScope scope;
   if ((int)ComputeType < 0 || (int)ComputeType > HYACIN_F16_COMPLEX) { return 0; }
   return svd_fit_segmented(handle, eps, opA, M, N, K, (int)ComputeType, A, lda, S, V, ldv, globalM <= 0 ? (int64_t)M : globalM);
 }
 
 extern "C" double hyacinCheckNorm(const hyacinHandle_t* handle, char opA, int32_t M, int32_t N, const void* A, int32_t lda, int32_t rank, const void* V, int32_t ldv, hyacinPrecision_t ComputeType) {
+  hyh::ApiScope scope;
   if ((int)ComputeType < 0 || (int)ComputeType > HYACIN_F16_COMPLEX) { return 0.; }
   return check_norm(handle, opA, M, N, rank, (int)ComputeType, V, ldv, A, lda);
 }

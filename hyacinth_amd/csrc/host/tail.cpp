@@ -31,6 +31,7 @@ struct Factor {
       Rt(h, (size_t)N * (size_t)std::min(N, Kmax + 1) * (size_t)hyh::elem_bytes(factor_type(Gtype))),
       work(h, hykPotrfpWorkspaceBytes(N, factor_type(Gtype))) {
     type = factor_type(Gtype); ldr = std::min(N, Kmax + 1); rtBytes = (size_t)N * ldr * hyh::elem_bytes(type); G = Gin; ldg = ldgIn;
+    if (!hyh::ok()) { return; }
     if (widened.p) { HYH_KERNEL(hykMatcopy(h->hipStream, 'A', N, N, Gtype, Gin, ldgIn, HYACIN_F64 + (Gtype & 1), widened.p, N)); G = widened.p; ldg = N; }
     HYH_KERNEL(hykGramWorkspaceClear(h->hipStream, Rt.p, rtBytes));
   }
@@ -39,12 +40,15 @@ struct Factor {
 const char* type_tag(int t) { switch (t) { case HYACIN_F64: return "FP64"; case HYACIN_F64_COMPLEX: return "FP64-COMPLEX"; case HYACIN_DD: return "FP128-DD"; default: return "FP128-DD-COMPLEX"; } }
 
 int32_t run_potrfp(const hyacinHandle_t* h, Factor& f, double eps, int32_t K, int32_t N, int32_t* jpiv) {
-  int32_t* word = (int32_t*)h->pinnedWorkspace; *word = 0;
+  int32_t* word = (int32_t*)h->pinnedWorkspace; if (!word) { hyh::fail(-1, "pivoted Cholesky", "the handle has no pinned word (hyacinCreate not called?)", __FILE__, __LINE__); }
+  if (!hyh::ok()) { return 0; }
+  *word = 0;
   HYH_KERNEL(hykPotrfp(h->hipStream, h->DeviceSMs, eps, K, N, f.type, f.G, f.ldg, f.Rt.p, f.ldr, jpiv, f.work.p, word));
   HYH_CHECK(hipStreamSynchronize(h->hipStream));
+  if (!hyh::ok()) { return 0; }
   int32_t rank = *word;
-  if (rank < 0) {   /* the workgroups lost each other (a wait inside the kernel gave up): report no basis rather than a wrong one */
-    if (h->logger) { std::fprintf((FILE*)h->logger, "POTRFP-%s [N=%d] gave up waiting for a workgroup\n", type_tag(f.type), N); }
+  if (rank < 0) {   /* the workgroups lost each other (a bounded wait inside the kernel gave up): no basis rather than a wrong one */
+    hyh::fail(-5, "pivoted Cholesky", "a workgroup gave up waiting for the others; no factor was produced", __FILE__, __LINE__);
     return 0;
   }
   if (h->logger) { std::fprintf((FILE*)h->logger, "POTRFP-%s [eps=%.1le] [N=%d] [K=%d] [Cholesky-rank=%d]\n", type_tag(f.type), eps, N, K, rank); }
@@ -54,6 +58,7 @@ int32_t run_potrfp(const hyacinHandle_t* h, Factor& f, double eps, int32_t K, in
 }  // namespace
 
 extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t N, int32_t K, hyacinPrecision_t Atype, void* X, int32_t ldx, void* S, hyacinPrecision_t Gtype, void* G, int32_t ldg) {
+  hyh::ApiScope scope;
   if (N <= 0) { return 0; }
   K = K <= 0 ? N : std::min(N, K);
   if ((int)Atype < 0 || (int)Atype > HYACIN_F16_COMPLEX || ((int)Atype & 1) != ((int)Gtype & 1)) { return 0; }
@@ -68,9 +73,10 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
   int32_t rank;
   { Factor f(handle, N, N, (int)Gtype, G, ldg);
     rank = run_potrfp(handle, f, lrqr ? eps : 0., N, N, jpiv.as<int32_t>());
-    if (rank <= 0) { return rank; }
+    if (rank <= 0 || !hyh::ok()) { return 0; }
     /* B = (R P^T)^H, N x rank, FP64 */
     hyh::Scratch B(handle, (size_t)N * rank * 8 * (1 + Complex)), sigma(handle, sizeof(double) * (size_t)rank), counter(handle, 64), carry(handle, hykJacobiCarryBytes(rank));
+    if (!hyh::ok()) { return 0; }
     HYH_KERNEL(hykFactorToB(s, N, rank, f.type, f.Rt.p, f.ldr, B.as<double>()));
     const int32_t maxSweeps = sweeps > 0 ? 5 * sweeps : 30; int32_t used = 0;
     /* A pair is rotated while its cosine exceeds the storage precision, but never below sqrt(N) FP64 roundings: that is
@@ -84,12 +90,14 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
       HYH_KERNEL(hykJacobiSweepCarry(s, Complex, N, rank, B.as<double>(), rotateAbove, counter.as<int32_t>(), carry.as<double>())); ++used;
       struct { int32_t rotations, pad; double cosine2; } seen = { 0, 0, 0. };
       HYH_CHECK(hipMemcpyAsync(&seen, counter.p, sizeof(seen), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
+      if (!hyh::ok()) { return 0; }
       if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: %d rotations, largest cosine %.2le\n", used, seen.rotations, std::sqrt(seen.cosine2)); }
       if (hyh::jacobi_sweeps_done(seen.rotations, seen.cosine2, lastCosine2, rotateAbove)) { break; }
       lastCosine2 = seen.cosine2;
     }
     HYH_KERNEL(hykColumnNorms(s, Complex, N, rank, B.as<double>(), sigma.as<double>()));
     std::vector<double> sig((size_t)rank); HYH_CHECK(hipMemcpyAsync(sig.data(), sigma.p, sizeof(double) * (size_t)rank, hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
+    if (!hyh::ok()) { return 0; }
     std::vector<int32_t> order((size_t)rank); std::iota(order.begin(), order.end(), 0);
     std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return sig[a] > sig[b]; });
     /* rank cut (reference: find_srank_kernel, src/gram_evd.cu:44-70): keep i < K while sum_{j>=i} sigma_j^2 > eps^2 sum_j sigma_j^2 */
@@ -98,17 +106,20 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
     for (int32_t i = 0; i < K; ++i) { if (i < rank && resid < suffix[i]) { Sout[i] = sig[order[i]]; ++kept; } }
     const int32_t svdRank = kept; rank = std::min(rank, kept);
     hyh::Scratch dS(handle, sizeof(double) * (size_t)K), dOrder(handle, sizeof(int32_t) * (size_t)std::max(1, rank));
+    if (!hyh::ok()) { return 0; }
     HYH_CHECK(hipMemcpyAsync(dS.p, Sout.data(), sizeof(double) * (size_t)K, hipMemcpyHostToDevice, s));
     if (rank > 0) { HYH_CHECK(hipMemcpyAsync(dOrder.p, order.data(), sizeof(int32_t) * (size_t)rank, hipMemcpyHostToDevice, s)); }
     HYH_KERNEL(hykValuesOut(s, K, (int32_t)Atype, dS.as<double>(), S));
     if (rank > 0) { HYH_KERNEL(hykBasisOut(s, N, rank, (int32_t)Atype, B.as<double>(), sigma.as<double>(), dOrder.as<int32_t>(), X, ldx)); }
     HYH_CHECK(hipStreamSynchronize(s));   /* Sout / order are host temporaries */
+    if (!hyh::ok()) { return 0; }
     if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ-%s [eps=%.1le] [M=%d] [N=%d] [K=%d] [sweeps=%d] [SVD-rank=%d]\n", Complex ? "FP64-COMPLEX" : "FP64", eps, N, rank, K, used, svdRank); }
   }
-  return rank;
+  return hyh::ok() ? rank : 0;
 }
 
 extern "C" int32_t hyacinXGinterp(const hyacinHandle_t* handle, double eps, int32_t N, int32_t K, hyacinPrecision_t Atype, void* X, int32_t ldx, int32_t* jpiv, hyacinPrecision_t Gtype, void* G, int32_t ldg) {
+  hyh::ApiScope scope;
   if (N <= 0) { return 0; }
   K = K <= 0 ? N : std::min(N, K);
   if ((int)Atype < 0 || (int)Atype > HYACIN_F16_COMPLEX || ((int)Atype & 1) != ((int)Gtype & 1)) { return 0; }
@@ -117,11 +128,12 @@ extern "C" int32_t hyacinXGinterp(const hyacinHandle_t* handle, double eps, int3
   const int Complex = (int)Atype & 1; eps = std::min(std::max(std::fabs(eps), storage_eps((int)Atype)), 1.);
   Factor f(handle, N, K, (int)Gtype, G, ldg);
   const int32_t rank = run_potrfp(handle, f, eps, K, N, jpiv);
-  if (rank <= 0) { return rank; }
-  if (rank >= N) { HYH_KERNEL(hykInterpOut(s, N, N, (int32_t)Atype, jpiv, nullptr, X, ldx)); return N; }
+  if (rank <= 0 || !hyh::ok()) { return 0; }
+  if (rank >= N) { HYH_KERNEL(hykInterpOut(s, N, N, (int32_t)Atype, jpiv, nullptr, X, ldx)); return hyh::ok() ? N : 0; }
   hyh::Scratch Rp(handle, (size_t)rank * rank * 8 * (1 + Complex)), Tt(handle, (size_t)rank * (N - rank) * 8 * (1 + Complex));
+  if (!hyh::ok()) { return 0; }
   HYH_KERNEL(hykInterpSolve(s, N, rank, f.type, f.Rt.p, f.ldr, jpiv, Rp.as<double>(), Tt.as<double>()));
   HYH_KERNEL(hykInterpOut(s, N, rank, (int32_t)Atype, jpiv, Tt.as<double>(), X, ldx));
   if (handle->logger) { std::fprintf((FILE*)handle->logger, "TRSM-LEFT-%s [M=%d] [N=%d]\n", Complex ? "FP64-COMPLEX" : "FP64", rank, N - rank); }
-  return rank;
+  return hyh::ok() ? rank : 0;
 }

@@ -879,7 +879,7 @@ extern "C" int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t
 }
 
 /* one sweep = every pair of the r columns of B (N x r, FP64, complex interleaved) once; rotations counts the rotations applied */
-static int g_jacobiVariant = 0;   /* 0: Gram-space rounds, 8-column blocks for real factors where they fit (default); 1: the step kernel everywhere; 2: Gram-space rounds, 4-column blocks */
+static thread_local int g_jacobiVariant = 0;   /* 0: Gram-space rounds, 8-column blocks for real factors where they fit (default); 1: the step kernel everywhere; 2: Gram-space rounds, 4-column blocks */
 
 template <int ROWS, int BC, int THREADS = T_THREADS, int PASSES = 1>
 static int gram_sweep(hipStream_t stream, int32_t N, int32_t r, double* B, double tol, int32_t* rotations, double* carry) {
@@ -1035,7 +1035,7 @@ extern "C" int hykOrthonormalize(hipStream_t stream, int32_t Complex, int32_t N,
   if (ldv != N) { return -1; }
   int32_t* counter = reinterpret_cast<int32_t*>(work); double* sigma = work + 8;
   for (int sweep = 0; sweep < 40 && r > 1; ++sweep) {
-    if (hipMemsetAsync(counter, 0, 64, stream) != hipSuccess) { return -3; }
+    if (hykGramWorkspaceClear(stream, counter, 64) != 0) { return -3; }
     if (hykJacobiSweep(stream, Complex, N, r, V, 2.220446049250313e-16 * sqrt((double)N), counter) != 0) { return -3; }
     struct { int32_t rotations, pad; double cosine2; } seen = { 0, 0, 0. }; const double level = 8. * 2.220446049250313e-16 * sqrt((double)N);
     if (hipMemcpyAsync(&seen, counter, sizeof(seen), hipMemcpyDeviceToHost, stream) != hipSuccess || hipStreamSynchronize(stream) != hipSuccess) { return -3; }

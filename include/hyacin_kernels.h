@@ -50,13 +50,14 @@ int hykGramCrt(hipStream_t stream, int32_t Complex, int32_t N, int32_t orderA, c
 int hykGramLimbs(hipStream_t stream, int32_t Complex, int32_t N, int32_t orderA, const int8_t* panels, int64_t ldb, int32_t K, int32_t beta, int32_t orderC, uint64_t* C, void* workspace);
 
 /* Measurement hooks (no counterpart in the reference): time every launch of the contraction kernel with HIP events on
- * its stream.  hykGramProfile(1) starts a fresh record, hykGramProfile(0) stops; Read waits for the recorded launches. */
+ * its stream.  hykGramProfile(1) starts a fresh record, hykGramProfile(0) stops; Read waits for the recorded launches.
+ * The record belongs to the calling host thread: it times that thread's launches only. */
 int hykGramProfile(int32_t enable);
 int hykGramProfileRead(double* totalMs, int32_t* launches);
 
 /* Variant of the contraction kernel (tuning knob): 0 = operand slabs loaded straight from global memory into a ring of
  * LDS units with 128-byte rows (default); 2 = the same with 64-byte rows and four stages; 64 / 128 = staged through
- * registers with that many K bytes per LDS stage. */
+ * registers with that many K bytes per LDS stage.  The setting is per host thread. */
 int hykGramSetSlab(int32_t bk);
 
 /* Measurement hook (no counterpart in the reference): int8 tera-ops per second that a register-only loop of
@@ -106,7 +107,7 @@ int hykJacobiSweepCarry(hipStream_t stream, int32_t Complex, int32_t N, int32_t 
  * one wavefront; real factors in blocks of 8 columns, complex ones in blocks of 4, the rows in two halves where N > 2048;
  * 1 one reduction and barrier per step; 2 as 0 with the narrower blocks that hold all rows at once (4 columns for real
  * factors, 2 for complex ones above 2048 rows).  All rotate by the same rule, and for equal block sizes they visit the
- * pairs in the same order; kept selectable so that tests cover every kernel.  Process-wide, not thread-safe. */
+ * pairs in the same order; kept selectable so that tests cover every kernel.  The setting is per host thread. */
 int hykJacobiSetVariant(int32_t variant);
 int hykColumnNorms(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, const double* B, double* sigma);
 int hykBasisOut(hipStream_t stream, int32_t N, int32_t rank, int32_t Atype, const double* B, const double* sigma, const int32_t* order, void* X, int64_t ldx);
@@ -141,6 +142,16 @@ int hykGemm(hipStream_t stream, char opA, char opB, int32_t M, int32_t N, int32_
  * Jacobi rotations, then column normalisation).  Replaces the Q factor of cuSOLVER geqrf + orgqr/ungqr,
  * src/lra.cpp:176-191: the same subspace, a different basis of it.  work: r * sizeof(element) + 64 bytes. */
 int hykOrthonormalize(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* V, int64_t ldv, double* work);
+
+/* Status of the last outermost hyacin.h call made on the calling thread: 0, or the code of the first failure inside it
+ * (a HIP error number, a negative kernel-layer return value, -4 a scratch allocation that failed, -5 a pivoted Cholesky
+ * whose workgroups lost each other).  A failed call has launched nothing after the failure and returned 0 / written no
+ * result.  No counterpart in the reference, which drops every status in release builds (include/internal.hpp:232-236). */
+int hykLastStatus(void);
+
+/* Test hook (no counterpart in the reference): the nth scratch acquisition from now on, in any thread, fails as if the
+ * memory pool were exhausted; 0 switches the hook off. */
+int hykTestFailAllocation(int32_t nth);
 
 #ifdef __cplusplus
 }
