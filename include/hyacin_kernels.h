@@ -145,8 +145,8 @@ int hykOrthonormalize(hipStream_t stream, int32_t Complex, int32_t N, int32_t r,
 
 /* Status of the last outermost hyacin.h call made on the calling thread: 0, or the code of the first failure inside it
  * (a HIP error number, a negative kernel-layer return value, -4 a scratch allocation that failed, -5 a pivoted Cholesky
- * whose workgroups lost each other).  A failed call has launched nothing after the failure and returned 0 / written no
- * result.  No counterpart in the reference, which drops every status in release builds (include/internal.hpp:232-236). */
+ * whose workgroups lost each other).  A failed call has launched nothing after the failure, returned 0 and written
+ * neither S nor V (the pivot vector of an interpolation may already hold the pivots).  No counterpart in the reference, which drops every status in release builds (include/internal.hpp:232-236). */
 int hykLastStatus(void);
 
 /* Test hook (no counterpart in the reference): the nth scratch acquisition from now on, in any thread, fails as if the
