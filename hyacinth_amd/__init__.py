@@ -33,7 +33,8 @@ KERNEL_SYMBOLS = [
     "hykGramWorkspaceBytes", "hykGramWorkspaceClear", "hykGramCrt", "hykGramLimbs", "hykGramSetSlab",
     "hykGramProfile", "hykGramProfileRead", "hykMfmaCeiling", "hykGramRange", "hykDequantize", "hykPotrfpWorkspaceBytes", "hykPotrfp", "hykPotrfpLeftLooking", "hykPotrfpStaticMaxN", "hykPotrfpStatic", "hykFactorToB", "hykJacobiSweep", "hykJacobiSweepCarry", "hykJacobiCarryBytes", "hykJacobiSetVariant",
     "hykColumnNorms", "hykBasisOut", "hykValuesOut", "hykInterpSolve", "hykInterpOut", "hykMatcopy",
-    "hykSumSquares", "hykMatmulCf16", "hykGemm", "hykOrthonormalize", "hykLastStatus", "hykTestFailAllocation",
+    "hykSumSquares", "hykMatmulCf16", "hykGemm", "hykOrthonormalize", "hykLastStatus", "hykTestFailAllocation", "hykColumnExponentsOp", "hykQuantizeLimbsOp", "hykQuantizeCrtOp",
+    "hykQuantizeScaleBatchOp", "hykHerkBatchOp", "hykLastHerkPlan",
 ]
 
 
@@ -49,6 +50,12 @@ class Handle(C.Structure):
         ("hipStream", C.c_void_p), ("rocblasHandle", C.c_void_p), ("solverHandle", C.c_void_p), ("mempool", C.c_void_p),
         ("pinnedWorkspace", C.c_void_p), ("timer", C.c_void_p), ("logger", C.c_void_p),
     ]
+
+
+class HerkPlan(C.Structure):
+    """hykHerkPlan (include/hyacin_kernels.h)."""
+    _fields_ = [("algorithm", C.c_int32), ("order", C.c_int32), ("chunkRows", C.c_int32), ("gramCalls", C.c_int32),
+                ("quantizeCalls", C.c_int32), ("reserved", C.c_int32), ("rows", C.c_int64), ("int8Ops", C.c_double)]
 
 
 _lib = None
@@ -106,6 +113,12 @@ def lib():
         L.hykMatmulCf16.argtypes = [vp, ch, i32, i32, i32, vp, i64, vp, i64, vp, i64]
         L.hykSumSquares.argtypes = [vp, i64, i64, vp, i64, vp]
         L.hykOrthonormalize.argtypes = [vp, i32, i32, i32, vp, i64, vp]
+        L.hykColumnExponentsOp.argtypes = [vp, ch, i32, i32, i32, i32, i32, vp, i64, i32, vp]
+        L.hykQuantizeLimbsOp.argtypes = [vp, ch, i32, i32, i32, i32, vp, i64, vp, vp, i64]
+        L.hykQuantizeCrtOp.argtypes = [vp, ch, i32, i32, i32, i32, vp, i64, vp, vp, i64, i32]
+        L.hykQuantizeScaleBatchOp.argtypes = [HP, ch, i32, i32, i32, i32, i32, vp, i64, i32, vp]; L.hykQuantizeScaleBatchOp.restype = None
+        L.hykHerkBatchOp.argtypes = [HP, ch, i32, i32, i32, i32, i32, vp, i64, i32, vp, i32, i32, vp]; L.hykHerkBatchOp.restype = None
+        L.hykLastHerkPlan.argtypes = [C.POINTER(HerkPlan)]
         L.hykLastStatus.argtypes = []
         L.hykTestFailAllocation.argtypes = [i32]
         L.hykFactorToB.argtypes = [vp, i32, i32, i32, vp, i32, vp]

@@ -66,6 +66,54 @@ __global__ __launch_bounds__(EXP_THREADS) void column_exponent_kernel(int32_t se
   }
 }
 
+/* A stored as its transpose: the N x M matrix S with op(A)[k, j] = S[j + k lda] (a conjugate changes no magnitude), rows of
+ * op(A) contiguous in memory.  A thread owns 16 bytes' worth of adjacent columns and walks down EXP_T_ROWS rows of one row
+ * slice, so every load instruction of a wavefront covers 1 KB of one stored row; the per-chunk results meet in mexp (filled
+ * with INT_MAX before) through an integer minimum: u - e is smallest where the magnitude is largest.  Replaces the
+ * transposing copy of src/lra.cpp:63-69 followed by src/fp_exponent.cu:23-51. */
+constexpr int EXP_T_ROWS = 64;
+template <typename SCALAR>
+__global__ __launch_bounds__(EXP_THREADS) void column_exponent_transposed_kernel(int32_t segM, int32_t lastM, int32_t comps, const SCALAR* __restrict__ S, int64_t lda_scalars, int32_t u, int32_t N, int32_t* __restrict__ mexp) {
+  constexpr int VEC = 16 / sizeof(SCALAR); constexpr SCALAR ABS = (SCALAR)(~(SCALAR)0) >> 1;
+  const int32_t b = blockIdx.y; const int64_t rows = (b + 1 == (int32_t)gridDim.y) ? lastM : segM;
+  const int64_t r0 = (int64_t)blockIdx.x * EXP_T_ROWS; if (r0 >= rows) { return; }
+  const int64_t r1 = r0 + EXP_T_ROWS < rows ? r0 + EXP_T_ROWS : rows, width = (int64_t)N * comps;
+  const int64_t c0 = ((int64_t)blockIdx.z * EXP_THREADS + threadIdx.x) * VEC; if (c0 >= width) { return; }
+  const SCALAR* base = S + ((int64_t)b * segM + r0) * lda_scalars + c0;
+  SCALAR mx[VEC];
+  #pragma unroll
+  for (int i = 0; i < VEC; ++i) { mx[i] = 0; }
+  const bool vec = c0 + VEC <= width && (((uintptr_t)base) & 15u) == 0 && ((lda_scalars * (int64_t)sizeof(SCALAR)) & 15) == 0;
+  if (vec) {
+    #pragma unroll 8
+    for (int64_t r = 0; r < r1 - r0; ++r) {
+      const u32x4 w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(base + r * lda_scalars));
+      SCALAR v[VEC];
+      if constexpr (sizeof(SCALAR) == 8) { v[0] = ((uint64_t)w.y << 32) | w.x; v[1] = ((uint64_t)w.w << 32) | w.z; }
+      else if constexpr (sizeof(SCALAR) == 4) { v[0] = w.x; v[1] = w.y; v[2] = w.z; v[3] = w.w; }
+      else { const uint32_t ws[4] = { w.x, w.y, w.z, w.w };
+        #pragma unroll
+        for (int t = 0; t < 4; ++t) { v[2 * t] = (SCALAR)(ws[t] & 0xffffu); v[2 * t + 1] = (SCALAR)(ws[t] >> 16); } }
+      #pragma unroll
+      for (int i = 0; i < VEC; ++i) { const SCALAR a = v[i] & ABS; mx[i] = a > mx[i] ? a : mx[i]; }
+    }
+  } else {
+    for (int64_t r = 0; r < r1 - r0; ++r) {
+      #pragma unroll
+      for (int i = 0; i < VEC; ++i) { if (c0 + i < width) { const SCALAR a = base[r * lda_scalars + i] & ABS; mx[i] = a > mx[i] ? a : mx[i]; } }
+    }
+  }
+  #pragma unroll
+  for (int i = 0; i < VEC; i += 1) {
+    if (c0 + i >= width) { break; }
+    if (comps == 2 && (i & 1)) { continue; }          /* the pair (re, im) is judged at its real part's turn */
+    SCALAR m = mx[i]; if (comps == 2 && i + 1 < VEC) { m = mx[i + 1] > m ? mx[i + 1] : m; }
+    int32_t e;
+    if constexpr (sizeof(SCALAR) == 8) { e = hyk::frexp_exp_f64(m); } else if constexpr (sizeof(SCALAR) == 4) { e = hyk::frexp_exp_f32(m); } else { e = hyk::frexp_exp_f16(m); }
+    if (e != HYK_INT_MAX) { atomicMin(&mexp[(int64_t)b * N + (c0 + i) / comps], u - e); }
+  }
+}
+
 __global__ void exponent_fill_kernel(int32_t N, int32_t* __restrict__ vexp) { int32_t i = blockIdx.x * blockDim.x + threadIdx.x; if (i < N) { vexp[i] = HYK_INT_MAX; } }
 
 __global__ void exponent_min_kernel(int32_t N, int32_t batches, int32_t* __restrict__ vexp) {
@@ -114,19 +162,36 @@ __global__ __launch_bounds__(EXP_THREADS) void gram_range_kernel(int32_t N, int3
 
 }  // namespace
 
-extern "C" int hykColumnExponents(hipStream_t stream, int32_t batches, int32_t segM, int32_t lastM, int32_t N, int32_t Atype, const void* A, int64_t lda, int32_t u, int32_t* vexp) {
+extern "C" int hykColumnExponentsOp(hipStream_t stream, char opA, int32_t batches, int32_t segM, int32_t lastM, int32_t N, int32_t Atype, const void* A, int64_t lda, int32_t u, int32_t* vexp) {
   if (N <= 0) { return 0; }
   if (Atype < HYK_F64 || Atype > HYK_F16C) { return -1; }
   if (batches <= 0 || u < 0) { exponent_fill_kernel<<<(N + 255) / 256, 256, 0, stream>>>(N, vexp); return 0; }
-  if (N > 65535 || segM <= 0 || lastM <= 0 || lastM > segM) { return -2; }
-  const int32_t comps = 1 + (Atype & 1); dim3 grid((uint32_t)batches, (uint32_t)N);
-  switch (Atype & ~1) {
-    case HYK_F64: column_exponent_kernel<uint64_t><<<grid, EXP_THREADS, 0, stream>>>(segM, lastM, comps, (const uint64_t*)A, lda * comps, u, N, &vexp[N]); break;
-    case HYK_F32: column_exponent_kernel<uint32_t><<<grid, EXP_THREADS, 0, stream>>>(segM, lastM, comps, (const uint32_t*)A, lda * comps, u, N, &vexp[N]); break;
-    default: column_exponent_kernel<uint16_t><<<grid, EXP_THREADS, 0, stream>>>(segM, lastM, comps, (const uint16_t*)A, lda * comps, u, N, &vexp[N]); break;
+  if (N > 65535 || batches > 65535 || segM <= 0 || lastM <= 0 || lastM > segM) { return -2; }
+  const int32_t comps = 1 + (Atype & 1);
+  const bool transposed = opA == 'T' || opA == 't' || opA == 'C' || opA == 'c';
+  if (!transposed) {
+    dim3 grid((uint32_t)batches, (uint32_t)N);
+    switch (Atype & ~1) {
+      case HYK_F64: column_exponent_kernel<uint64_t><<<grid, EXP_THREADS, 0, stream>>>(segM, lastM, comps, (const uint64_t*)A, lda * comps, u, N, &vexp[N]); break;
+      case HYK_F32: column_exponent_kernel<uint32_t><<<grid, EXP_THREADS, 0, stream>>>(segM, lastM, comps, (const uint32_t*)A, lda * comps, u, N, &vexp[N]); break;
+      default: column_exponent_kernel<uint16_t><<<grid, EXP_THREADS, 0, stream>>>(segM, lastM, comps, (const uint16_t*)A, lda * comps, u, N, &vexp[N]); break;
+    }
+  } else {
+    const int64_t cells = (int64_t)batches * N; exponent_fill_kernel<<<(uint32_t)((cells + 255) / 256), 256, 0, stream>>>((int32_t)cells, &vexp[N]);
+    const int scalarBytes = (Atype & ~1) == HYK_F64 ? 8 : ((Atype & ~1) == HYK_F32 ? 4 : 2); const int64_t perBlock = (int64_t)EXP_THREADS * (16 / scalarBytes);
+    dim3 grid((uint32_t)((segM + EXP_T_ROWS - 1) / EXP_T_ROWS), (uint32_t)batches, (uint32_t)(((int64_t)N * comps + perBlock - 1) / perBlock));
+    switch (Atype & ~1) {
+      case HYK_F64: column_exponent_transposed_kernel<uint64_t><<<grid, EXP_THREADS, 0, stream>>>(segM, lastM, comps, (const uint64_t*)A, lda * comps, u, N, &vexp[N]); break;
+      case HYK_F32: column_exponent_transposed_kernel<uint32_t><<<grid, EXP_THREADS, 0, stream>>>(segM, lastM, comps, (const uint32_t*)A, lda * comps, u, N, &vexp[N]); break;
+      default: column_exponent_transposed_kernel<uint16_t><<<grid, EXP_THREADS, 0, stream>>>(segM, lastM, comps, (const uint16_t*)A, lda * comps, u, N, &vexp[N]); break;
+    }
   }
   exponent_min_kernel<<<(N + 255) / 256, 256, 0, stream>>>(N, batches, vexp);
-  return 0;
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+extern "C" int hykColumnExponents(hipStream_t stream, int32_t batches, int32_t segM, int32_t lastM, int32_t N, int32_t Atype, const void* A, int64_t lda, int32_t u, int32_t* vexp) {
+  return hykColumnExponentsOp(stream, 'N', batches, segM, lastM, N, Atype, A, lda, u, vexp);
 }
 
 extern "C" int hykSliceRange(hipStream_t stream, int32_t batches, int32_t N, int32_t u, const int32_t* vexp, int32_t* segU) {

@@ -57,6 +57,10 @@ void timer_mark(const hyacinHandle_t* h, Segment s);
 struct GramPlan { char alg; int32_t order; int32_t second; };  /* second: limb capacity in bits ('L') or rows per CRT chunk ('C') */
 GramPlan gram_algorithm(char alg, int32_t K, int32_t u, int32_t Complex, int32_t segmentK, double batchPenalty);
 
+/* the Gram stages with the storage order of A as an argument ('N' column-major M x N; 'T' / 'C' the stored N x M transpose) */
+void quantize_scale_batch(const hyacinHandle_t* h, char op, int32_t batches, int32_t segM, int32_t lastM, int32_t N, int Atype, const void* A, int64_t lda, int32_t uA, int32_t* vexp);
+void herk_batch(const hyacinHandle_t* h, char op, int32_t batches, int32_t segM, int32_t lastM, int32_t N, int Atype, const void* A, int64_t lda, int32_t u, const int32_t* vexp, int32_t beta, int32_t orderC, uint64_t* C);
+
 inline int32_t round_up(int32_t v, int32_t a) { return (v + a - 1) / a * a; }
 
 }  // namespace hyh

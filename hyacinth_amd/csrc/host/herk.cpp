@@ -61,18 +61,23 @@ extern "C" void hyacinXherkBatchInit(const hyacinHandle_t* handle, double eps, u
   if (lPanels) { *lPanels = 0 <= uc ? (63 + std::max(0, 2 * (uc + Complex)) + (int32_t)std::ceil(std::log2((double)Mp))) / 63 : 0; }
 }
 
+void hyh::quantize_scale_batch(const hyacinHandle_t* handle, char op, int32_t batches, int32_t segM, int32_t lastM, int32_t N, int Atype, const void* A, int64_t lda, int32_t uA, int32_t* vexp) {
+  if (N <= 0 || Atype > HYACIN_F16_COMPLEX) { return; }
+  hyh::timer_mark(handle, hyh::Segment::dist_kernel);
+  HYH_KERNEL(hykColumnExponentsOp(handle->hipStream, op, batches, segM, lastM, N, (int32_t)Atype, A, lda, uA, vexp));
+}
+
 extern "C" void hyacinXquantizeScaleBatch(const hyacinHandle_t* handle, int32_t batches, int32_t segM, int32_t lastM, int32_t N, hyacinPrecision_t Atype, const void* A, int32_t lda, int32_t uA, int32_t* vexp) {
   hyh::ApiScope scope;
-  if (N <= 0 || (int)Atype > HYACIN_F16_COMPLEX) { return; }
-  hyh::timer_mark(handle, hyh::Segment::dist_kernel);
-  HYH_KERNEL(hykColumnExponents(handle->hipStream, batches, segM, lastM, N, (int32_t)Atype, A, lda, uA, vexp));
+  hyh::quantize_scale_batch(handle, 'N', batches, segM, lastM, N, (int)Atype, A, lda, uA, vexp);
 }
 
 namespace {
 
-struct Ctx { const hyacinHandle_t* h; hipStream_t s; int32_t N, Atype, Complex, u; const char* A; int64_t lda; const int32_t* vexp; int32_t beta, orderC; uint64_t* C; };
+/* op: 'N' A is column-major M x N; 'T' / 'C' A is the stored N x M (conjugate) transpose, op(A)[k, j] = (conj) A[j + k lda] */
+struct Ctx { const hyacinHandle_t* h; hipStream_t s; char op; int32_t N, Atype, Complex, u; const char* A; int64_t lda; const int32_t* vexp; int32_t beta, orderC; uint64_t* C; };
 
-const void* row_ptr(const Ctx& c, int64_t row) { return c.A + row * (int64_t)hyh::elem_bytes(c.Atype); }
+const void* row_ptr(const Ctx& c, int64_t row) { return c.A + row * (c.op == 'N' ? 1 : c.lda) * (int64_t)hyh::elem_bytes(c.Atype); }
 
 int32_t crt_panels(int32_t order, int32_t Complex) { return Complex ? 2 * order + std::max(0, order - HYK_CRT_CPLX_SPLIT) : order; }
 
@@ -83,6 +88,17 @@ int64_t panel_ld(int64_t cap) { return cap + ((cap % 4096 == 0) ? 256 : 0); }
 
 /* a list of row runs [first, first + count) of A, quantized back to back into one compact panel set and contracted */
 struct Run { int64_t first; int32_t count; };
+
+/* what the last hyacinXherkBatch of this thread did (hykLastHerkPlan) */
+thread_local hykHerkPlan g_plan;
+void note_quantize() { ++g_plan.quantizeCalls; }
+void note_gram(const Ctx& c, char alg, int32_t order, int32_t chunkRows, int32_t rows) {
+  /* algorithmic int8 operations (2 per multiply-add, triangle only) of one contraction over `rows` rows */
+  const double M = rows, N = c.N; double ops;
+  if (alg == 'C') { ops = c.Complex ? std::min(order, HYK_CRT_CPLX_SPLIT) * 2. * M * N * N + std::max(order - HYK_CRT_CPLX_SPLIT, 0) * (M * N * (N + 1.) + 2. * M * N * N) : order * M * N * (N + 1.); }
+  else { ops = order * M * N * (N + 1.) + (double)order * (order - 1) * M * N * N + (c.Complex ? (double)order * order * 2. * M * N * N : 0.); }
+  g_plan.algorithm = alg; g_plan.order = order; g_plan.chunkRows = chunkRows; ++g_plan.gramCalls; g_plan.rows += rows; g_plan.int8Ops += ops;
+}
 
 void log_gemm(const Ctx& c, const char* kind, int32_t K, int32_t order) {
   if (c.h->logger) { std::fprintf((FILE*)c.h->logger, "I8I32-GEMM-%s [algo=TN,%s] [M=N=%d] [K=%d] [Order=%d]\n", c.Complex ? "COMPLEX" : "REAL", kind, (c.N + 63) & ~63, K, order); }
@@ -101,13 +117,13 @@ void limb_bucket(Ctx& c, const std::vector<Run>& runs, int32_t order) {
   auto flush = [&]() {
     if (filled <= 0) { return; } const int32_t K = hyh::round_up(filled, 128);
     HYH_KERNEL(hykZeroRows(c.s, W.as<int8_t>(), ld, (int64_t)c.N * order * groups, filled, K));
-    HYH_KERNEL(hykGramLimbs(c.s, c.Complex, c.N, order, W.as<int8_t>(), ld, K, c.beta, c.orderC, c.C, ws.p)); c.beta = 1; log_gemm(c, "limbs", K, order); filled = 0;
+    HYH_KERNEL(hykGramLimbs(c.s, c.Complex, c.N, order, W.as<int8_t>(), ld, K, c.beta, c.orderC, c.C, ws.p)); c.beta = 1; log_gemm(c, "limbs", K, order); note_gram(c, 'L', order, (int32_t)cap, filled); filled = 0;
   };
   for (const Run& r : runs) {
     int64_t first = r.first; int32_t left = r.count;
     while (left > 0) {
       const int32_t take = (int32_t)std::min<int64_t>(left, cap - filled);
-      HYH_KERNEL(hykQuantizeLimbs(c.s, take, c.N, order, c.Atype, row_ptr(c, first), c.lda, c.vexp, W.as<int8_t>() + filled, ld));
+      HYH_KERNEL(hykQuantizeLimbsOp(c.s, c.op, take, c.N, order, c.Atype, row_ptr(c, first), c.lda, c.vexp, W.as<int8_t>() + filled, ld)); note_quantize();
       filled += take; first += take; left -= take; if (filled == cap) { flush(); }
     }
   }
@@ -128,13 +144,13 @@ void crt_bucket(Ctx& c, const std::vector<Run>& runs, int32_t order, int32_t chu
   auto flush = [&]() {
     if (filled <= 0) { return; } const int32_t K = hyh::round_up(filled, 128);
     HYH_KERNEL(hykZeroRows(c.s, W.as<int8_t>(), ld, (int64_t)c.N * panels, filled, K));
-    HYH_KERNEL(hykGramCrt(c.s, c.Complex, c.N, order, W.as<int8_t>(), ld, K, c.beta, c.orderC, c.C, ws.p)); c.beta = 1; log_gemm(c, "crt", K, order); filled = 0;
+    HYH_KERNEL(hykGramCrt(c.s, c.Complex, c.N, order, W.as<int8_t>(), ld, K, c.beta, c.orderC, c.C, ws.p)); c.beta = 1; log_gemm(c, "crt", K, order); note_gram(c, 'C', order, (int32_t)cap, filled); filled = 0;
   };
   for (const Run& r : runs) {
     int64_t first = r.first; int32_t left = r.count;
     while (left > 0) {
       const int32_t take = (int32_t)std::min<int64_t>(left, cap - filled);
-      HYH_KERNEL(hykQuantizeCrt(c.s, take, c.N, order, c.Atype, row_ptr(c, first), c.lda, c.vexp, W.as<int8_t>() + filled, ld, maxBits));
+      HYH_KERNEL(hykQuantizeCrtOp(c.s, c.op, take, c.N, order, c.Atype, row_ptr(c, first), c.lda, c.vexp, W.as<int8_t>() + filled, ld, maxBits)); note_quantize();
       filled += take; first += take; left -= take; if (filled == cap) { flush(); }
     }
   }
@@ -195,13 +211,29 @@ void herk_sliced(Ctx& c, int32_t batches, int32_t segM, int32_t lastM) {
 
 }  // namespace
 
-extern "C" void hyacinXherkBatch(const hyacinHandle_t* handle, int32_t batches, int32_t segM, int32_t lastM, int32_t N, hyacinPrecision_t Atype, const void* A, int32_t lda, int32_t u, const int32_t* vexp, int32_t beta, int32_t orderC, uint64_t* C) {
-  hyh::ApiScope scope;
-  if (N <= 0 || orderC <= 0 || (int)Atype < 0 || (int)Atype > HYACIN_F16_COMPLEX) { return; }
+void hyh::herk_batch(const hyacinHandle_t* handle, char op, int32_t batches, int32_t segM, int32_t lastM, int32_t N, int Atype, const void* A, int64_t lda, int32_t u, const int32_t* vexp, int32_t beta, int32_t orderC, uint64_t* C) {
+  if (N <= 0 || orderC <= 0 || Atype < 0 || Atype > HYACIN_F16_COMPLEX) { return; }
   hyh::timer_mark(handle, hyh::Segment::dist_kernel);
-  Ctx c{ handle, handle->hipStream, N, (int32_t)Atype, (int32_t)Atype & 1, u, (const char*)A, lda, vexp, beta, orderC, C };
+  g_plan = hykHerkPlan{};
+  Ctx c{ handle, handle->hipStream, (op == 'T' || op == 'C') ? op : 'N', N, (int32_t)Atype, (int32_t)Atype & 1, u, (const char*)A, lda, vexp, beta, orderC, C };
   if (batches <= 1) { herk_single(c, lastM); } else { herk_sliced(c, batches, segM, lastM); }
 }
+
+extern "C" void hyacinXherkBatch(const hyacinHandle_t* handle, int32_t batches, int32_t segM, int32_t lastM, int32_t N, hyacinPrecision_t Atype, const void* A, int32_t lda, int32_t u, const int32_t* vexp, int32_t beta, int32_t orderC, uint64_t* C) {
+  hyh::ApiScope scope;
+  hyh::herk_batch(handle, 'N', batches, segM, lastM, N, (int)Atype, A, lda, u, vexp, beta, orderC, C);
+}
+
+/* the two stage functions above with the storage order of A as an argument (the reference transposes first, src/lra.cpp:63-69) */
+extern "C" void hykQuantizeScaleBatchOp(const void* handle, char opA, int32_t batches, int32_t segM, int32_t lastM, int32_t N, int32_t Atype, const void* A, int64_t lda, int32_t uA, int32_t* vexp) {
+  hyh::ApiScope scope; const char op = (opA == 'T' || opA == 't') ? 'T' : ((opA == 'C' || opA == 'c') ? 'C' : 'N');
+  hyh::quantize_scale_batch((const hyacinHandle_t*)handle, op, batches, segM, lastM, N, Atype, A, lda, uA, vexp);
+}
+extern "C" void hykHerkBatchOp(const void* handle, char opA, int32_t batches, int32_t segM, int32_t lastM, int32_t N, int32_t Atype, const void* A, int64_t lda, int32_t u, const int32_t* vexp, int32_t beta, int32_t orderC, uint64_t* C) {
+  hyh::ApiScope scope; const char op = (opA == 'T' || opA == 't') ? 'T' : ((opA == 'C' || opA == 'c') ? 'C' : 'N');
+  hyh::herk_batch((const hyacinHandle_t*)handle, op, batches, segM, lastM, N, Atype, A, lda, u, vexp, beta, orderC, C);
+}
+extern "C" int hykLastHerkPlan(hykHerkPlan* out) { if (!out) { return -1; } *out = g_plan; return 0; }
 
 extern "C" void hyacinXdequantizeInit(const hyacinHandle_t* handle, int32_t N, int32_t orderC, const uint64_t* C, const int32_t* vexp, hyacinPrecision_t Atype, hyacinPrecision_t* Gtype, int32_t* gElemBytes) {
   hyh::ApiScope scope;

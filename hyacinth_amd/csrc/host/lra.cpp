@@ -30,18 +30,11 @@ int32_t fit_common(const hyacinHandle_t* h, double eps, char opA, int32_t M, int
   hyacinXherkBatchInit(h, eps, (uint64_t)globalM, N, (hyacinPrecision_t)Atype, &u, &cPanels, &lPanels, &strideC);
   hyh::Scratch vexp(h, sizeof(int32_t) * (size_t)(sl.batches + 1) * (size_t)N), C(h, sizeof(uint64_t) * (size_t)cPanels * (size_t)std::max(1, lPanels) * (size_t)strideC);
   if (!hyh::ok()) { return 0; }
-  if (opA == 'T' || opA == 'C') {
-    hyh::Scratch AH(h, (size_t)M * (size_t)N * (size_t)hyh::elem_bytes(Atype));
-    if (!hyh::ok()) { return 0; }
-    HYH_KERNEL(hykMatcopy(s, opA, M, N, Atype, A, lda, Atype, AH.p, M));
-    hyacinXquantizeScaleBatch(h, sl.batches, sl.batchIter, sl.lastM, N, (hyacinPrecision_t)Atype, AH.p, M, u, vexp.as<int32_t>());
-    hyacinAllReduceVExp(h, (uint64_t)N, vexp.as<int32_t>());
-    hyacinXherkBatch(h, sl.batches, sl.batchIter, sl.lastM, N, (hyacinPrecision_t)Atype, AH.p, M, u, vexp.as<int32_t>(), 0, lPanels, C.as<uint64_t>());
-  } else {
-    hyacinXquantizeScaleBatch(h, sl.batches, sl.batchIter, sl.lastM, N, (hyacinPrecision_t)Atype, A, lda, u, vexp.as<int32_t>());
-    hyacinAllReduceVExp(h, (uint64_t)N, vexp.as<int32_t>());
-    hyacinXherkBatch(h, sl.batches, sl.batchIter, sl.lastM, N, (hyacinPrecision_t)Atype, A, lda, u, vexp.as<int32_t>(), 0, lPanels, C.as<uint64_t>());
-  }
+  /* opA = 'T' / 'C': the exponent and quantization kernels read the stored N x M matrix directly (the reference makes a
+   * transposed copy first, src/lra.cpp:63-69) */
+  hyh::quantize_scale_batch(h, opA, sl.batches, sl.batchIter, sl.lastM, N, Atype, A, lda, u, vexp.as<int32_t>());
+  hyacinAllReduceVExp(h, (uint64_t)N, vexp.as<int32_t>());
+  hyh::herk_batch(h, opA, sl.batches, sl.batchIter, sl.lastM, N, Atype, A, lda, u, vexp.as<int32_t>(), 0, lPanels, C.as<uint64_t>());
   hyacinAllReduce1Drow(h, cPanels, lPanels, strideC, C.as<uint64_t>());
   if (lPanels <= 0 || !hyh::ok()) { return 0; }   /* u < 0: nothing was quantized */
   hyacinPrecision_t Gtype = HYACIN_F64; int32_t gBytes = 8;

@@ -69,15 +69,12 @@ __device__ __forceinline__ void store_panel(int8_t* dst, uint32_t packed, int va
 }
 
 /* ------------------------------------------------------------------ limbs */
+/* The work of one thread: Q_ROWS consecutive rows i0 .. of column j, given as raw elements (missing rows zero). */
 template <typename E>
-__global__ __launch_bounds__(Q_THREADS) void quantize_limbs_kernel(int32_t M, int32_t order, const typename E::T* __restrict__ A, int64_t lda, const int32_t* __restrict__ vexp, int8_t* __restrict__ B, int64_t ldb, int64_t strideB) {
-  const int32_t j = blockIdx.y; const int64_t i0 = ((int64_t)blockIdx.x * Q_THREADS + threadIdx.x) * Q_ROWS;
-  if (i0 >= M) { return; }
-  const int valid = (M - i0) < Q_ROWS ? (int)(M - i0) : Q_ROWS; const int32_t expon = vexp[j];
-  int8_t* out = B + (int64_t)j * ldb + i0; const bool aligned = ((uintptr_t)out & 3u) == 0;
+__device__ __forceinline__ void limbs_rows(int32_t order, int32_t expon, const typename E::T (&raw)[Q_ROWS], int valid, int8_t* out, bool aligned, int64_t strideB) {
   constexpr int GROUPS = E::cplx ? 3 : 1;
   if (expon == HYK_INT_MAX) { for (int p = 0; p < order * GROUPS; ++p) { store_panel(out + p * strideB, 0u, valid, aligned); } return; }
-  hyk::I96 q[GROUPS][Q_ROWS]; typename E::T raw[Q_ROWS]; fetch_rows(&A[(int64_t)j * lda + i0], valid, raw);
+  hyk::I96 q[GROUPS][Q_ROWS];
   #pragma unroll
   for (int r = 0; r < Q_ROWS; ++r) {
     hyk::Dec re{ 0, 0, 0 }, im{ 0, 0, 0 }; E::load(&raw[r], re, im);
@@ -98,6 +95,7 @@ __global__ __launch_bounds__(Q_THREADS) void quantize_limbs_kernel(int32_t M, in
     }
   }
 }
+struct LimbsRows { template <typename E> static __device__ __forceinline__ void run(int32_t order, int32_t expon, const typename E::T (&raw)[Q_ROWS], int valid, int8_t* out, bool aligned, int64_t strideB) { limbs_rows<E>(order, expon, raw, valid, out, aligned, strideB); } };
 
 /* ------------------------------------------------------------------ CRT */
 /* DOTS = dwords of the biased two's complement of q that the byte dot products cover: |q| < 2^(32 DOTS - 1) */
@@ -117,18 +115,15 @@ __device__ __forceinline__ void crt_real_step(int32_t order, const hyk::I96 (&q)
   }
 }
 
-template <typename E, int DOTS>
-__global__ __launch_bounds__(Q_THREADS) void quantize_crt_real_kernel(int32_t M, int32_t order, const typename E::T* __restrict__ A, int64_t lda, const int32_t* __restrict__ vexp, int8_t* __restrict__ B, int64_t ldb, int64_t strideB) {
-  const int32_t j = blockIdx.y; const int64_t i0 = ((int64_t)blockIdx.x * Q_THREADS + threadIdx.x) * Q_ROWS;
-  if (i0 >= M) { return; }
-  const int valid = (M - i0) < Q_ROWS ? (int)(M - i0) : Q_ROWS; const int32_t expon = vexp[j];
-  int8_t* out = B + (int64_t)j * ldb + i0; const bool aligned = ((uintptr_t)out & 3u) == 0;
-  if (expon == HYK_INT_MAX) { for (int p = 0; p < order; ++p) { store_panel(out + p * strideB, 0u, valid, aligned); } return; }
-  hyk::I96 q[Q_ROWS]; typename E::T raw[Q_ROWS]; fetch_rows(&A[(int64_t)j * lda + i0], valid, raw);
-  #pragma unroll
-  for (int r = 0; r < Q_ROWS; ++r) { hyk::Dec re{ 0, 0, 0 }, im{ 0, 0, 0 }; E::load(&raw[r], re, im); q[r] = hyk::round_scaled(re, expon); }
-  crt_real_step<E, DOTS, 0>(order, q, out, strideB, valid, aligned);
-}
+template <int DOTS> struct CrtRealRows {
+  template <typename E> static __device__ __forceinline__ void run(int32_t order, int32_t expon, const typename E::T (&raw)[Q_ROWS], int valid, int8_t* out, bool aligned, int64_t strideB) {
+    if (expon == HYK_INT_MAX) { for (int p = 0; p < order; ++p) { store_panel(out + p * strideB, 0u, valid, aligned); } return; }
+    hyk::I96 q[Q_ROWS];
+    #pragma unroll
+    for (int r = 0; r < Q_ROWS; ++r) { hyk::Dec re{ 0, 0, 0 }, im{ 0, 0, 0 }; E::load(&raw[r], re, im); q[r] = hyk::round_scaled(re, expon); }
+    crt_real_step<E, DOTS, 0>(order, q, out, strideB, valid, aligned);
+  }
+};
 
 template <typename E, int DOTS, int X>
 __device__ __forceinline__ void crt_cplx_step(int32_t order, const hyk::I96 (&qr)[Q_ROWS], const hyk::I96 (&qi)[Q_ROWS], int8_t* out, int64_t strideB, int valid, bool aligned) {
@@ -158,19 +153,16 @@ __device__ __forceinline__ void crt_cplx_step(int32_t order, const hyk::I96 (&qr
   }
 }
 
-template <typename E, int DOTS>
-__global__ __launch_bounds__(Q_THREADS) void quantize_crt_cplx_kernel(int32_t M, int32_t order, const typename E::T* __restrict__ A, int64_t lda, const int32_t* __restrict__ vexp, int8_t* __restrict__ B, int64_t ldb, int64_t strideB) {
-  const int32_t j = blockIdx.y; const int64_t i0 = ((int64_t)blockIdx.x * Q_THREADS + threadIdx.x) * Q_ROWS;
-  if (i0 >= M) { return; }
-  const int valid = (M - i0) < Q_ROWS ? (int)(M - i0) : Q_ROWS; const int32_t expon = vexp[j];
-  int8_t* out = B + (int64_t)j * ldb + i0; const bool aligned = ((uintptr_t)out & 3u) == 0;
-  const int panels = order <= HYK_CRT_CPLX_SPLIT ? 2 * order : 3 * order - HYK_CRT_CPLX_SPLIT;
-  if (expon == HYK_INT_MAX) { for (int p = 0; p < panels; ++p) { store_panel(out + p * strideB, 0u, valid, aligned); } return; }
-  hyk::I96 qr[Q_ROWS], qi[Q_ROWS]; typename E::T raw[Q_ROWS]; fetch_rows(&A[(int64_t)j * lda + i0], valid, raw);
-  #pragma unroll
-  for (int r = 0; r < Q_ROWS; ++r) { hyk::Dec re{ 0, 0, 0 }, im{ 0, 0, 0 }; E::load(&raw[r], re, im); qr[r] = hyk::round_scaled(re, expon); qi[r] = hyk::round_scaled(im, expon); }
-  crt_cplx_step<E, DOTS, 0>(order, qr, qi, out, strideB, valid, aligned);
-}
+__device__ __forceinline__ int crt_cplx_panels(int32_t order) { return 2 * (order < HYK_CRT_CPLX_SPLIT ? order : HYK_CRT_CPLX_SPLIT) + 3 * (order > HYK_CRT_CPLX_SPLIT ? order - HYK_CRT_CPLX_SPLIT : 0); }
+template <int DOTS> struct CrtCplxRows {
+  template <typename E> static __device__ __forceinline__ void run(int32_t order, int32_t expon, const typename E::T (&raw)[Q_ROWS], int valid, int8_t* out, bool aligned, int64_t strideB) {
+    if (expon == HYK_INT_MAX) { const int panels = crt_cplx_panels(order); for (int p = 0; p < panels; ++p) { store_panel(out + p * strideB, 0u, valid, aligned); } return; }
+    hyk::I96 qr[Q_ROWS], qi[Q_ROWS];
+    #pragma unroll
+    for (int r = 0; r < Q_ROWS; ++r) { hyk::Dec re{ 0, 0, 0 }, im{ 0, 0, 0 }; E::load(&raw[r], re, im); qr[r] = hyk::round_scaled(re, expon); qi[r] = hyk::round_scaled(im, expon); }
+    crt_cplx_step<E, DOTS, 0>(order, qr, qi, out, strideB, valid, aligned);
+  }
+};
 
 /* ------------------------------------------------------------------ CRT, quantized values below 2^51
  * q = rint(x * 2^vexp) is then exact in a double (ldexp and rint are exact operations), and every residue costs three
@@ -210,18 +202,15 @@ __device__ __forceinline__ void crt_real_f64_step(int32_t order, const double (&
   }
 }
 
-template <typename E>
-__global__ __launch_bounds__(Q_THREADS) void quantize_crt_real_f64_kernel(int32_t M, int32_t order, const typename E::T* __restrict__ A, int64_t lda, const int32_t* __restrict__ vexp, int8_t* __restrict__ B, int64_t ldb, int64_t strideB) {
-  const int32_t j = blockIdx.y; const int64_t i0 = ((int64_t)blockIdx.x * Q_THREADS + threadIdx.x) * Q_ROWS;
-  if (i0 >= M) { return; }
-  const int valid = (M - i0) < Q_ROWS ? (int)(M - i0) : Q_ROWS; const int32_t expon = vexp[j];
-  int8_t* out = B + (int64_t)j * ldb + i0; const bool aligned = ((uintptr_t)out & 3u) == 0;
-  if (expon == HYK_INT_MAX) { for (int p = 0; p < order; ++p) { store_panel(out + p * strideB, 0u, valid, aligned); } return; }
-  double a[Q_ROWS], ab[Q_ROWS]; typename E::T raw[Q_ROWS]; fetch_rows(&A[(int64_t)j * lda + i0], valid, raw);
-  #pragma unroll
-  for (int r = 0; r < Q_ROWS; ++r) { double re = 0., im = 0.; E::load_f64(&raw[r], re, im); a[r] = __builtin_rint(__builtin_ldexp(re, expon)); ab[r] = a[r] + LOW_BITS; }
-  crt_real_f64_step<0>(order, a, ab, out, strideB, valid, aligned);
-}
+struct CrtRealF64Rows {
+  template <typename E> static __device__ __forceinline__ void run(int32_t order, int32_t expon, const typename E::T (&raw)[Q_ROWS], int valid, int8_t* out, bool aligned, int64_t strideB) {
+    if (expon == HYK_INT_MAX) { for (int p = 0; p < order; ++p) { store_panel(out + p * strideB, 0u, valid, aligned); } return; }
+    double a[Q_ROWS], ab[Q_ROWS];
+    #pragma unroll
+    for (int r = 0; r < Q_ROWS; ++r) { double re = 0., im = 0.; E::load_f64(&raw[r], re, im); a[r] = __builtin_rint(__builtin_ldexp(re, expon)); ab[r] = a[r] + LOW_BITS; }
+    crt_real_f64_step<0>(order, a, ab, out, strideB, valid, aligned);
+  }
+};
 
 template <int X>
 __device__ __forceinline__ void crt_cplx_f64_step(int32_t order, const double (&ar)[Q_ROWS], const double (&ai)[Q_ROWS], int8_t* out, int64_t strideB, int valid, bool aligned) {
@@ -251,21 +240,67 @@ __device__ __forceinline__ void crt_cplx_f64_step(int32_t order, const double (&
   }
 }
 
-template <typename E>
-__global__ __launch_bounds__(Q_THREADS) void quantize_crt_cplx_f64_kernel(int32_t M, int32_t order, const typename E::T* __restrict__ A, int64_t lda, const int32_t* __restrict__ vexp, int8_t* __restrict__ B, int64_t ldb, int64_t strideB) {
+struct CrtCplxF64Rows {
+  template <typename E> static __device__ __forceinline__ void run(int32_t order, int32_t expon, const typename E::T (&raw)[Q_ROWS], int valid, int8_t* out, bool aligned, int64_t strideB) {
+    if (expon == HYK_INT_MAX) { const int panels = crt_cplx_panels(order); for (int p = 0; p < panels; ++p) { store_panel(out + p * strideB, 0u, valid, aligned); } return; }
+    double ar[Q_ROWS], ai[Q_ROWS];
+    #pragma unroll
+    for (int r = 0; r < Q_ROWS; ++r) {
+      double re = 0., im = 0.; E::load_f64(&raw[r], re, im);
+      ar[r] = __builtin_rint(__builtin_ldexp(re, expon)); ai[r] = __builtin_rint(__builtin_ldexp(im, expon));
+    }
+    crt_cplx_f64_step<0>(order, ar, ai, out, strideB, valid, aligned);
+  }
+};
+
+/* A column-major (M x N, leading dimension lda): one thread takes Q_ROWS consecutive rows of one column straight from memory. */
+template <typename E, typename ROWS>
+__global__ __launch_bounds__(Q_THREADS) void quantize_kernel(int32_t M, int32_t order, const typename E::T* __restrict__ A, int64_t lda, const int32_t* __restrict__ vexp, int8_t* __restrict__ B, int64_t ldb, int64_t strideB) {
   const int32_t j = blockIdx.y; const int64_t i0 = ((int64_t)blockIdx.x * Q_THREADS + threadIdx.x) * Q_ROWS;
   if (i0 >= M) { return; }
   const int valid = (M - i0) < Q_ROWS ? (int)(M - i0) : Q_ROWS; const int32_t expon = vexp[j];
   int8_t* out = B + (int64_t)j * ldb + i0; const bool aligned = ((uintptr_t)out & 3u) == 0;
-  const int panels = 2 * (order < HYK_CRT_CPLX_SPLIT ? order : HYK_CRT_CPLX_SPLIT) + 3 * (order > HYK_CRT_CPLX_SPLIT ? order - HYK_CRT_CPLX_SPLIT : 0);
-  if (expon == HYK_INT_MAX) { for (int p = 0; p < panels; ++p) { store_panel(out + p * strideB, 0u, valid, aligned); } return; }
-  double ar[Q_ROWS], ai[Q_ROWS]; typename E::T raw[Q_ROWS]; fetch_rows(&A[(int64_t)j * lda + i0], valid, raw);
-  #pragma unroll
-  for (int r = 0; r < Q_ROWS; ++r) {
-    double re = 0., im = 0.; E::load_f64(&raw[r], re, im);
-    ar[r] = __builtin_rint(__builtin_ldexp(re, expon)); ai[r] = __builtin_rint(__builtin_ldexp(im, expon));
+  typename E::T raw[Q_ROWS];
+  if (expon != HYK_INT_MAX) { fetch_rows(&A[(int64_t)j * lda + i0], valid, raw); } else { for (int r = 0; r < Q_ROWS; ++r) { raw[r] = typename E::T{}; } }
+  ROWS::template run<E>(order, expon, raw, valid, out, aligned, strideB);
+}
+
+/* A stored as its (conjugate) transpose: the N x M matrix S with op(A)[k, j] = S[j + k lda] (conjugated when CONJ), i.e.
+ * the rows of op(A) are contiguous in memory.  A workgroup moves a tile of TJ columns x T_ROWS rows through LDS (reads
+ * run along j, whole rows of the stored matrix; the quantized bytes leave along k, 128 per panel and column), then every
+ * thread quantizes groups of Q_ROWS rows exactly as in the column-major kernel.  Replaces the transposing copy of the
+ * reference (src/lra.cpp:63-69, src/matcopy.cu:36-43) together with the kernel that followed it. */
+constexpr int T_ROWS = 128;
+template <typename T> struct TileCols { static constexpr int value = sizeof(T) >= 8 ? 32 : 64; };
+template <typename E> __device__ __forceinline__ typename E::T conj_elem(typename E::T v) {
+  if constexpr (!E::cplx) { return v; }
+  else if constexpr (sizeof(typename E::T) == 16) { v.y ^= 0x8000000000000000ull; return v; }
+  else if constexpr (sizeof(typename E::T) == 8) { v.y ^= 0x80000000u; return v; }
+  else { return v ^ 0x80000000u; }   /* two halves in one word: the imaginary part is the upper one */
+}
+template <typename E, typename ROWS, bool CONJ>
+__global__ __launch_bounds__(Q_THREADS) void quantize_transposed_kernel(int32_t M, int32_t N, int32_t order, const typename E::T* __restrict__ S, int64_t lda, const int32_t* __restrict__ vexp, int8_t* __restrict__ B, int64_t ldb, int64_t strideB) {
+  using T = typename E::T; constexpr int TJ = TileCols<T>::value, PITCH = T_ROWS + 1;
+  extern __shared__ __attribute__((aligned(16))) unsigned char tileBytes[];
+  T* tile = reinterpret_cast<T*>(tileBytes);
+  const int64_t k0 = (int64_t)blockIdx.x * T_ROWS; const int32_t j0 = blockIdx.y * TJ;
+  for (int e = threadIdx.x; e < TJ * T_ROWS; e += Q_THREADS) {
+    const int jj = e % TJ, kk = e / TJ; T v = T{};
+    if (j0 + jj < N && k0 + kk < M) { v = S[(int64_t)(j0 + jj) + (k0 + kk) * lda]; if constexpr (CONJ) { v = conj_elem<E>(v); } }
+    tile[jj * PITCH + kk] = v;
   }
-  crt_cplx_f64_step<0>(order, ar, ai, out, strideB, valid, aligned);
+  __syncthreads();
+  constexpr int GROUPS = T_ROWS / Q_ROWS;   /* 32 row groups per column: a wavefront covers two columns */
+  for (int e = threadIdx.x; e < TJ * GROUPS; e += Q_THREADS) {
+    const int kg = e % GROUPS, jj = e / GROUPS; const int32_t j = j0 + jj; const int64_t i0 = k0 + (int64_t)kg * Q_ROWS;
+    if (j >= N || i0 >= M) { continue; }
+    const int valid = (M - i0) < Q_ROWS ? (int)(M - i0) : Q_ROWS; const int32_t expon = vexp[j];
+    int8_t* out = B + (int64_t)j * ldb + i0; const bool aligned = ((uintptr_t)out & 3u) == 0;
+    T raw[Q_ROWS];
+    #pragma unroll
+    for (int r = 0; r < Q_ROWS; ++r) { raw[r] = tile[jj * PITCH + kg * Q_ROWS + r]; }
+    ROWS::template run<E>(order, expon, raw, valid, out, aligned, strideB);
+  }
 }
 
 /* rows [row0, row1) of `panels` panels set to zero: the Gram kernel contracts over whole 128-row blocks */
@@ -275,49 +310,75 @@ __global__ void zero_rows_kernel(int8_t* __restrict__ B, int64_t ldb, int64_t co
   (void)cols;
 }
 
-}  // namespace
+template <typename E, typename ROWS>
+int launch_quantize(hipStream_t stream, char op, int32_t M, int32_t N, int32_t order, const void* A, int64_t lda, const int32_t* vexp, int8_t* B, int64_t ldb) {
+  using T = typename E::T; const int64_t strideB = (int64_t)N * ldb;
+  if (op == 'N') {
+    dim3 grid((uint32_t)((M + Q_THREADS * Q_ROWS - 1) / (Q_THREADS * Q_ROWS)), (uint32_t)N);
+    quantize_kernel<E, ROWS><<<grid, Q_THREADS, 0, stream>>>(M, order, (const T*)A, lda, vexp, B, ldb, strideB);
+  } else {
+    constexpr int TJ = TileCols<T>::value; const size_t lds = (size_t)TJ * (T_ROWS + 1) * sizeof(T);
+    dim3 grid((uint32_t)((M + T_ROWS - 1) / T_ROWS), (uint32_t)((N + TJ - 1) / TJ));
+    if (op == 'C' && E::cplx) {
+      if (lds > 65536 && hipFuncSetAttribute(reinterpret_cast<const void*>(&quantize_transposed_kernel<E, ROWS, true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) { return -3; }
+      quantize_transposed_kernel<E, ROWS, true><<<grid, Q_THREADS, lds, stream>>>(M, N, order, (const T*)A, lda, vexp, B, ldb, strideB);
+    } else {
+      if (lds > 65536 && hipFuncSetAttribute(reinterpret_cast<const void*>(&quantize_transposed_kernel<E, ROWS, false>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) { return -3; }
+      quantize_transposed_kernel<E, ROWS, false><<<grid, Q_THREADS, lds, stream>>>(M, N, order, (const T*)A, lda, vexp, B, ldb, strideB);
+    }
+  }
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
 
-#define HYK_QGRID dim3 grid((uint32_t)((M + Q_THREADS * Q_ROWS - 1) / (Q_THREADS * Q_ROWS)), (uint32_t)N)
-
-extern "C" int hykQuantizeLimbs(hipStream_t stream, int32_t M, int32_t N, int32_t orderA, int32_t Atype, const void* A, int64_t lda, const int32_t* vexp, int8_t* B, int64_t ldb) {
-  if (M <= 0 || N <= 0) { return 0; }
-  if (orderA < 1 || orderA > 12 || N > 65535 || ldb < M) { return -1; }
-  const int64_t strideB = (int64_t)N * ldb; HYK_QGRID;
+template <typename ROWS>
+int launch_quantize_type(hipStream_t stream, char op, int32_t M, int32_t N, int32_t order, int32_t Atype, const void* A, int64_t lda, const int32_t* vexp, int8_t* B, int64_t ldb) {
   switch (Atype) {
-    case HYK_F64: quantize_limbs_kernel<ElemF64><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const uint64_t*)A, lda, vexp, B, ldb, strideB); break;
-    case HYK_F32: quantize_limbs_kernel<ElemF32><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const uint32_t*)A, lda, vexp, B, ldb, strideB); break;
-    case HYK_F16: quantize_limbs_kernel<ElemF16><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const uint16_t*)A, lda, vexp, B, ldb, strideB); break;
-    case HYK_F64C: quantize_limbs_kernel<ElemF64C><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const ulonglong2*)A, lda, vexp, B, ldb, strideB); break;
-    case HYK_F32C: quantize_limbs_kernel<ElemF32C><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const uint2*)A, lda, vexp, B, ldb, strideB); break;
-    case HYK_F16C: quantize_limbs_kernel<ElemF16C><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const uint32_t*)A, lda, vexp, B, ldb, strideB); break;
+    case HYK_F64: return launch_quantize<ElemF64, ROWS>(stream, op, M, N, order, A, lda, vexp, B, ldb);
+    case HYK_F32: return launch_quantize<ElemF32, ROWS>(stream, op, M, N, order, A, lda, vexp, B, ldb);
+    case HYK_F16: return launch_quantize<ElemF16, ROWS>(stream, op, M, N, order, A, lda, vexp, B, ldb);
+    case HYK_F64C: return launch_quantize<ElemF64C, ROWS>(stream, op, M, N, order, A, lda, vexp, B, ldb);
+    case HYK_F32C: return launch_quantize<ElemF32C, ROWS>(stream, op, M, N, order, A, lda, vexp, B, ldb);
+    case HYK_F16C: return launch_quantize<ElemF16C, ROWS>(stream, op, M, N, order, A, lda, vexp, B, ldb);
     default: return -1;
   }
-  return 0;
+}
+
+char norm_op(char op) { return (op == 'T' || op == 't') ? 'T' : ((op == 'C' || op == 'c') ? 'C' : 'N'); }
+
+}  // namespace
+
+extern "C" int hykQuantizeLimbsOp(hipStream_t stream, char opA, int32_t M, int32_t N, int32_t orderA, int32_t Atype, const void* A, int64_t lda, const int32_t* vexp, int8_t* B, int64_t ldb) {
+  if (M <= 0 || N <= 0) { return 0; }
+  const char op = norm_op(opA);
+  if (orderA < 1 || orderA > 12 || N > 65535 || ldb < M || lda < (op == 'N' ? M : N)) { return -1; }
+  return launch_quantize_type<LimbsRows>(stream, op, M, N, orderA, Atype, A, lda, vexp, B, ldb);
+}
+
+extern "C" int hykQuantizeLimbs(hipStream_t stream, int32_t M, int32_t N, int32_t orderA, int32_t Atype, const void* A, int64_t lda, const int32_t* vexp, int8_t* B, int64_t ldb) {
+  return hykQuantizeLimbsOp(stream, 'N', M, N, orderA, Atype, A, lda, vexp, B, ldb);
 }
 
 /* maxBits: an upper bound on the bit length of |q| (u + 1 covers re + im as well); <= 0 means unknown */
-extern "C" int hykQuantizeCrt(hipStream_t stream, int32_t M, int32_t N, int32_t orderA, int32_t Atype, const void* A, int64_t lda, const int32_t* vexp, int8_t* B, int64_t ldb, int32_t maxBits) {
+extern "C" int hykQuantizeCrtOp(hipStream_t stream, char opA, int32_t M, int32_t N, int32_t orderA, int32_t Atype, const void* A, int64_t lda, const int32_t* vexp, int8_t* B, int64_t ldb, int32_t maxBits) {
   if (M <= 0 || N <= 0) { return 0; }
-  const int cplx = Atype & 1;
-  if (orderA < 1 || orderA > (cplx ? HYK_CRT_CPLX_COUNT : HYK_CRT_REAL_COUNT) || N > 65535 || ldb < M) { return -1; }
-  const int64_t strideB = (int64_t)N * ldb; HYK_QGRID; const int dots = (0 < maxBits && maxBits <= 31) ? 1 : (0 < maxBits && maxBits <= 63) ? 2 : 3;
+  const int cplx = Atype & 1; const char op = norm_op(opA);
+  if (orderA < 1 || orderA > (cplx ? HYK_CRT_CPLX_COUNT : HYK_CRT_REAL_COUNT) || N > 65535 || ldb < M || lda < (op == 'N' ? M : N)) { return -1; }
+  const int dots = (0 < maxBits && maxBits <= 31) ? 1 : (0 < maxBits && maxBits <= 63) ? 2 : 3;
   const bool viaF64 = (0 < maxBits && maxBits <= 51);   /* |q|, and |re + im| for complex input, below 2^51: exact in a double */
-  #define HYK_LAUNCH_CRT(KERNEL, ELEM, TYPE) \
-    if (viaF64) { KERNEL##_f64_kernel<ELEM><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const TYPE*)A, lda, vexp, B, ldb, strideB); } \
-    else if (dots == 1) { KERNEL##_kernel<ELEM, 1><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const TYPE*)A, lda, vexp, B, ldb, strideB); } \
-    else if (dots == 2) { KERNEL##_kernel<ELEM, 2><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const TYPE*)A, lda, vexp, B, ldb, strideB); } \
-    else { KERNEL##_kernel<ELEM, 3><<<grid, Q_THREADS, 0, stream>>>(M, orderA, (const TYPE*)A, lda, vexp, B, ldb, strideB); }
-  switch (Atype) {
-    case HYK_F64: HYK_LAUNCH_CRT(quantize_crt_real, ElemF64, uint64_t) break;
-    case HYK_F32: HYK_LAUNCH_CRT(quantize_crt_real, ElemF32, uint32_t) break;
-    case HYK_F16: HYK_LAUNCH_CRT(quantize_crt_real, ElemF16, uint16_t) break;
-    case HYK_F64C: HYK_LAUNCH_CRT(quantize_crt_cplx, ElemF64C, ulonglong2) break;
-    case HYK_F32C: HYK_LAUNCH_CRT(quantize_crt_cplx, ElemF32C, uint2) break;
-    case HYK_F16C: HYK_LAUNCH_CRT(quantize_crt_cplx, ElemF16C, uint32_t) break;
-    default: return -1;
+  if (!cplx) {
+    if (viaF64) { return launch_quantize_type<CrtRealF64Rows>(stream, op, M, N, orderA, Atype, A, lda, vexp, B, ldb); }
+    if (dots == 1) { return launch_quantize_type<CrtRealRows<1>>(stream, op, M, N, orderA, Atype, A, lda, vexp, B, ldb); }
+    if (dots == 2) { return launch_quantize_type<CrtRealRows<2>>(stream, op, M, N, orderA, Atype, A, lda, vexp, B, ldb); }
+    return launch_quantize_type<CrtRealRows<3>>(stream, op, M, N, orderA, Atype, A, lda, vexp, B, ldb);
   }
-  #undef HYK_LAUNCH_CRT
-  return 0;
+  if (viaF64) { return launch_quantize_type<CrtCplxF64Rows>(stream, op, M, N, orderA, Atype, A, lda, vexp, B, ldb); }
+  if (dots == 1) { return launch_quantize_type<CrtCplxRows<1>>(stream, op, M, N, orderA, Atype, A, lda, vexp, B, ldb); }
+  if (dots == 2) { return launch_quantize_type<CrtCplxRows<2>>(stream, op, M, N, orderA, Atype, A, lda, vexp, B, ldb); }
+  return launch_quantize_type<CrtCplxRows<3>>(stream, op, M, N, orderA, Atype, A, lda, vexp, B, ldb);
+}
+
+extern "C" int hykQuantizeCrt(hipStream_t stream, int32_t M, int32_t N, int32_t orderA, int32_t Atype, const void* A, int64_t lda, const int32_t* vexp, int8_t* B, int64_t ldb, int32_t maxBits) {
+  return hykQuantizeCrtOp(stream, 'N', M, N, orderA, Atype, A, lda, vexp, B, ldb, maxBits);
 }
 
 extern "C" int hykZeroRows(hipStream_t stream, int8_t* B, int64_t ldb, int64_t cols, int32_t row0, int32_t row1) {

@@ -22,6 +22,11 @@ extern "C" {
  * vexp: (batches + 1) * N int32 = [global | slice 0 | slice 1 | ...]. lda in elements. */
 int hykColumnExponents(hipStream_t stream, int32_t batches, int32_t segM, int32_t lastM, int32_t N, int32_t Atype, const void* A, int64_t lda, int32_t u, int32_t* vexp);
 
+/* The same with the storage order of A as an argument: opA 'N' as above; 'T' / 'C': A is the stored N x M matrix with
+ * op(A)[k, j] = A[j + k lda] (lda >= N), read in place.  Replaces the transposing copy of src/lra.cpp:63-69 +
+ * src/matcopy.cu:36-43 followed by the kernels above. */
+int hykColumnExponentsOp(hipStream_t stream, char opA, int32_t batches, int32_t segM, int32_t lastM, int32_t N, int32_t Atype, const void* A, int64_t lda, int32_t u, int32_t* vexp);
+
 /* Bits needed per row slice.  Replaces internal::int8::vector_range, src/fp_exponent.cu:67-76. */
 int hykSliceRange(hipStream_t stream, int32_t batches, int32_t N, int32_t u, const int32_t* vexp, int32_t* segU);
 
@@ -32,6 +37,13 @@ int hykQuantizeLimbs(hipStream_t stream, int32_t M, int32_t N, int32_t orderA, i
 /* CRT residue panels.  Replaces internal::int8::quantize_crt, src/quantize_crt_real.cu:63-112 and
  * src/quantize_crt_complex.cu:72-123.  maxBits: bound on the bit length of the quantized magnitudes (<= 0: unknown). */
 int hykQuantizeCrt(hipStream_t stream, int32_t M, int32_t N, int32_t orderA, int32_t Atype, const void* A, int64_t lda, const int32_t* vexp, int8_t* B, int64_t ldb, int32_t maxBits);
+
+/* The two quantizers reading op(A) from the stored N x M (conjugate) transpose when opA is 'T' / 'C' (A points at the
+ * first of the M stored columns to quantize, lda >= N): a workgroup moves a tile through LDS, so the reads run along the
+ * stored columns and the panel bytes still leave K-contiguous; 'C' conjugates on the way.  Same panels, bit for bit, as
+ * a transposing copy followed by the column-major kernel (src/lra.cpp:63-69, src/matcopy.cu:36-43). */
+int hykQuantizeLimbsOp(hipStream_t stream, char opA, int32_t M, int32_t N, int32_t orderA, int32_t Atype, const void* A, int64_t lda, const int32_t* vexp, int8_t* B, int64_t ldb);
+int hykQuantizeCrtOp(hipStream_t stream, char opA, int32_t M, int32_t N, int32_t orderA, int32_t Atype, const void* A, int64_t lda, const int32_t* vexp, int8_t* B, int64_t ldb, int32_t maxBits);
 
 /* Rows [row0, row1) of `cols` consecutive panel columns set to zero.  Replaces the cudaMemset2DAsync padding of
  * src/hyacin_herk.cpp:154,261,275. */
@@ -142,6 +154,19 @@ int hykGemm(hipStream_t stream, char opA, char opB, int32_t M, int32_t N, int32_
  * Jacobi rotations, then column normalisation).  Replaces the Q factor of cuSOLVER geqrf + orgqr/ungqr,
  * src/lra.cpp:176-191: the same subspace, a different basis of it.  work: r * sizeof(element) + 64 bytes. */
 int hykOrthonormalize(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* V, int64_t ldv, double* work);
+
+/* hyacinXquantizeScaleBatch / hyacinXherkBatch (include/hyacin.h) with the storage order of A as an argument, as the
+ * fits call them: opA 'N' column-major M x N, 'T' / 'C' the stored N x M (conjugate) transpose, lda >= N.  handle is a
+ * const hyacinHandle_t*. */
+void hykQuantizeScaleBatchOp(const void* handle, char opA, int32_t batches, int32_t segM, int32_t lastM, int32_t N, int32_t Atype, const void* A, int64_t lda, int32_t uA, int32_t* vexp);
+void hykHerkBatchOp(const void* handle, char opA, int32_t batches, int32_t segM, int32_t lastM, int32_t N, int32_t Atype, const void* A, int64_t lda, int32_t u, const int32_t* vexp, int32_t beta, int32_t orderC, uint64_t* C);
+
+/* What the last hyacinXherkBatch / hykHerkBatchOp of the calling thread planned and issued (no counterpart in the
+ * reference, which prints the same facts through its logger): algorithm ('L' limbs / 'C' residues) and order of the last
+ * bucket, rows per contraction call, calls issued, rows contracted, and the algorithmic int8 operations of all
+ * contraction calls together (2 per multiply-add, upper triangle only). */
+typedef struct { int32_t algorithm, order, chunkRows, gramCalls, quantizeCalls, reserved; int64_t rows; double int8Ops; } hykHerkPlan;
+int hykLastHerkPlan(hykHerkPlan* out);
 
 /* Status of the last outermost hyacin.h call made on the calling thread: 0, or the code of the first failure inside it
  * (a HIP error number, a negative kernel-layer return value, -4 a scratch allocation that failed, -5 a pivoted Cholesky

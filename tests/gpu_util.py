@@ -47,6 +47,25 @@ def colmajor_bytes(A):
     return dev(flat), lda, ho.atype_of(A)
 
 
+def stored_transpose(A, op, pad=0):
+    """The stored N x M matrix S with op(S) = A (op 'T' or 'C'), column-major with leading dimension N + pad: returns
+    (device tensor, lda, precision enum).  S[j + k lda] = A[k, j], conjugated for 'C'; the padding holds NaN."""
+    from oracle import ho
+    at = ho.atype_of(A)
+    M, N = A.shape[0], A.shape[1]
+    if A.ndim == 3:                                   # complex half as [M, N, 2]
+        body = A.copy()
+        if op == "C":
+            body[..., 1] = -body[..., 1]
+        buf = np.full((M, N + pad, 2), np.nan, np.float16)
+        buf[:, :N] = body
+    else:
+        body = np.conj(A) if (op == "C" and np.iscomplexobj(A)) else A
+        buf = np.full((M, N + pad), np.nan, A.dtype)
+        buf[:, :N] = body
+    return dev(buf), N + pad, at
+
+
 def check(rc):
     assert rc == 0, "kernel layer returned %d" % rc
 
@@ -62,6 +81,29 @@ class Lib:
         check(self.L.hykColumnExponents(stream(), batches, segM, lastM, N, at, ptr(d), lda, u, ptr(vexp)))
         sync()
         return host(vexp, np.int32)
+
+    def column_exponents_op(self, A, op, batches, segM, lastM, u, pad=0):
+        d, lda, at = stored_transpose(A, op, pad)
+        N = A.shape[1]
+        vexp = zeros(4 * (max(batches, 0) + 1) * N)
+        check(self.L.hykColumnExponentsOp(stream(), op.encode(), batches, segM, lastM, N, at, ptr(d), lda, u, ptr(vexp)))
+        sync()
+        return host(vexp, np.int32)
+
+    def quantize_op(self, kind, A, op, order, vexp, ldb=None, max_bits=0, pad=0):
+        from oracle import ho
+        d, lda, at = stored_transpose(A, op, pad)
+        M, N = A.shape[0], A.shape[1]
+        ldb = ldb or M
+        panels = ho.n_panels(kind, order, at & 1)
+        B = zeros(panels * N * ldb)
+        dv = dev(np.ascontiguousarray(vexp[:N]))
+        if kind == "limbs":
+            check(self.L.hykQuantizeLimbsOp(stream(), op.encode(), M, N, order, at, ptr(d), lda, ptr(dv), ptr(B), ldb))
+        else:
+            check(self.L.hykQuantizeCrtOp(stream(), op.encode(), M, N, order, at, ptr(d), lda, ptr(dv), ptr(B), ldb, max_bits))
+        sync()
+        return host(B, np.int8, (panels, N, ldb))
 
     def quantize(self, kind, A, order, vexp, ldb=None, row_offset=0, max_bits=0):
         from oracle import ho

@@ -87,6 +87,33 @@ def test_quantize_panels_bit_exact(gl, oracle, kind):
     assert np.array_equal(got[:, :, 7:57], want) and not got[:, :, :7].any() and not got[:, :, 57:].any()
 
 
+@pytest.mark.parametrize("op", ["T", "C"])
+@pytest.mark.parametrize("kind", ALL_KINDS)
+def test_transposed_storage_bit_exact(gl, oracle, kind, op):
+    """opA = 'T' / 'C' without a transposed copy (the reference copies first, src/lra.cpp:63-69): exponents and panels read
+    from the stored N x M matrix equal the oracle's on op(A), bit for bit.  Leading dimension above N, sizes off the
+    128 x 32 / 64 tiles, several row slices, a zero column, both residue paths, limbs."""
+    rng = np.random.default_rng(133)
+    cplx = kind.startswith("c")
+    for (M, N, segM, pad) in [(70, 9, 16, 0), (300, 45, 128, 3), (1029, 70, 1029, 8), (257, 130, 100, 1)]:
+        A = special(rng, M, N, kind)
+        batches, lastM = (M + segM - 1) // segM, M - (M - 1) // segM * segM
+        for u in (23, 46):
+            print("transposed exponents", kind, op, M, N, segM, u, flush=True)
+            want = oracle.quantize_scale_batch(A, batches, segM, lastM, u)
+            got = gl.column_exponents_op(A, op, batches, segM, lastM, u, pad)
+            assert np.array_equal(got[:len(want)], want)
+        for u in (23, 62):
+            vexp = oracle.quantize_scale_batch(A, 1, M, M, u)
+            print("transposed limbs", kind, op, M, N, u, flush=True)
+            assert np.array_equal(gl.quantize_op("limbs", A, op, 4, vexp, ldb=M + 5, pad=pad), oracle.quantize("limbs", A, 4, vexp, ldb=M + 5))
+            order = 21 if cplx else 14
+            want = oracle.quantize("crt", A, order, vexp, ldb=M + 3)
+            for mb in (0, u + 1):
+                print("transposed crt", kind, op, M, N, u, order, mb, flush=True)
+                assert np.array_equal(gl.quantize_op("crt", A, op, order, vexp, ldb=M + 3, max_bits=mb, pad=pad), want)
+
+
 def random_panels(rng, p, N, K, rows, lo=-128, hi=128):
     P = rng.integers(lo, hi, size=(p, N, K), dtype=np.int64).astype(np.int8)
     P[:, :, rows:] = 0
