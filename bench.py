@@ -1,20 +1,32 @@
 #!/usr/bin/env python3
 """Benchmark of the quantized Gram build (the hot path of hyacinTsvdFit) on one MI355X.
 
-A step = hyacinXquantizeScaleBatch + hyacinXherkBatch on a synthetic matrix that is already resident in
-HBM: per-column exponents, int8 CRT-residue / limb quantization, the int8 MFMA contraction and the
-reconstruction of the exact integer Gram.  Prints ONE JSON line:
+A step = column exponents + exact integer Gram (hyacinXquantizeScaleBatch + hyacinXherkBatch, through the entry points that
+take the storage order of A) on a synthetic matrix that is already resident in HBM: per-column exponents, int8 CRT-residue
+/ limb quantization, the int8 MFMA contraction and the reconstruction of the exact integer Gram.  Prints ONE JSON line:
   value      effective Gram TFLOP/s = M N (N+1) (x4 complex) / step time  (the FP SYRK/HERK flops replaced)
-  roofline   the contraction kernel alone, timed with HIP events on its stream: algorithmic int8 ops / time
-             against the dense INT8 MFMA peak
-  cpu_baseline  the same limb / CRT algorithm compiled for the host (the oracle), timed on a row sample, with
-             OpenBLAS DSYRK / ZHERK on the same sample and LAPACK syevd / heevd on its N x N Gram beside it
+  roofline   the contraction kernel alone, timed with HIP events on its stream: algorithmic int8 ops (as the library
+             reports them for what it launched) / time against the dense INT8 MFMA peak; board power and shader clock
+             sampled while that kernel runs back to back
+  tsvd_fit_ms  the fit the configuration names, wall clock, median of 5 after 2 warm-ups
+  cpu_baseline  the same limb / CRT algorithm compiled for the host (the oracle), timed on a row sample of the same matrix,
+             with OpenBLAS DSYRK / ZHERK on the same sample and LAPACK syevd / heevd on its N x N Gram beside it
+
+Workloads are generated on the device from a fixed seed per configuration (0x48594143494E0000 + number; torch's Philox
+generator, so a seed fixes the matrix).  Orthonormal factors: V (N x N) is Haar (QR of a Gaussian with the sign fix); the
+tall factor U (M x N) is D2 H [D1; 0] / sqrt(M) with random sign (phase) diagonals D1, D2 and H the Hartley (real) or
+Fourier (complex) transform of length M: orthonormal columns with entries of even size, O(M N log M) to build.
 """
 import argparse
 import ctypes as C
+import glob
+import hashlib
 import json
+import math
 import os
+import re
 import sys
+import threading
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
@@ -22,27 +34,62 @@ sys.path.insert(0, ROOT)
 
 INT8_PEAK_TOPS = 5000.0   # MI355X dense INT8 MFMA peak, 5.0 POP/s
 HBM_PEAK_GBS = 8000.0     # MI355X HBM3E peak, 8 TB/s
-
-# HBM bytes per launch of the contraction kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this script
-# (profiles/gram_ring_kernel_target_hbm_traffic.md), each scaled by what the counter reads for copy_kernel's known 1 GiB.
-MEASURED_TRAFFIC = {("target", 0): 5.65e9 + 0.12e9}
+SEED0 = 0x48594143494E0000
 
 WORKLOADS = {
-    # name: (type, opA, M, N, K, eps, algorithm, description)
-    "target": (0, "N", 131072, 2048, 1024, 1e-12, b"A", "real FP64 M=131072 N=2048 eps=1e-12 (CRT real, 14 moduli)"),
-    "cfg1": (0, "N", 4096, 256, 256, 1e-10, b"L", "real FP64 M=4096 N=256 eps=1e-10 (limbs, 6 digits)"),
-    "cfg2": (2, "T", 65536, 1024, 512, 1e-5, b"A", "real FP32 opA=T M=65536 N=1024 eps=1e-5 (CRT real, 8 moduli)"),
-    "cfg3": (1, "N", 131072, 2048, 1024, 1e-12, b"A", "complex FP64 M=131072 N=2048 eps=1e-12 (CRT complex, 15 moduli)"),
-    "cfg4": (5, "C", 262144, 4096, 256, 1e-3, b"L", "complex FP16 opA=C M=262144 N=4096 eps=1e-3 (limbs, 3 digits x 3 groups)"),
-    "cfg5": (0, "N", 1048576, 4096, 2048, 1e-8, b"A", "real FP64 M=1048576 N=4096 eps=1e-8 (CRT real, 11 moduli)"),
+    # name: (number, type, opA, M, N, K, eps, algorithm, fit entry point, description)
+    "cfg1": (1, 0, "N", 4096, 256, 256, 1e-10, b"L", "hyacinTsvdFit", "real FP64 M=4096 N=256 eps=1e-10: U diag(10^(-i/16)) V^T (limbs, 6 digits)"),
+    "cfg2": (2, 2, "T", 65536, 1024, 512, 1e-5, b"A", "hyacinTsvdFit", "real FP32 opA=T (stored N x M) M=65536 N=1024 eps=1e-5: U diag(2^(-i/32)) V^T + 1e-7 G (CRT real, 8 moduli)"),
+    "cfg3": (3, 1, "N", 131072, 2048, 1024, 1e-12, b"A", "hyacinTsvdFitSegmentN", "complex FP64 M=131072 N=2048 eps=1e-12: U diag(10^(-i/128)) V^H + 1e-14 (Gr + i Gi) (CRT complex, 15 moduli)"),
+    "cfg4": (4, 5, "C", 262144, 4096, 256, 1e-3, b"L", "hyacinTsvdFit", "complex FP16 opA=C (stored N x M) M=262144 N=4096 eps=1e-3: rank-256 L R + 1e-4 noise (limbs, 3 digits x 3 groups)"),
+    "cfg5": (5, 0, "N", 1048576, 4096, 2048, 1e-8, b"A", "hyacinInterpolateFit", "real FP64 M=1048576 N=4096 eps=1e-8: (U diag(10^(-i/256)) V^T) D, D log-uniform in [1e-6, 1e6] (CRT real, 11 moduli)"),
+    "target": (6, 0, "N", 131072, 2048, 1024, 1e-12, b"A", "hyacinTsvdFit", "real FP64 M=131072 N=2048 eps=1e-12: U diag(10^(-i/128)) V^T + 1e-14 G (CRT real, 14 moduli)"),
 }
 
 
-def synth_low_rank(torch, M, N, rank, noise, seed):
-    """Configuration 4's own recipe: a rank-`rank` product L R with entries complex N(0, 1 / 256) plus complex Gaussian
-    noise of size `noise`, cast to half; column-major M x N (the tensor is [N][M][re, im])."""
-    g = torch.Generator(device="cuda")
-    g.manual_seed(seed)
+# ------------------------------------------------------------------ seeded workloads
+def haar(torch, g, n, m, cplx):
+    """n x m with orthonormal columns, Haar distributed: QR of a Gaussian, columns scaled by the phases of diag(R)."""
+    a = torch.randn((n, m), generator=g, device="cuda", dtype=torch.float64)
+    if cplx:
+        a = torch.complex(a, torch.randn((n, m), generator=g, device="cuda", dtype=torch.float64))
+    q, r = torch.linalg.qr(a)
+    d = torch.diagonal(r)
+    return q * (d / d.abs())
+
+
+def spread(torch, g, W, M, cplx, out, scale_cols=None, noise=0.0):
+    """out[j, :] (column j of the M x N result, column-major) = column j of D2 H [D1 W; 0] / sqrt(M) (+ noise), W N x N."""
+    N = W.shape[0]
+    if cplx:
+        ph = torch.rand(N, generator=g, device="cuda", dtype=torch.float64) * (2 * math.pi)
+        d1 = torch.polar(torch.ones_like(ph), ph)
+        ph2 = torch.rand(M, generator=g, device="cuda", dtype=torch.float64) * (2 * math.pi)
+        d2 = torch.polar(torch.ones_like(ph2), ph2)
+    else:
+        d1 = (torch.randint(0, 2, (N,), generator=g, device="cuda") * 2 - 1).to(torch.float64)
+        d2 = (torch.randint(0, 2, (M,), generator=g, device="cuda") * 2 - 1).to(torch.float64)
+    Wd = (d1[:, None] * W).T.contiguous()                     # [column j][row i] of D1 W
+    slab = max(1, min(N, (1 << 27) // M))                      # columns per transform: 2 GB of complex128 at most
+    inv = 1.0 / math.sqrt(M)
+    for j in range(0, N, slab):
+        x = torch.zeros((min(slab, N - j), M), device="cuda", dtype=torch.complex128)
+        x[:, :N] = Wd[j:j + slab]
+        y = torch.fft.fft(x, dim=1)
+        a = (y if cplx else (y.real - y.imag)) * inv * d2[None, :]
+        if scale_cols is not None:
+            a = a * scale_cols[j:j + slab, None]
+        if noise:
+            nz = torch.randn(a.shape, generator=g, device="cuda", dtype=torch.float64)
+            if cplx:
+                nz = torch.complex(nz, torch.randn(a.shape, generator=g, device="cuda", dtype=torch.float64))
+            a = a + noise * nz
+        out[j:j + slab] = torch.view_as_real(a) if cplx else a
+        del x, y, a
+
+
+def low_rank_half(torch, g, M, N, rank, noise):
+    """Configuration 4: L R with entries complex N(0, 1 / 256) plus complex Gaussian noise, cast to half; [N][M][re, im]."""
     s = (1.0 / 512.0) ** 0.5                                   # real and imaginary part: variance 1 / 512 each
     Lt = torch.view_as_complex(torch.randn((rank, M, 2), generator=g, device="cuda", dtype=torch.float32) * s)   # L^T
     Rt = torch.view_as_complex(torch.randn((N, rank, 2), generator=g, device="cuda", dtype=torch.float32) * s)   # R^T
@@ -55,57 +102,65 @@ def synth_low_rank(torch, M, N, rank, noise, seed):
     return out
 
 
-def synth(torch, at, M, N, seed):
-    """Column-scaled Gaussian test matrix generated on the device, column-major M x N."""
+def make_workload(torch, name):
+    """Returns (tensor as the configuration stores it, lda).  opA = 'N': column-major M x N, tensor [N][M](, 2);
+    opA = 'T' / 'C': the stored N x M matrix, tensor [M][N](, 2) (conjugated for 'C', so that op(stored) = A)."""
+    num, at, opA, M, N, K, eps, alg, fit, desc = WORKLOADS[name]
     g = torch.Generator(device="cuda")
-    g.manual_seed(seed)
-    real = torch.float64 if at in (0, 1) else torch.float32
-    comps = 2 if at & 1 else 1
-    decades = 2.0 if at in (4, 5) else 8.0          # FP16 storage holds five decades in all
-    scale = torch.pow(10.0, -torch.arange(N, device="cuda", dtype=torch.float64) * (decades / N)).to(real)
-    A = torch.randn((N, M, comps), generator=g, device="cuda", dtype=real)
-    A.mul_(scale[:, None, None])
-    return A.half().contiguous() if at in (4, 5) else A.contiguous()
+    g.manual_seed(SEED0 + num)
+    cplx = at & 1
+    i = torch.arange(N, device="cuda", dtype=torch.float64)
+    if name == "cfg4":
+        A = low_rank_half(torch, g, M, N, 256, 1e-4)
+    else:
+        s = {"cfg1": 10.0 ** (-i / 16.0), "cfg2": 2.0 ** (-i / 32.0), "cfg3": 10.0 ** (-i / 128.0), "cfg5": 10.0 ** (-i / 256.0), "target": 10.0 ** (-i / 128.0)}[name]
+        noise = {"cfg2": 1e-7, "cfg3": 1e-14, "target": 1e-14}.get(name, 0.0)
+        V = haar(torch, g, N, N, cplx)
+        W = s[:, None] * V.conj().T                             # diag(s) V^H
+        scale = None
+        if name == "cfg5":
+            scale = 10.0 ** (torch.rand(N, generator=g, device="cuda", dtype=torch.float64) * 12.0 - 6.0)
+        out = torch.empty((N, M, 2) if cplx else (N, M), device="cuda", dtype=torch.float64)
+        if name == "cfg1":                                      # small enough for a Haar U as well
+            U = haar(torch, g, M, N, cplx)
+            out.copy_((U @ W).T)
+        else:
+            spread(torch, g, W, M, cplx, out, scale, noise)
+        A = out.float() if at in (2, 3) else out
+        del out
+    if opA == "N":
+        return A.contiguous(), M
+    St = A.transpose(0, 1).contiguous()                         # [M][N]: row k of op(A) contiguous = the stored N x M matrix
+    if opA == "C":
+        St[..., 1].neg_()
+    return St, N
 
 
-def algorithmic_ops(alg, order, cplx, M, N):
-    if alg == "C":
-        if not cplx:
-            return order * M * N * (N + 1)
-        return min(order, 20) * 2 * M * N * N + max(order - 20, 0) * (M * N * (N + 1) + 2 * M * N * N)
-    ops = order * M * N * (N + 1) + order * (order - 1) * M * N * N
-    return ops + (order * order * 2 * M * N * N if cplx else 0)
-
-
-def cpu_baseline(at, M, N, eps, alg, order, u, sample_rows):
-    """The oracle's quantize + int8 Gram + reconstruction on the first sample_rows rows, all host cores."""
+def cpu_baseline(Ahost, at, alg, order, u):
+    """The oracle's quantize + int8 Gram + reconstruction on a row sample of the workload, all host cores."""
     import numpy as np
     from oracle import ho
-    rng = np.random.default_rng(3)
+    rows, N = Ahost.shape[0], Ahost.shape[1]
     cplx = at & 1
-    A = rng.standard_normal((sample_rows, N)) * 10.0 ** (-np.arange(N) / (N / 8.0))
-    if cplx:
-        A = A + 1j * rng.standard_normal((sample_rows, N)) * 10.0 ** (-np.arange(N) / (N / 8.0))
-    A = A.astype({0: np.float64, 1: np.complex128, 2: np.float32, 3: np.complex64}[at])
     ho.build()
     t0 = time.perf_counter()
-    vexp = ho.quantize_scale_batch(A, 1, sample_rows, sample_rows, u)
+    vexp = ho.quantize_scale_batch(Ahost, 1, rows, rows, u)
     kind = "crt" if alg == "C" else "limbs"
-    K = (sample_rows + 127) // 128 * 128
-    panels = ho.quantize(kind, A, order, vexp, ldb=K)
+    K = (rows + 127) // 128 * 128
+    panels = ho.quantize(kind, Ahost, order, vexp, ldb=K)
     ho.i8herk(kind, cplx, N, order, panels, 0, 2)
     dt = time.perf_counter() - t0
-    feff = sample_rows * N * (N + 1) * (4 if cplx else 1)
+    feff = rows * N * (N + 1) * (4 if cplx else 1)
     threads = int(os.environ.get("OMP_NUM_THREADS") or len(os.sched_getaffinity(0)))   # what the OpenMP loops of the oracle run on
     out = {"value": feff / dt / 1e12, "unit": "TFLOP/s (FP-equivalent Gram flops)", "cores": threads, "kind": "port",
-           "sample": "first %d of %d rows (int8 work is linear in rows), %s order %d, %.2f s" % (sample_rows, M, kind, order, dt)}
+           "sample": "first %d rows of the workload (int8 work is linear in rows), %s order %d, %.2f s" % (rows, kind, order, dt)}
     try:   # FP reference: SYRK / HERK from the BLAS scipy ships, on the same sample
         from scipy.linalg import blas
+        wide = Ahost[..., 0].astype(np.float64) + 1j * Ahost[..., 1].astype(np.float64) if Ahost.ndim == 3 else Ahost.astype(np.complex128 if cplx else np.float64)
         t0 = time.perf_counter()
-        G = (blas.zherk if cplx else blas.dsyrk)(1.0, np.asfortranarray(A.astype(np.complex128 if cplx else np.float64)), trans=2 if cplx else 1)
+        G = (blas.zherk if cplx else blas.dsyrk)(1.0, np.asfortranarray(wide), trans=2 if cplx else 1)
         out["fp_blas_tflops"] = feff / (time.perf_counter() - t0) / 1e12
-        # eigenvalues of the N x N Gram with LAPACK's divide and conquer: the FP counterpart of the fit's tail
-        from scipy.linalg import lapack
+        from scipy.linalg import lapack   # eigenvalues of the N x N Gram with LAPACK's divide and conquer: the FP counterpart of the fit's tail
         t0 = time.perf_counter()
         (lapack.zheevd if cplx else lapack.dsyevd)(G, compute_v=1, lower=0)
         out["fp_lapack_syevd_ms"] = (time.perf_counter() - t0) * 1e3
@@ -115,16 +170,79 @@ def cpu_baseline(at, M, N, eps, alg, order, u, sample_rows):
     return out
 
 
+# ------------------------------------------------------------------ board telemetry
+class Telemetry:
+    """Samples board power (hwmon power1_input / power1_average, microwatts) and the shader clock (the starred line of
+    pp_dpm_sclk) every few milliseconds while `running`."""
+    def __init__(self):
+        hw = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*"))
+        self.power = next((p for d in hw for p in (d + "/power1_input", d + "/power1_average") if os.access(p, os.R_OK)), None)
+        self.cap = next((p for d in hw for p in (d + "/power1_cap",) if os.access(p, os.R_OK)), None)
+        self.sclk = next((p for p in sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk")) if os.access(p, os.R_OK)), None)
+        self.watts, self.mhz, self.running = [], [], False
+
+    def _read(self, path):
+        try:
+            with open(path) as f:
+                return f.read()
+        except OSError:
+            return None
+
+    def _loop(self):
+        while self.running:
+            t = self._read(self.power) if self.power else None
+            if t:
+                self.watts.append(int(t) / 1e6)
+            t = self._read(self.sclk) if self.sclk else None
+            if t:
+                m = re.search(r"(\d+)\s*[Mm][Hh]z\s*\*", t)
+                if m:
+                    self.mhz.append(int(m.group(1)))
+            time.sleep(0.005)
+
+    def __enter__(self):
+        self.running = True
+        self.thread = threading.Thread(target=self._loop, daemon=True)
+        self.thread.start()
+        return self
+
+    def __exit__(self, *a):
+        self.running = False
+        self.thread.join()
+
+    def summary(self):
+        cap = self._read(self.cap) if self.cap else None
+        w = sorted(self.watts)
+        return {"power_w": (sum(w) / len(w)) if w else None, "power_w_max": w[-1] if w else None, "power_samples": len(w),
+                "power_cap_w": int(cap) / 1e6 if cap else None,
+                "sclk_mhz_sysfs": (sum(self.mhz) / len(self.mhz)) if self.mhz else None}
+
+
+def measured_traffic(workload):
+    """HBM bytes per launch of the contraction kernel from the rocprofv3 counter summary under profiles/, if that summary was
+    made from the kernel source as it is now (it records the SHA-256 of gram_mfma.hip); None otherwise."""
+    path = os.path.join(ROOT, "profiles", "gram_ring_kernel_%s_hbm_traffic.md" % workload)
+    try:
+        txt = open(path).read()
+        src = hashlib.sha256(open(os.path.join(ROOT, "hyacinth_amd", "csrc", "gram_mfma.hip"), "rb").read()).hexdigest()
+        m, h = re.search(r"traffic_bytes_per_launch:\s*([0-9.eE+]+)", txt), re.search(r"kernel_source_sha256:\s*([0-9a-f]{64})", txt)
+        if m and h and h.group(1) == src:
+            return float(m.group(1))
+    except OSError:
+        pass
+    return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=5)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="target", choices=sorted(WORKLOADS))
-    ap.add_argument("--no-fit", action="store_true", help="skip the end-to-end hyacinTsvdFit timing")
+    ap.add_argument("--no-fit", action="store_true", help="skip the end-to-end fit timing")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-stages", action="store_true", help="skip the separate timing of the HBM-bound stages (exponents, quantize, dequantize)")
-    ap.add_argument("--no-ceiling", action="store_true", help="skip the register-only MFMA ceiling measurement")
+    ap.add_argument("--no-ceiling", action="store_true", help="skip the register-only MFMA ceiling and the power / clock sampling")
     ap.add_argument("--cpu-rows", type=int, default=65536, help="rows of the workload the CPU baseline is timed on (about 15 s of host work)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="before the timed region, run three plain 1 GiB -> 1 GiB device copies (copy_kernel): the known-size reference for HBM traffic counters")
@@ -138,14 +256,14 @@ def main():
     import hyacinth_amd as ha
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     L = ha.lib()
-    at, opA, M, N, K, eps, alg, desc = WORKLOADS[a.workload]
+    num, at, opA, M, N, K, eps, alg, fit_name, desc = WORKLOADS[a.workload]
     if a.slab >= 0:
         assert L.hykGramSetSlab(a.slab) == 0
     stream = torch.cuda.current_stream().cuda_stream
     h = ha.create_handle(stream=stream, GramMatrixAlgorithm=alg)
     cplx = at & 1
-    A = synth_low_rank(torch, M, N, 256, 1e-4, 0x4859) if a.workload == "cfg4" else synth(torch, at, M, N, 0x4859)          # stored column-major M x N; opA='T' workloads are benchmarked on the transposed copy the fit makes
-    lda = M
+    A, lda = make_workload(torch, a.workload)
+    op = opA.encode()
     u, cP, lP, stride = ha.herk_batch_init(h, eps, M, N, at)
     seg = min(h.GramSegmentK, M) if h.GramSegmentK > 0 else M
     batches, lastM = (M + seg - 1) // seg, M - (M - 1) // seg * seg
@@ -154,8 +272,8 @@ def main():
     pA, pV, pC = C.c_void_p(A.data_ptr()), C.c_void_p(vexp.data_ptr()), C.c_void_p(Cq.data_ptr())
 
     def step():
-        L.hyacinXquantizeScaleBatch(C.byref(h), batches, seg, lastM, N, at, pA, lda, u, pV)
-        L.hyacinXherkBatch(C.byref(h), batches, seg, lastM, N, at, pA, lda, u, pV, 0, lP, pC)
+        L.hykQuantizeScaleBatchOp(C.byref(h), op, batches, seg, lastM, N, at, pA, lda, u, pV)
+        L.hykHerkBatchOp(C.byref(h), op, batches, seg, lastM, N, at, pA, lda, u, pV, 0, lP, pC)
 
     if a.copy_calibration:
         src = torch.ones(2 ** 27, dtype=torch.float64, device="cuda")
@@ -177,22 +295,32 @@ def main():
     kms, kn = C.c_double(), C.c_int32()
     L.hykGramProfileRead(C.byref(kms), C.byref(kn))
     L.hykGramProfile(0)
+    assert L.hykLastStatus() == 0, "the Gram stage reported a failure"
 
-    # the plan the library followed (same planner, host side)
-    from oracle import ho
-    plan_alg, order, plan_rows = ho.gram_algorithm(alg.decode(), M if batches <= 1 else M, u + cplx, cplx, h.TCGemmTargetK, h.StrideBatchPerfPenalty)
-    ops = algorithmic_ops(plan_alg, order, cplx, M, N)
+    plan = ha.HerkPlan()                              # what the library planned and issued in the last step
+    assert L.hykLastHerkPlan(C.byref(plan)) == 0
+    plan_alg, order, plan_rows, ops = chr(plan.algorithm), plan.order, plan.chunkRows, plan.int8Ops
     feff = M * N * (N + 1) * (4 if cplx else 1)
     launches_per_step = max(1, kn.value // a.steps)
     t_kernel = kms.value / 1e3 / a.steps            # contraction kernel time per step
     achieved = ops / t_kernel / 1e12 if t_kernel > 0 else 0.0
 
-    ceiling = None
-    if not a.no_ceiling:   # what a register-only MFMA loop sustains on this device with random operands (power-limited clock)
+    ceiling, board = None, None
+    if not a.no_ceiling:
+        # what a register-only MFMA loop sustains on this device with random operands (power-limited clock)
         tops, ghz = C.c_double(), C.c_double()
         if L.hykMfmaCeiling(stream, h.DeviceSMs, 20000, 1, C.byref(tops), C.byref(ghz)) == 0:
             ceiling = {"value": tops.value, "unit": "TFLOP/s", "clock_ghz": ghz.value,
                        "what": "register-only v_mfma_i32_32x32x32_i8 loop, random int8 operands, one workgroup of 4 waves per CU"}
+        # board power and clock while the Gram stage runs back to back for about a second (outside the timed region)
+        with Telemetry() as tel:
+            t1 = time.perf_counter()
+            while time.perf_counter() - t1 < 1.0:
+                for _ in range(10):
+                    step()
+                torch.cuda.synchronize()
+        board = tel.summary()
+        board["what"] = "hwmon power and pp_dpm_sclk sampled every 5 ms while the Gram stage (exponents, quantization, contraction, reconstruction) runs back to back for 1 s"
 
     # HBM-bound stages on their own (HIP events on the launch stream, outside the timed region): algorithmic bytes / time
     def timed_ms(fn, reps=3):
@@ -206,9 +334,9 @@ def main():
     eb = {0: 8, 1: 16, 2: 4, 3: 8, 4: 2, 5: 4}[at]
     stages = {}
     if not a.no_stages:
-        t = timed_ms(lambda: L.hyacinXquantizeScaleBatch(C.byref(h), batches, seg, lastM, N, at, pA, lda, u, pV))
+        t = timed_ms(lambda: L.hykQuantizeScaleBatchOp(C.byref(h), op, batches, seg, lastM, N, at, pA, lda, u, pV))
         stages["column_exponents"] = {"ms": t, "bytes": M * N * eb, "GB/s": M * N * eb / t / 1e6, "frac_of_hbm_peak": M * N * eb / t / 1e6 / HBM_PEAK_GBS}
-        rows = min(M, plan_rows) if plan_alg == "C" and plan_rows > 0 else M   # the rows the library quantizes per call (one residue chunk, or all)
+        rows = min(M, plan_rows) if plan_rows > 0 else M   # the rows the library quantizes per contraction call
         if plan_alg == "C":
             npan = 2 * min(order, 20) + 3 * max(order - 20, 0) if cplx else order
         else:
@@ -218,9 +346,9 @@ def main():
         panels = torch.empty(npan * N * ldb, dtype=torch.int8, device="cuda")
         pB = C.c_void_p(panels.data_ptr())
         if plan_alg == "C":
-            quant = lambda: L.hykQuantizeCrt(stream, rows, N, order, at, pA, lda, pV, pB, ldb, u + cplx)
+            quant = lambda: L.hykQuantizeCrtOp(stream, op, rows, N, order, at, pA, lda, pV, pB, ldb, u + 1)   # u + 1: the bound the library passes
         else:
-            quant = lambda: L.hykQuantizeLimbs(stream, rows, N, order, at, pA, lda, pV, pB, ldb)
+            quant = lambda: L.hykQuantizeLimbsOp(stream, op, rows, N, order, at, pA, lda, pV, pB, ldb)
         assert quant() == 0
         t = timed_ms(quant)
         qbytes = rows * N * eb + npan * rows * N
@@ -234,38 +362,60 @@ def main():
         stages["dequantize"] = {"ms": t, "bytes": dbytes, "GB/s": dbytes / t / 1e6, "frac_of_hbm_peak": dbytes / t / 1e6 / HBM_PEAK_GBS}
         del G
 
-    fit_ms = None
+    fit_ms, fit_rank = None, None
     if not a.no_fit:
-        S = torch.zeros(K, dtype=torch.float64, device="cuda")
-        V = torch.zeros(N * K * (2 if cplx else 1), dtype=torch.float64 if at in (0, 1) else torch.float32, device="cuda")
+        real = torch.float64 if at in (0, 1) else (torch.float32 if at in (2, 3) else torch.float16)
+        S = torch.zeros(max(K, N), dtype=torch.float64, device="cuda")      # singular values, or the pivot vector of the interpolation
+        V = torch.zeros(N * K * (2 if cplx else 1), dtype=real, device="cuda")
+        fit = getattr(L, fit_name)
         times = []
-        for i in range(3):
+        for i in range(7):
             torch.cuda.synchronize()
             t1 = time.perf_counter()
-            rank = L.hyacinTsvdFit(C.byref(h), eps, b"N", M, N, K, pA, lda, C.c_void_p(S.data_ptr()), C.c_void_p(V.data_ptr()), N, 0, at)
+            fit_rank = fit(C.byref(h), eps, op, M, N, K, pA, lda, C.c_void_p(S.data_ptr()), C.c_void_p(V.data_ptr()), N, 0, at)
             torch.cuda.synchronize()
             times.append((time.perf_counter() - t1) * 1e3)
-        fit_ms = sorted(times[1:])[len(times[1:]) // 2]
+        assert L.hykLastStatus() == 0, "the fit reported a failure"
+        fit_ms = sorted(times[2:])[len(times[2:]) // 2]
 
+    roofline = {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s", "frac": achieved / INT8_PEAK_TOPS,
+                "traffic": measured_traffic(a.workload) if a.slab <= 0 else None,
+                "kernel": "gram_ring_kernel" if a.slab <= 0 else ("gram_dma_kernel" if a.slab == 2 else "gram_kernel<%d>" % a.slab),
+                "ops": "int8 multiply-adds x2, upper triangle only, as reported by the library for the calls it issued",
+                "launches_per_step": launches_per_step, "avg_launch_ms": kms.value / max(1, kn.value), "algorithmic_ops_per_step": ops,
+                "sustained_mfma_ceiling": ceiling}
+    if ceiling:
+        roofline["frac_of_sustained_ceiling"] = achieved / ceiling["value"]
+        roofline["clock_ghz"] = ceiling["clock_ghz"]
+    if board:
+        roofline.update({k: board[k] for k in ("power_w", "power_w_max", "power_cap_w", "sclk_mhz_sysfs")})
+        roofline["power_note"] = board["what"]
     out = {
         "metric": "Gram-build effective TFLOPS (+ % INT8 MFMA peak; hyacinTsvdFit wall ms)",
         "value": feff / dt / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-        "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8 (i32 accumulate)", "data": "synthetic",
-        "config": {"workload": "%s: %s" % (a.workload, desc), "M": M, "N": N, "eps": eps, "algorithm": plan_alg, "order": order,
-                   "quant_bits": u, "gram_limbs": lP, "row_slices": batches},
+        "ms_per_step": dt * 1e3, "higher_is_better": True, "scaling": "none (one GPU)", "vs_baseline": None,
+        "dtype": "int8 (i32 accumulate)", "data": "synthetic (seeded recipe of the configuration, seed 0x%X)" % (SEED0 + num),
+        "config": {"workload": "%s: %s" % (a.workload, desc), "M": M, "N": N, "opA": opA, "eps": eps, "algorithm": plan_alg, "order": order,
+                   "quant_bits": u, "gram_limbs": lP, "row_slices": batches, "rows_per_contraction": plan_rows, "contraction_calls": plan.gramCalls},
         "pct_int8_mfma_peak": 100.0 * achieved / INT8_PEAK_TOPS,
-        "tsvd_fit_ms": fit_ms,
+        "tsvd_fit_ms": fit_ms, "fit": {"call": fit_name, "K": K, "rank": fit_rank, "ms": fit_ms, "timing": "median of 5 after 2 warm-ups"},
         "hbm_stages": stages,
-        "roofline": {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s", "frac": achieved / INT8_PEAK_TOPS,
-                     "traffic": MEASURED_TRAFFIC.get((a.workload, max(a.slab, 0))),
-                     "kernel": "gram_ring_kernel" if a.slab <= 0 else ("gram_dma_kernel" if a.slab == 2 else "gram_kernel<%d>" % a.slab), "ops": "int8 multiply-adds x2, upper triangle only", "launches_per_step": launches_per_step,
-                     "avg_launch_ms": kms.value / max(1, kn.value), "algorithmic_ops_per_step": ops,
-                     "sustained_mfma_ceiling": ceiling},
+        "roofline": roofline,
     }
     if not a.no_cpu:
         rows = min(a.cpu_rows, M)
-        out["cpu_baseline"] = cpu_baseline(at, M, N, eps, plan_alg, order, u, rows)
+        if opA == "N":
+            sample = A[:, :rows].transpose(0, 1).contiguous().cpu().numpy()
+        else:
+            sample = A[:rows].clone()
+            if opA == "C":
+                sample[..., 1].neg_()
+            sample = sample.cpu().numpy()
+        if cplx and at != 5:
+            import numpy as np
+            sample = sample[..., 0] + 1j * sample[..., 1]
+            sample = sample.astype(np.complex128 if at == 1 else np.complex64)
+        out["cpu_baseline"] = cpu_baseline(sample, at, plan_alg, order, u)
     ha.destroy_handle(h)
     print(json.dumps(out))
 

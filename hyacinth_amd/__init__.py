@@ -31,7 +31,7 @@ API_SYMBOLS = [
 KERNEL_SYMBOLS = [
     "hykColumnExponents", "hykSliceRange", "hykQuantizeLimbs", "hykQuantizeCrt", "hykZeroRows",
     "hykGramWorkspaceBytes", "hykGramWorkspaceClear", "hykGramCrt", "hykGramLimbs", "hykGramSetSlab",
-    "hykGramProfile", "hykGramProfileRead", "hykMfmaCeiling", "hykGramRange", "hykDequantize", "hykPotrfpWorkspaceBytes", "hykPotrfp", "hykPotrfpLeftLooking", "hykPotrfpStaticMaxN", "hykPotrfpStatic", "hykFactorToB", "hykJacobiSweep", "hykJacobiSweepCarry", "hykJacobiCarryBytes", "hykJacobiSetVariant",
+    "hykGramProfile", "hykGramProfileRead", "hykMfmaCeiling", "hykGramRange", "hykDequantize", "hykPotrfpWorkspaceBytes", "hykPotrfp", "hykPotrfpLeftLooking", "hykPotrfpStaticMaxN", "hykPotrfpStatic", "hykFactorToB", "hykJacobiSweep", "hykJacobiSweepCarry", "hykJacobiSweepTop", "hykJacobiCarryBytes", "hykJacobiSetVariant",
     "hykColumnNorms", "hykBasisOut", "hykValuesOut", "hykInterpSolve", "hykInterpOut", "hykMatcopy",
     "hykSumSquares", "hykMatmulCf16", "hykGemm", "hykOrthonormalize", "hykLastStatus", "hykTestFailAllocation", "hykColumnExponentsOp", "hykQuantizeLimbsOp", "hykQuantizeCrtOp",
     "hykQuantizeScaleBatchOp", "hykHerkBatchOp", "hykLastHerkPlan",
@@ -97,6 +97,7 @@ def lib():
         L.hykJacobiSetVariant.argtypes = [i32]
         L.hykJacobiSweep.argtypes = [vp, i32, i32, i32, vp, dbl, vp]
         L.hykJacobiSweepCarry.argtypes = [vp, i32, i32, i32, vp, dbl, vp, vp]
+        L.hykJacobiSweepTop.argtypes = [vp, i32, i32, i32, i32, i32, vp, dbl, vp, vp]
         L.hykJacobiCarryBytes.argtypes = [i32]; L.hykJacobiCarryBytes.restype = C.c_size_t
         L.hykGramProfile.argtypes = [i32]
         L.hykGramProfileRead.argtypes = [C.POINTER(dbl), C.POINTER(i32)]

@@ -7,6 +7,8 @@
 #pragma once
 #include <algorithm>
 #include <cmath>
+#include <functional>
+#include <vector>
 
 namespace hyh {
 
@@ -24,6 +26,31 @@ inline bool jacobi_sweeps_done(int rotations, double cosine2, double lastCosine2
     if (contraction <= 16. && contraction * cosine2 <= 8. * rotateAbove) { return true; }
   }
   return false;
+}
+
+/* A second way for the sweeps to end: what is handed out has stopped moving.
+ * Only the `kept` largest singular values and their vectors leave the library (K of them at most, and none below the rank
+ * cut), the values to an absolute accuracy of a few eps sigma_max and the vectors through the projection residual
+ * |A - A V V^H|, whose square is at most the sum of the squared norms of the columns that are not handed out, whatever
+ * state those are in (the columns of B stay an orthogonal transform of the factor).  A cyclic sweep changes a column's squared
+ * norm by the sum of the eigenvalue shifts of its 2 x 2 rotations, which is, to first order, how far that norm still is from
+ * its singular value squared.  So the iteration may end after a sweep in which
+ *   (i)  no kept value moved by more than eps sigma_max / 4, and
+ *   (ii) the kept columns gained at most 1 / 32 of what is left outside them (the residual bound has stopped improving).
+ * A noise floor of hundreds of nearly equal small columns, which a cyclic Jacobi method needs ten and more sweeps to resolve
+ * and which is never handed out, then no longer decides when the sweeps end.  With nothing left outside (kept = all columns
+ * and a zero cut) rule (ii) never holds and the rules above decide alone.
+ * before / after: the column norms (not squared) at the start and at the end of the sweep, in the same column order. */
+inline bool jacobi_output_settled(const std::vector<double>& before, const std::vector<double>& after, int kept, double eps) {
+  const size_t r = after.size(); if (before.size() != r || r == 0 || kept <= 0 || (size_t)kept >= r) { return false; }
+  std::vector<double> a(before), b(after);
+  std::sort(a.begin(), a.end(), std::greater<double>()); std::sort(b.begin(), b.end(), std::greater<double>());
+  double moved = 0.; for (int i = 0; i < kept; ++i) { moved = std::max(moved, std::fabs(b[(size_t)i] - a[(size_t)i])); }
+  if (!(moved <= 0.25 * eps * b[0])) { return false; }
+  double outsideBefore = 0., outsideAfter = 0.;   /* summed from the small end: no cancellation against the large values */
+  for (size_t i = r; i-- > (size_t)kept;) { outsideBefore += a[i] * a[i]; outsideAfter += b[i] * b[i]; }
+  const double gained = outsideBefore - outsideAfter;
+  return gained <= outsideAfter / 32.;
 }
 
 }  // namespace hyh

@@ -85,15 +85,24 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
      * cosines of that size move a singular value by less than eps / 2 of the largest one. */
     const double rotateAbove = std::max(std::max(machineEps, std::sqrt((double)N) * 2.220446049250313e-16), eps / 16.);
     double lastCosine2 = 0.;
+    std::vector<double> before((size_t)rank), after((size_t)rank);
+    auto fetch_norms = [&](std::vector<double>& v) {
+      HYH_KERNEL(hykColumnNorms(s, Complex, N, rank, B.as<double>(), sigma.as<double>()));
+      HYH_CHECK(hipMemcpyAsync(v.data(), sigma.p, sizeof(double) * (size_t)rank, hipMemcpyDeviceToHost, s));
+    };
+    const bool watchOutput = K < rank;   /* with every column handed out only the cosines can end the sweeps */
+    if (watchOutput && rank > 1) { fetch_norms(before); }
     for (int32_t sw = 0; sw < maxSweeps && rank > 1; ++sw) {
       HYH_KERNEL(hykGramWorkspaceClear(s, counter.p, 64));
       HYH_KERNEL(hykJacobiSweepCarry(s, Complex, N, rank, B.as<double>(), rotateAbove, counter.as<int32_t>(), carry.as<double>())); ++used;
+      if (watchOutput) { fetch_norms(after); }
       struct { int32_t rotations, pad; double cosine2; } seen = { 0, 0, 0. };
       HYH_CHECK(hipMemcpyAsync(&seen, counter.p, sizeof(seen), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
       if (!hyh::ok()) { return 0; }
       if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: %d rotations, largest cosine %.2le\n", used, seen.rotations, std::sqrt(seen.cosine2)); }
       if (hyh::jacobi_sweeps_done(seen.rotations, seen.cosine2, lastCosine2, rotateAbove)) { break; }
-      lastCosine2 = seen.cosine2;
+      if (watchOutput && hyh::jacobi_output_settled(before, after, K, eps)) { if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ: the %d values handed out have settled\n", K); } break; }
+      lastCosine2 = seen.cosine2; before.swap(after);
     }
     HYH_KERNEL(hykColumnNorms(s, Complex, N, rank, B.as<double>(), sigma.as<double>()));
     std::vector<double> sig((size_t)rank); HYH_CHECK(hipMemcpyAsync(sig.data(), sigma.p, sizeof(double) * (size_t)rank, hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));

@@ -170,12 +170,13 @@ __device__ __forceinline__ double squared_cosine(double g2, double alpha, double
 }
 
 template <bool CPLX>
-__global__ __launch_bounds__(T_THREADS) void jacobi_round_kernel(int32_t N, int32_t n, int32_t r, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations) {
+__global__ __launch_bounds__(T_THREADS) void jacobi_round_kernel(int32_t N, int32_t n, int32_t r, int32_t head, int32_t top, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations) {
   __shared__ double scratch[T_THREADS / 64];
   const int i = blockIdx.x; int p, q;
   if (i == 0) { p = n - 1; q = round; } else { p = (round + i) % (n - 1); q = (round - i + (n - 1)) % (n - 1); }
   if (p >= r || q >= r) { return; }
   if (p > q) { int t = p; p = q; q = t; }
+  if (p >= top) { return; }                        /* both columns belong to the tail that is left alone */
   constexpr int W = CPLX ? 2 : 1;
   double* bp = &B[(int64_t)p * N * W]; double* bq = &B[(int64_t)q * N * W];
   double alpha = 0., beta = 0., gre = 0., gim = 0.;
@@ -187,7 +188,7 @@ __global__ __launch_bounds__(T_THREADS) void jacobi_round_kernel(int32_t N, int3
   }
   alpha = block_sum(alpha, scratch); beta = block_sum(beta, scratch); gre = block_sum(gre, scratch); if constexpr (CPLX) { gim = block_sum(gim, scratch); }
   const double g2 = gre * gre + gim * gim;
-  if (threadIdx.x == 0) { report_cosine(rotations, squared_cosine(g2, alpha, beta)); }
+  if (threadIdx.x == 0 && p < head) { report_cosine(rotations, squared_cosine(g2, alpha, beta)); }
   if (!(g2 > tol * tol * alpha * beta) || !(g2 > 0.)) { return; }
   const double gabs = sqrt(g2), zeta = (beta - alpha) / (2. * gabs);
   const double t = (zeta >= 0. ? 1. : -1.) / (fabs(zeta) + sqrt(1. + zeta * zeta)), cs = 1. / sqrt(1. + t * t), sn = cs * t;
@@ -247,7 +248,7 @@ __device__ __forceinline__ void block_sum_many(double (&v)[NV], double* red, int
 }
 
 template <bool CPLX, int ROWS, int BC, bool FULL, int THREADS>
-__global__ __launch_bounds__(THREADS) void jacobi_block_round_kernel(int32_t N, int32_t nb, int32_t r, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations) {
+__global__ __launch_bounds__(THREADS) void jacobi_block_round_kernel(int32_t N, int32_t nb, int32_t r, int32_t head, int32_t top, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations) {
   constexpr int W = CPLX ? 2 : 1, NC = 2 * BC, GV = BC * W;
   constexpr int HALF = (THREADS / 64) * (NC > GV ? NC : GV);
   __shared__ double red[2 * HALF];
@@ -257,7 +258,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_block_round_kernel(int32_t N, 
   int col[NC]; bool live[NC];
   #pragma unroll
   for (int c = 0; c < NC; ++c) { col[c] = (c < BC ? P : Q) * BC + (c % BC); live[c] = col[c] < r; }
-  if (!live[0]) { return; }                       /* both blocks beyond the last column */
+  if (!live[0] || col[0] >= top) { return; }      /* both blocks beyond the last column, or wholly in the tail that is left alone */
   /* rows of this thread */
   double x[NC][ROWS][W];
   #pragma unroll
@@ -305,15 +306,15 @@ __global__ __launch_bounds__(THREADS) void jacobi_block_round_kernel(int32_t N, 
     const int lane = threadIdx.x & 63;
     double gre = sum, gim = 0.;
     if constexpr (CPLX) { gre = __shfl(sum, 2 * lane, 64); gim = __shfl(sum, 2 * lane + 1, 64); }
-    double alpha = 0., beta = 0.; bool pairLive = false;
+    double alpha = 0., beta = 0.; bool pairLive = false, counted = false;
     #pragma unroll
     for (int j = 0; j < BC; ++j) {
       const int fa = (j == 0) ? NC - 1 : (step + j) % (NC - 1), fb = (j == 0) ? step : (step - j + (NC - 1)) % (NC - 1);
       const int c0 = FULL ? (fa < fb ? fa : fb) : j, c1 = FULL ? (fa < fb ? fb : fa) : BC + (j + step) % BC;
-      if (lane == j) { alpha = norm[c0]; beta = norm[c1]; pairLive = live[c0] && live[c1]; }
+      if (lane == j) { alpha = norm[c0]; beta = norm[c1]; pairLive = live[c0] && live[c1] && (col[c0] < top || col[c1] < top); counted = col[c0] < head || col[c1] < head; }
     }
     const double g2 = gre * gre + gim * gim;
-    if (pairLive) {                                /* worst = max(worst, squared_cosine(g2, alpha, beta)), dividing only where the maximum moves */
+    if (pairLive && counted) {                     /* worst = max(worst, squared_cosine(g2, alpha, beta)), dividing only where the maximum moves */
       const double ab = alpha * beta;
       if (ab > 0.) { if (g2 > worst * ab) { worst = g2 / ab; } } else if (g2 > 0.) { worst = fmax(worst, 1.); }
     }
@@ -409,7 +410,7 @@ template <int BC> __device__ __forceinline__ void carried_pair(int t, int& i, in
  * half, then of the second (which stays in registers), the steps, and the replay on the second half and then on the first,
  * loaded again: three loads and two stores of half the rows instead of one each of all, for blocks twice as wide. */
 template <int ROWS, int BC, bool FULL, int THREADS, bool CARRY, int PASSES>
-__global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, int32_t nb, int32_t r, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations, double* __restrict__ carry) {
+__global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, int32_t nb, int32_t r, int32_t head, int32_t top, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations, double* __restrict__ carry) {
   constexpr int NC = 2 * BC, NG = NC * (NC + 1) / 2, WAVES = THREADS / 64, STEPS = FULL ? NC - 1 : BC, GS = NC + 1;
   constexpr bool SLIM = CARRY && !FULL;                    /* norms and cross products only */
   constexpr int NW = BC * (BC - 1) / 2, NP = SLIM ? NC + BC * BC : NG;
@@ -435,6 +436,9 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
   #pragma unroll
   for (int c = 0; c < NC; ++c) { col[c] = (c < BC ? P : Q) * BC + (c % BC); live[c] = col[c] < r; }
   if (!live[0]) { return; }
+  /* Columns from `top` on are the tail that is left alone: pairs of two tail columns are not rotated.  A block pair wholly
+   * in the tail has nothing to do, except in the first round of a sweep, which also refreshes the carried products. */
+  if (!FULL && col[0] >= top) { return; }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   [[maybe_unused]] double carried = 0.;
   if constexpr (SLIM) { if (wave == 0 && lane < 2 * NW) { carried = carry[(int64_t)(lane < NW ? P : Q) * NW + lane % NW]; } }
@@ -504,9 +508,10 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
           c0 = fa < fb ? fa : fb; c1 = fa < fb ? fb : fa;
         } else { c0 = j; c1 = BC + (j + step) % BC; }
         const double alpha = Gs[c0 * GS + c0], beta = Gs[c1 * GS + c1], gre = Gs[c0 * GS + c1];
-        const bool pairLive = ((c0 < BC ? P : Q) * BC + (c0 % BC) < r) && ((c1 < BC ? P : Q) * BC + (c1 % BC) < r);
+        const int i0 = (c0 < BC ? P : Q) * BC + (c0 % BC), i1 = (c1 < BC ? P : Q) * BC + (c1 % BC);
+        const bool pairLive = i0 < r && i1 < r && (i0 < top || i1 < top), counted = i0 < head || i1 < head;
         const double g2 = gre * gre;
-        if (pairLive) {
+        if (pairLive && counted) {
           const double ab = alpha * beta;
           if (ab > 0.) { if (g2 > worst * ab) { worst = g2 / ab; } } else if (g2 > 0.) { worst = fmax(worst, 1.); }
         }
@@ -596,7 +601,7 @@ struct Cx { double re, im; };
 __device__ __forceinline__ Cx cmul(double ar, double ai, Cx b) { return Cx{ ar * b.re - ai * b.im, ar * b.im + ai * b.re }; }
 
 template <int ROWS, int BC, bool FULL, int THREADS, int PASSES, bool CARRY>
-__global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t N, int32_t nb, int32_t r, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations, double* __restrict__ carry) {
+__global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t N, int32_t nb, int32_t r, int32_t head, int32_t top, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations, double* __restrict__ carry) {
   constexpr int NC = 2 * BC, NG = NC * (NC + 1) / 2, NT = NC * NC, WAVES = THREADS / 64, STEPS = FULL ? NC - 1 : BC, GS = NC + 1;
   /* CARRY as in the real kernel: the products inside a block (real and imaginary part, 2 NW doubles per block) come from
    * the round before; summed are the NC norms and the BC^2 cross products (real parts, then imaginary parts) */
@@ -623,6 +628,9 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t
   #pragma unroll
   for (int c = 0; c < NC; ++c) { col[c] = (c < BC ? P : Q) * BC + (c % BC); live[c] = col[c] < r; }
   if (!live[0]) { return; }
+  /* Columns from `top` on are the tail that is left alone: pairs of two tail columns are not rotated.  A block pair wholly
+   * in the tail has nothing to do, except in the first round of a sweep, which also refreshes the carried products. */
+  if (!FULL && col[0] >= top) { return; }
   static_assert(PASSES == 1 || PASSES == 2, "all rows at once or in two halves (as in the real kernel)");
   double x[NC][ROWS][2];
   auto load_rows = [&](int pass) {
@@ -692,9 +700,10 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t
           c0 = fa < fb ? fa : fb; c1 = fa < fb ? fb : fa;
         } else { c0 = j; c1 = BC + (j + step) % BC; }
         const double alpha = Gre[c0 * GS + c0], beta = Gre[c1 * GS + c1], gre = Gre[c0 * GS + c1], gim = Gim[c0 * GS + c1];
-        const bool pairLive = ((c0 < BC ? P : Q) * BC + (c0 % BC) < r) && ((c1 < BC ? P : Q) * BC + (c1 % BC) < r);
+        const int i0 = (c0 < BC ? P : Q) * BC + (c0 % BC), i1 = (c1 < BC ? P : Q) * BC + (c1 % BC);
+        const bool pairLive = i0 < r && i1 < r && (i0 < top || i1 < top), counted = i0 < head || i1 < head;
         const double g2 = gre * gre + gim * gim;
-        if (pairLive) {
+        if (pairLive && counted) {
           const double ab = alpha * beta;
           if (ab > 0.) { if (g2 > worst * ab) { worst = g2 / ab; } } else if (g2 > 0.) { worst = fmax(worst, 1.); }
         }
@@ -882,36 +891,36 @@ extern "C" int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t
 static thread_local int g_jacobiVariant = 0;   /* 0: Gram-space rounds, 8-column blocks for real factors where they fit (default); 1: the step kernel everywhere; 2: Gram-space rounds, 4-column blocks */
 
 template <int ROWS, int BC, int THREADS = T_THREADS, int PASSES = 1>
-static int gram_sweep(hipStream_t stream, int32_t N, int32_t r, double* B, double tol, int32_t* rotations, double* carry) {
+static int gram_sweep(hipStream_t stream, int32_t N, int32_t r, int32_t head, int32_t top, double* B, double tol, int32_t* rotations, double* carry) {
   const int blocks = (r + BC - 1) / BC, nb = (blocks + 1) & ~1;
   if (carry) {
-    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations, carry);
-    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations, carry); }
+    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, tol, rotations, carry);
+    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, tol, rotations, carry); }
   } else {
-    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, false, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations, nullptr);
-    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, false, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations, nullptr); }
+    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, false, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, tol, rotations, nullptr);
+    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, false, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, tol, rotations, nullptr); }
   }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
 template <int ROWS, int BC, int THREADS = T_THREADS, int PASSES = 1>
-static int gram_sweep_cplx(hipStream_t stream, int32_t N, int32_t r, double* B, double tol, int32_t* rotations, double* carry) {
+static int gram_sweep_cplx(hipStream_t stream, int32_t N, int32_t r, int32_t head, int32_t top, double* B, double tol, int32_t* rotations, double* carry) {
   const int blocks = (r + BC - 1) / BC, nb = (blocks + 1) & ~1;
   if (carry) {
-    jacobi_gram_round_cplx_kernel<ROWS, BC, true, THREADS, PASSES, true><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations, carry);
-    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_cplx_kernel<ROWS, BC, false, THREADS, PASSES, true><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations, carry); }
+    jacobi_gram_round_cplx_kernel<ROWS, BC, true, THREADS, PASSES, true><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, tol, rotations, carry);
+    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_cplx_kernel<ROWS, BC, false, THREADS, PASSES, true><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, tol, rotations, carry); }
   } else {
-    jacobi_gram_round_cplx_kernel<ROWS, BC, true, THREADS, PASSES, false><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations, nullptr);
-    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_cplx_kernel<ROWS, BC, false, THREADS, PASSES, false><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations, nullptr); }
+    jacobi_gram_round_cplx_kernel<ROWS, BC, true, THREADS, PASSES, false><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, tol, rotations, nullptr);
+    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_cplx_kernel<ROWS, BC, false, THREADS, PASSES, false><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, tol, rotations, nullptr); }
   }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
 template <bool CPLX, int ROWS, int BC, int THREADS = T_THREADS>
-static int blocked_sweep(hipStream_t stream, int32_t N, int32_t r, double* B, double tol, int32_t* rotations) {
+static int blocked_sweep(hipStream_t stream, int32_t N, int32_t r, int32_t head, int32_t top, double* B, double tol, int32_t* rotations) {
   const int blocks = (r + BC - 1) / BC, nb = (blocks + 1) & ~1;
-  jacobi_block_round_kernel<CPLX, ROWS, BC, true, THREADS><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, 0, B, tol, rotations);
-  for (int round = 1; round < nb - 1; ++round) { jacobi_block_round_kernel<CPLX, ROWS, BC, false, THREADS><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, round, B, tol, rotations); }
+  jacobi_block_round_kernel<CPLX, ROWS, BC, true, THREADS><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, tol, rotations);
+  for (int round = 1; round < nb - 1; ++round) { jacobi_block_round_kernel<CPLX, ROWS, BC, false, THREADS><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, tol, rotations); }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
@@ -919,41 +928,44 @@ extern "C" int hykJacobiSetVariant(int32_t variant) { if (variant < 0 || variant
 
 extern "C" size_t hykJacobiCarryBytes(int32_t r) { return r <= 0 ? 0 : ((size_t)r / 4 + 2) * 28 * sizeof(double); }
 
-extern "C" int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations) { return hykJacobiSweepCarry(stream, Complex, N, r, B, tol, rotations, nullptr); }
+extern "C" int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations) { return hykJacobiSweepTop(stream, Complex, N, r, r, r, B, tol, rotations, nullptr); }
 
-extern "C" int hykJacobiSweepCarry(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations, double* carry) {
+extern "C" int hykJacobiSweepCarry(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations, double* carry) { return hykJacobiSweepTop(stream, Complex, N, r, r, r, B, tol, rotations, carry); }
+
+extern "C" int hykJacobiSweepTop(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, int32_t head, int32_t top, double* B, double tol, int32_t* rotations, double* carry) {
   if (N <= 0 || r <= 1) { return 0; }
+  if (top > r) { top = r; } if (top < 0) { top = 0; } if (head > r) { head = r; } if (head < 0) { head = 0; }
   /* blocked kernel when the rows of two column blocks fit the registers of a workgroup */
   /* real factors: Gram-space rounds; blocks of 8 columns where the rows of 16 columns fit the registers of 512 threads
    * (half as many rounds, each 1.4 times as long at N = 2048; up to 4096 rows in two halves), blocks of 4 otherwise */
   if (!Complex && r >= 32 && g_jacobiVariant == 0) {
-    if (N <= 2 * 512) { return gram_sweep<2, 8, 512>(stream, N, r, B, tol, rotations, carry); }
-    if (N <= 4 * 512) { return gram_sweep<4, 8, 512>(stream, N, r, B, tol, rotations, carry); }
-    if (N <= 8 * 512) { return gram_sweep<4, 8, 512, 2>(stream, N, r, B, tol, rotations, carry); }
+    if (N <= 2 * 512) { return gram_sweep<2, 8, 512>(stream, N, r, head, top, B, tol, rotations, carry); }
+    if (N <= 4 * 512) { return gram_sweep<4, 8, 512>(stream, N, r, head, top, B, tol, rotations, carry); }
+    if (N <= 8 * 512) { return gram_sweep<4, 8, 512, 2>(stream, N, r, head, top, B, tol, rotations, carry); }
   }
   if (!Complex && r >= 16 && g_jacobiVariant != 1) {
-    if (N <= 4 * T_THREADS) { return gram_sweep<4, 4>(stream, N, r, B, tol, rotations, carry); }
-    if (N <= 8 * T_THREADS) { return gram_sweep<8, 4>(stream, N, r, B, tol, rotations, carry); }
-    if (N <= 8 * 512) { return gram_sweep<8, 4, 512>(stream, N, r, B, tol, rotations, carry); }
+    if (N <= 4 * T_THREADS) { return gram_sweep<4, 4>(stream, N, r, head, top, B, tol, rotations, carry); }
+    if (N <= 8 * T_THREADS) { return gram_sweep<8, 4>(stream, N, r, head, top, B, tol, rotations, carry); }
+    if (N <= 8 * 512) { return gram_sweep<8, 4, 512>(stream, N, r, head, top, B, tol, rotations, carry); }
   }
   if (!Complex && r >= 16) {
-    if (N <= 4 * T_THREADS) { return blocked_sweep<false, 4, 4>(stream, N, r, B, tol, rotations); }
-    if (N <= 8 * T_THREADS) { return blocked_sweep<false, 8, 4>(stream, N, r, B, tol, rotations); }
-    if (N <= 8 * 512) { return blocked_sweep<false, 8, 4, 512>(stream, N, r, B, tol, rotations); }
+    if (N <= 4 * T_THREADS) { return blocked_sweep<false, 4, 4>(stream, N, r, head, top, B, tol, rotations); }
+    if (N <= 8 * T_THREADS) { return blocked_sweep<false, 8, 4>(stream, N, r, head, top, B, tol, rotations); }
+    if (N <= 8 * 512) { return blocked_sweep<false, 8, 4, 512>(stream, N, r, head, top, B, tol, rotations); }
   }
   if (Complex && r >= 16 && g_jacobiVariant != 1) {
-    if (N <= 4 * T_THREADS) { return gram_sweep_cplx<4, 4>(stream, N, r, B, tol, rotations, carry); }
-    if (N <= 4 * 512) { return gram_sweep_cplx<4, 4, 512>(stream, N, r, B, tol, rotations, carry); }
-    if (N <= 8 * 512) { return g_jacobiVariant == 0 ? gram_sweep_cplx<4, 4, 512, 2>(stream, N, r, B, tol, rotations, carry) : gram_sweep_cplx<8, 2, 512>(stream, N, r, B, tol, rotations, carry); }
+    if (N <= 4 * T_THREADS) { return gram_sweep_cplx<4, 4>(stream, N, r, head, top, B, tol, rotations, carry); }
+    if (N <= 4 * 512) { return gram_sweep_cplx<4, 4, 512>(stream, N, r, head, top, B, tol, rotations, carry); }
+    if (N <= 8 * 512) { return g_jacobiVariant == 0 ? gram_sweep_cplx<4, 4, 512, 2>(stream, N, r, head, top, B, tol, rotations, carry) : gram_sweep_cplx<8, 2, 512>(stream, N, r, head, top, B, tol, rotations, carry); }
   }
   if (Complex && r >= 16) {
-    if (N <= 4 * T_THREADS) { return blocked_sweep<true, 4, 4>(stream, N, r, B, tol, rotations); }
-    if (N <= 4 * 512) { return blocked_sweep<true, 4, 4, 512>(stream, N, r, B, tol, rotations); }
-    if (N <= 8 * 512) { return blocked_sweep<true, 8, 2, 512>(stream, N, r, B, tol, rotations); }
+    if (N <= 4 * T_THREADS) { return blocked_sweep<true, 4, 4>(stream, N, r, head, top, B, tol, rotations); }
+    if (N <= 4 * 512) { return blocked_sweep<true, 4, 4, 512>(stream, N, r, head, top, B, tol, rotations); }
+    if (N <= 8 * 512) { return blocked_sweep<true, 8, 2, 512>(stream, N, r, head, top, B, tol, rotations); }
   }
   const int n = (r + 1) & ~1;
   for (int round = 0; round < n - 1; ++round) {
-    if (Complex) { jacobi_round_kernel<true><<<n / 2, T_THREADS, 0, stream>>>(N, n, r, round, B, tol, rotations); } else { jacobi_round_kernel<false><<<n / 2, T_THREADS, 0, stream>>>(N, n, r, round, B, tol, rotations); }
+    if (Complex) { jacobi_round_kernel<true><<<n / 2, T_THREADS, 0, stream>>>(N, n, r, head, top, round, B, tol, rotations); } else { jacobi_round_kernel<false><<<n / 2, T_THREADS, 0, stream>>>(N, n, r, head, top, round, B, tol, rotations); }
   }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }

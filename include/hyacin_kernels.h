@@ -115,6 +115,11 @@ int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, do
  * column block from one round to the next instead of summing them again (ignored by the kernels of variant 1).  The memory needs no initialisation and holds nothing a later sweep relies on. */
 size_t hykJacobiCarryBytes(int32_t r);
 int hykJacobiSweepCarry(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations, double* carry);
+/* The same sweep with two index limits.  Pairs of two columns with index >= top are not rotated (block pairs wholly behind
+ * `top` are skipped); the largest cosine is reported over the pairs with at least one column before `head` only (the pairs
+ * whose convergence the caller waits for), while rotations[0] still counts every rotation.  head = top = r is the plain
+ * sweep.  carry may be null. */
+int hykJacobiSweepTop(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, int32_t head, int32_t top, double* B, double tol, int32_t* rotations, double* carry);
 /* Which kernel a sweep runs: 0 (default) one Gram matrix per round and workgroup, the steps of the round taken on it by
  * one wavefront; real factors in blocks of 8 columns, complex ones in blocks of 4, the rows in two halves where N > 2048;
  * 1 one reduction and barrier per step; 2 as 0 with the narrower blocks that hold all rows at once (4 columns for real

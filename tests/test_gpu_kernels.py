@@ -487,3 +487,52 @@ def test_jacobi_sweep_kernels(gl, variant, carry, cplx, N, r):
     assert np.max(np.abs(Un.conj().T @ Un - np.eye(r))) <= 16 * tol
     Qb, _ = np.linalg.qr(B)                                               # same column space
     assert np.linalg.norm(Un - Qb @ (Qb.conj().T @ Un)) <= 1e-9 * np.sqrt(r)
+
+
+@pytest.mark.parametrize("variant,carry", [(0, 1), (0, 0), (1, 0), (2, 1)])
+@pytest.mark.parametrize("cplx,N,r,head,top", [(0, 1000, 130, 37, 37), (0, 2048, 96, 40, 64), (1, 600, 50, 9, 9), (1, 2048, 40, 12, 20), (0, 700, 20, 5, 20), (0, 300, 40, 0, 0)])
+def test_jacobi_sweeps_with_limits(gl, variant, carry, cplx, N, r, head, top):
+    """hykJacobiSweepTop: pairs of two columns from `top` on are never rotated, and only the pairs with a column before
+    `head` are reported.  The columns behind `head` are 1e-5 of the others (the separation under which the host uses the
+    limits).  Sweeps run until the reported cosine is at the threshold's level; then the columns before `head` are
+    orthogonal to every other column, so the singular values are their norms together with those of the block behind
+    them, and the span is unchanged.  With head = top = r the sweep is the plain one, bit for bit."""
+    from gpu_util import dev, host, ptr, stream, sync, zeros
+    rng = np.random.default_rng(7000 + N + r + cplx)
+    B = rng.standard_normal((N, r)) + (1j * rng.standard_normal((N, r)) if cplx else 0)
+    B = (B @ (np.triu(rng.standard_normal((r, r))) * 0.1 + np.eye(r))) * 10.0 ** (-2.0 * np.arange(r) / r)
+    B[:, head:] *= 1e-5
+    want = np.linalg.svd(B, compute_uv=False)
+    tol = float(2.220446049250313e-16 * np.sqrt(N))
+    assert gl.L.hykJacobiSetVariant(variant) == 0
+    try:
+        dB = dev(np.ascontiguousarray(B.T)); counter = zeros(64)
+        carried = zeros(gl.L.hykJacobiCarryBytes(r)); carried.fill_(255)
+        for sweeps in range(30):
+            counter.zero_()
+            print("jacobi limits", variant, carry, cplx, N, r, head, top, "sweep", sweeps, flush=True)
+            assert gl.L.hykJacobiSweepTop(stream(), cplx, N, r, head, top, ptr(dB), tol, ptr(counter), ptr(carried) if carry else None) == 0
+            sync()
+            if float(host(counter, np.float64)[1]) <= (8 * tol) ** 2:
+                break
+        else:
+            raise AssertionError("no convergence")
+        # one plain sweep through both entry points: identical bits
+        d1, d2 = dev(np.ascontiguousarray(B.T)), dev(np.ascontiguousarray(B.T)); c1, c2 = zeros(64), zeros(64)
+        assert gl.L.hykJacobiSweep(stream(), cplx, N, r, ptr(d1), tol, ptr(c1)) == 0
+        assert gl.L.hykJacobiSweepTop(stream(), cplx, N, r, r, r, ptr(d2), tol, ptr(c2), None) == 0
+        sync()
+        assert np.array_equal(host(d1, np.uint8), host(d2, np.uint8)) and np.array_equal(host(c1, np.uint8), host(c2, np.uint8))
+    finally:
+        gl.L.hykJacobiSetVariant(0)
+    U = host(dB, np.complex128 if cplx else np.float64, (r, N)).T
+    G = U.conj().T @ U
+    nrm = np.sqrt(np.abs(np.diagonal(G)))
+    Gn = G / np.outer(nrm, nrm)
+    off = Gn - np.diag(np.diagonal(Gn))
+    assert np.abs(off[:head, :]).max(initial=0.0) <= 64 * tol             # leading columns: orthogonal to everything
+    sv = np.sort(np.concatenate([nrm[:head], np.linalg.svd(U[:, head:], compute_uv=False)]))[::-1]
+    assert np.max(np.abs(sv - want)) <= 32 * 2.220446049250313e-16 * want[0] * np.sqrt(r)
+    Qb, _ = np.linalg.qr(B)                                               # same column space
+    Un = U / nrm
+    assert np.linalg.norm(Un - Qb @ (Qb.conj().T @ Un)) <= 1e-9 * np.sqrt(r)

@@ -24,6 +24,8 @@ def hm():
     L.hm_reduce_i32.restype = C.c_int32
     L.hm_jacobi_done.argtypes = [C.c_int, C.c_double, C.c_double, C.c_double]
     L.hm_jacobi_done.restype = C.c_int
+    L.hm_jacobi_settled.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_double]
+    L.hm_jacobi_settled.restype = C.c_int
     return L
 
 
@@ -203,3 +205,29 @@ def test_jacobi_stop_rule(hm):
     assert hm.hm_jacobi_done(0, 0.25, 0.0, 1e-14) == 1
     # first sweep never ends on the contraction rule (no sweep before it)
     assert hm.hm_jacobi_done(10, 1e-20, 0.0, 1e-14) == 0
+
+
+def test_jacobi_output_settled_rule(hm):
+    """The second way for the sweeps to end (host/jacobi_stop.hpp): the kept values moved by at most eps sigma_max / 4 during
+    the sweep and the kept columns gained at most 1 / 32 of the squared norm left outside them."""
+    def settled(before, after, kept, eps):
+        a, b = np.ascontiguousarray(before, dtype=np.float64), np.ascontiguousarray(after, dtype=np.float64)
+        return hm.hm_jacobi_settled(_p(a), _p(b), len(b), kept, eps)
+    s = 10.0 ** (-np.arange(40) / 4.0)
+    assert settled(s, s, 10, 1e-12) == 1
+    assert settled(s, s, 40, 1e-12) == 0 and settled(s, s, 0, 1e-12) == 0          # nothing outside / nothing kept: the other rules decide
+    moved = s.copy(); moved[3] += 0.2e-12                                            # a kept value moved by less than eps sigma_max / 4
+    assert settled(s, moved, 10, 1e-12) == 1
+    moved[3] += 0.2e-12
+    assert settled(s, moved, 10, 1e-12) == 0
+    # energy still flowing from the columns outside into the kept ones: the residual bound is still improving
+    out = s.copy(); out[10:] *= 0.9                                                  # the outside lost 19 % of its squared norm
+    assert settled(s, out, 10, 1e-3) == 0
+    out = s.copy(); out[10:] *= 0.99                                                 # 2 %: below 1 / 32 of what is left
+    assert settled(s, out, 10, 1e-3) == 1
+    # the order of the columns does not matter, only the sorted values
+    perm = np.random.default_rng(3).permutation(40)
+    assert settled(s[perm], out[perm], 10, 1e-3) == 1
+    # a flat floor that keeps mixing (its norms move among themselves, their sum stays) does not hold the end back
+    floor = np.concatenate([s[:10], np.full(30, 1e-9)]); mixed = floor.copy(); mixed[10:] = 1e-9 * np.sqrt(np.linspace(0.5, 1.5, 30))
+    assert abs((mixed[10:] ** 2).sum() - (floor[10:] ** 2).sum()) < 1e-30 and settled(floor, mixed, 10, 1e-12) == 1
