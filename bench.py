@@ -44,6 +44,9 @@ WORKLOADS = {
     "cfg4": (4, 5, "C", 262144, 4096, 256, 1e-3, b"L", "hyacinTsvdFit", "complex FP16 opA=C (stored N x M) M=262144 N=4096 eps=1e-3: rank-256 L R + 1e-4 noise (limbs, 3 digits x 3 groups)"),
     "cfg5": (5, 0, "N", 1048576, 4096, 2048, 1e-8, b"A", "hyacinInterpolateFit", "real FP64 M=1048576 N=4096 eps=1e-8: (U diag(10^(-i/256)) V^T) D, D log-uniform in [1e-6, 1e6] (CRT real, 11 moduli)"),
     "target": (6, 0, "N", 131072, 2048, 1024, 1e-12, b"A", "hyacinTsvdFit", "real FP64 M=131072 N=2048 eps=1e-12: U diag(10^(-i/128)) V^T + 1e-14 G (CRT real, 14 moduli)"),
+    # the target's shape on a plain Gaussian matrix with column scales 10^(-8 j / N): full numerical rank, well separated
+    # values (an easy case for the Cholesky / Jacobi tail; kept to compare tails across kinds of spectra)
+    "gauss": (7, 0, "N", 131072, 2048, 1024, 1e-12, b"A", "hyacinTsvdFit", "real FP64 M=131072 N=2048 eps=1e-12: Gaussian entries, column scales 10^(-8 j / N) (CRT real, 14 moduli)"),
 }
 
 
@@ -112,6 +115,8 @@ def make_workload(torch, name):
     i = torch.arange(N, device="cuda", dtype=torch.float64)
     if name == "cfg4":
         A = low_rank_half(torch, g, M, N, 256, 1e-4)
+    elif name == "gauss":
+        A = torch.randn((N, M), generator=g, device="cuda", dtype=torch.float64) * (10.0 ** (-i * (8.0 / N)))[:, None]
     else:
         s = {"cfg1": 10.0 ** (-i / 16.0), "cfg2": 2.0 ** (-i / 32.0), "cfg3": 10.0 ** (-i / 128.0), "cfg5": 10.0 ** (-i / 256.0), "target": 10.0 ** (-i / 128.0)}[name]
         noise = {"cfg2": 1e-7, "cfg3": 1e-14, "target": 1e-14}.get(name, 0.0)

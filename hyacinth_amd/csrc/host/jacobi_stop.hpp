@@ -53,4 +53,22 @@ inline bool jacobi_output_settled(const std::vector<double>& before, const std::
   return gained <= outsideAfter / 32.;
 }
 
+/* Columns a sweep may leave alone.  Let nu be the K-th largest column norm and b = max(nu^2, eps^2 sum of all squared norms).
+ * The tail is the longest index range [top, r) whose squared norms sum to at most b / 1024; it is used only when it holds
+ * at least half of the columns (a few large columns in front of a broad floor of small ones: a low-rank matrix plus noise),
+ * else top = r.  Pairs of two tail columns are then never rotated.  Once the columns before `top` are orthogonal to all
+ * others, the singular values are their norms together with the values of the tail block, and those are at most
+ * sqrt(trace of its Gram matrix) <= max(nu, eps |B|_F) / 32, below everything that is handed out; the tail's share of
+ * sum sigma^2 is the sum of its squared norms in whatever basis.  What rotations inside the tail would have removed from the
+ * rows of a column p in front decays linearly, by about (tail sum) / |p|^2 per sweep: at most 1 / 1024 for the K columns
+ * that are handed out.  norm: the r column norms (not squared) as they are now. */
+inline int jacobi_tail_start(const std::vector<double>& norm, int K, double eps) {
+  const int r = (int)norm.size(); if (r == 0 || K < 1 || K >= r) { return r; }
+  double total = 0.; for (int i = r - 1; i >= 0; --i) { total += norm[(size_t)i] * norm[(size_t)i]; }
+  std::vector<double> v(norm); std::nth_element(v.begin(), v.begin() + (K - 1), v.end(), std::greater<double>());
+  const double nu2 = v[(size_t)(K - 1)] * v[(size_t)(K - 1)], bound = std::max(nu2, eps * eps * total) / 1024.;
+  double sum = 0.; int t = r; while (t > 0 && sum + norm[(size_t)(t - 1)] * norm[(size_t)(t - 1)] <= bound) { sum += norm[(size_t)(t - 1)] * norm[(size_t)(t - 1)]; --t; }
+  return 2 * t <= r ? t : r;
+}
+
 }  // namespace hyh

@@ -93,13 +93,15 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
     const bool watchOutput = K < rank;   /* with every column handed out only the cosines can end the sweeps */
     if (watchOutput && rank > 1) { fetch_norms(before); }
     for (int32_t sw = 0; sw < maxSweeps && rank > 1; ++sw) {
+      if (watchOutput) { HYH_CHECK(hipStreamSynchronize(s)); if (!hyh::ok()) { return 0; } }   /* `before` is on the host now */
+      const int32_t top = watchOutput ? hyh::jacobi_tail_start(before, K, eps) : rank;   /* a broad floor of small columns is left alone */
       HYH_KERNEL(hykGramWorkspaceClear(s, counter.p, 64));
-      HYH_KERNEL(hykJacobiSweepCarry(s, Complex, N, rank, B.as<double>(), rotateAbove, counter.as<int32_t>(), carry.as<double>())); ++used;
+      HYH_KERNEL(hykJacobiSweepTop(s, Complex, N, rank, top, top, B.as<double>(), rotateAbove, counter.as<int32_t>(), carry.as<double>())); ++used;
       if (watchOutput) { fetch_norms(after); }
       struct { int32_t rotations, pad; double cosine2; } seen = { 0, 0, 0. };
       HYH_CHECK(hipMemcpyAsync(&seen, counter.p, sizeof(seen), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
       if (!hyh::ok()) { return 0; }
-      if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: %d rotations, largest cosine %.2le\n", used, seen.rotations, std::sqrt(seen.cosine2)); }
+      if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: %d rotations, largest cosine %.2le%s\n", used, seen.rotations, std::sqrt(seen.cosine2), top < rank ? " (floor of small columns left alone)" : ""); }
       if (hyh::jacobi_sweeps_done(seen.rotations, seen.cosine2, lastCosine2, rotateAbove)) { break; }
       if (watchOutput && hyh::jacobi_output_settled(before, after, K, eps)) { if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ: the %d values handed out have settled\n", K); } break; }
       lastCosine2 = seen.cosine2; before.swap(after);

@@ -95,6 +95,7 @@ void hm_crt_lift(int cplxTable, int order, const uint32_t* residues, uint64_t* w
 /* the host's rule for ending the Jacobi sweeps of the SVD tail */
 int hm_jacobi_done(int rotations, double cosine2, double lastCosine2, double rotateAbove) { return hyh::jacobi_sweeps_done(rotations, cosine2, lastCosine2, rotateAbove) ? 1 : 0; }
 /* ... and for ending them when what is handed out has settled */
+int hm_jacobi_tail_start(const double* norm, int r, int K, double eps) { return hyh::jacobi_tail_start(std::vector<double>(norm, norm + r), K, eps); }
 int hm_jacobi_settled(const double* before, const double* after, int r, int kept, double eps) { return hyh::jacobi_output_settled(std::vector<double>(before, before + r), std::vector<double>(after, after + r), kept, eps) ? 1 : 0; }
 
 }

@@ -24,6 +24,8 @@ def hm():
     L.hm_reduce_i32.restype = C.c_int32
     L.hm_jacobi_done.argtypes = [C.c_int, C.c_double, C.c_double, C.c_double]
     L.hm_jacobi_done.restype = C.c_int
+    L.hm_jacobi_tail_start.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_double]
+    L.hm_jacobi_tail_start.restype = C.c_int
     L.hm_jacobi_settled.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_double]
     L.hm_jacobi_settled.restype = C.c_int
     return L
@@ -231,3 +233,35 @@ def test_jacobi_output_settled_rule(hm):
     # a flat floor that keeps mixing (its norms move among themselves, their sum stays) does not hold the end back
     floor = np.concatenate([s[:10], np.full(30, 1e-9)]); mixed = floor.copy(); mixed[10:] = 1e-9 * np.sqrt(np.linspace(0.5, 1.5, 30))
     assert abs((mixed[10:] ** 2).sum() - (floor[10:] ** 2).sum()) < 1e-30 and settled(floor, mixed, 10, 1e-12) == 1
+
+
+def test_jacobi_tail_rule(hm):
+    """Which columns the sweeps leave alone (host/jacobi_stop.hpp): the longest trailing index range whose squared norms sum to
+    at most 1 / 1024 of max(K-th largest squared norm, eps^2 sum), used only when it holds at least half of the columns.
+    Whatever the singular values of that block are, they stay below 1 / 32 of the smallest value handed out (trace bound),
+    checked here on an explicit matrix."""
+    rng = np.random.default_rng(5)
+    def top(norm, K, eps):
+        a = np.ascontiguousarray(norm, dtype=np.float64)
+        return hm.hm_jacobi_tail_start(_p(a), len(a), K, eps)
+    # a few large columns in front of a broad floor: the floor is left alone once its sum is small enough
+    assert top(np.concatenate([np.ones(8), np.full(100, 1e-3)]), 8, 0.0) == 8
+    assert top(np.concatenate([np.ones(8), np.full(200, 2.0 ** -8)]), 8, 0.0) == 208           # 64 of the 200 would fit (64 / 2^16 = 1 / 1024): fewer than half of all
+    assert top(np.concatenate([np.ones(8), np.full(100, 2.0 ** -8)]), 8, 0.0) == 108 - 64      # and here 64 are more than half of 108
+    # graded norms: the tail starts where the remaining squared sum drops below nu^2 / 1024; with K close to r too few qualify
+    g = 10.0 ** (-np.arange(64) / 8.0); t = top(g, 16, 0.0)
+    assert 16 < t <= 32 and (g[t:] ** 2).sum() <= g[15] ** 2 / 1024 < (g[t - 1:] ** 2).sum()
+    assert top(g, 40, 0.0) == 64
+    # every column handed out, or none: nothing is left alone
+    assert top(np.ones(5), 5, 0.0) == 5 and top(np.ones(5), 0, 0.0) == 5 and top(np.zeros(0), 3, 1e-3) == 0
+    # unsorted norms: the range ends at the first column (from the back) that does not fit
+    assert top(np.array([1.0, 1.0, 1e-4, 1.0, 1e-4, 1e-4, 1e-4, 1e-4]), 3, 0.0) == 4
+    # the claim behind the rule, on a matrix whose last block is far from diagonal
+    K, r = 6, 30
+    B = rng.standard_normal((200, r)) * np.concatenate([np.ones(K), np.full(r - K, 0.0004)])
+    Q, _ = np.linalg.qr(B[:, :K]); B[:, K:] -= Q @ (Q.T @ B[:, K:])              # leading columns orthogonal to the rest
+    B[:, :K] = Q * np.linalg.norm(B[:, :K], axis=0)
+    nrm = np.sqrt((B ** 2).sum(axis=0))
+    assert top(nrm, K, 0.0) == K
+    sv = np.linalg.svd(B, compute_uv=False)
+    assert np.allclose(np.sort(sv[:K]), np.sort(nrm[:K]), rtol=1e-12) and sv[K] <= nrm[:K].min() / 32
