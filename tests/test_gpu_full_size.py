@@ -153,3 +153,71 @@ def test_fit_at_full_width(env, at, M, N, K, eps):
     tail2 = (ev[K:] ** 2).sum().item()
     assert abs(resid2 - tail2) <= 1e-6 * tail2 + max(1e-12, (10 * eps) ** 2) * (ev ** 2).sum().item()
     assert outs[1][0] == rank and torch.equal(outs[1][1], S) and torch.equal(outs[1][2], V)
+
+
+# (name, entry point, type, opA, M, N, K, eps, algorithm, |entries| bound, rows of the repeated block)
+API_CASES = [
+    ("config 2: hyacinTsvdFit opA=T real FP32 65536 x 1024", "hyacinTsvdFit", F32, "T", 65536, 1024, 512, 1e-5, b"A", 1 << 10, 64),
+    ("config 4: hyacinTsvdFit opA=C complex FP16 262144 x 4096, limbs", "hyacinTsvdFit", F16C, "C", 262144, 4096, 256, 1e-3, b"L", 30, 32),
+    ("config 5: hyacinInterpolateFit real FP64 1048576 x 4096", "hyacinInterpolateFit", F64, "N", 1048576, 4096, 2048, 1e-8, b"A", 1 << 16, 32),
+    ("config 3: hyacinTsvdFitSegmentN complex FP64 131072 x 2048", "hyacinTsvdFitSegmentN", F64C, "N", 131072, 2048, 1024, 1e-12, b"A", 1 << 20, 64),
+]
+
+
+@pytest.mark.parametrize("name,fit,at,opA,M,N,K,eps,alg,bound,m0", API_CASES, ids=[c[0].split(":")[0] + " fit" for c in API_CASES])
+def test_fit_entry_points_at_configuration_size(env, name, fit, at, opA, M, N, K, eps, alg, bound, m0):
+    """The fit each configuration names (include/hyacin.h:67-113), at its size, storage order and type, on the repeated
+    integer block: the matrix has exactly the rank of the block (its rows), so the fit must stop there; its singular values
+    are sqrt(M / m0) times the block's; the basis must capture the matrix (hyacinCheckNorm <= (10 eps)^2 |A|^2), the
+    interpolation must reproduce the block from the chosen columns."""
+    ha, h, torch = env
+    L = ha.lib()
+    rng = np.random.default_rng(77)
+    re, im, _, _ = block_and_gram(rng, at, N, bound, m0)
+    re[:, N // 3] = rng.integers(1, bound + 1, m0)        # no all-zero column here: every column can be a pivot
+    if im is not None:
+        im[:, N // 3] = rng.integers(1, bound + 1, m0)
+    reps = M // m0
+    cplx = at & 1
+    real_t = {F64: torch.float64, F64C: torch.float64, F32: torch.float32, F16C: torch.float16}[at]
+    A0 = (re + 1j * im) if cplx else re.astype(np.float64)                              # the block, m0 x N
+    if at in (F16, F16C):
+        A0 = A0 * 2.0 ** -6                      # singular values of the order of 2000: the half-precision S can hold them
+    stored = np.conj(A0) if opA == "C" else A0                                          # op(stored) = A
+    blk = np.stack([stored.real, stored.imag], axis=-1) if cplx else stored[..., None]  # [m0][N][comps]
+    comps = 2 if cplx else 1
+    if opA == "N":                                                                      # column-major M x N: [N][M][comps]
+        blk_d = torch.from_numpy(np.ascontiguousarray(np.transpose(blk, (1, 0, 2)))).to("cuda").to(real_t)
+        A = blk_d.unsqueeze(1).expand(N, reps, m0, comps).reshape(N, M, comps).contiguous(); lda = M
+    else:                                                                               # the stored N x M matrix: [M][N][comps]
+        blk_d = torch.from_numpy(np.ascontiguousarray(blk)).to("cuda").to(real_t)
+        A = blk_d.unsqueeze(0).expand(reps, m0, N, comps).reshape(M, N, comps).contiguous(); lda = N
+    print(name, "device bytes", A.element_size() * A.numel(), flush=True)
+    pA = C.c_void_p(A.data_ptr())
+    S = torch.zeros(max(K, N), dtype=torch.float64, device="cuda")
+    V = torch.zeros(N * K * comps, dtype=real_t, device="cuda")
+    h.GramMatrixAlgorithm = alg
+    try:
+        rank = getattr(L, fit)(C.byref(h), eps, opA.encode(), M, N, K, pA, lda, C.c_void_p(S.data_ptr()), C.c_void_p(V.data_ptr()), N, 0, at)
+        torch.cuda.synchronize()
+        assert L.hykLastStatus() == 0
+        assert rank == m0, (rank, m0)
+        want = np.linalg.svd(A0, compute_uv=False) * np.sqrt(reps)
+        storage_eps = {torch.float64: 2.2e-16, torch.float32: 6e-8, torch.float16: 4.9e-4}[real_t]
+        if fit == "hyacinInterpolateFit":
+            jp = S.view(torch.int32)[:N].cpu().numpy()
+            assert sorted(jp.tolist()) == list(range(1, N + 1))
+            X = V.cpu().numpy().reshape(K, N).T[:, :rank]                               # N x rank
+            sel = jp[:rank] - 1
+            assert np.allclose(X[sel], np.eye(rank), atol=1e-12)
+            assert np.linalg.norm(A0 - A0[:, sel] @ X.T) <= 50 * max(eps, storage_eps) * np.linalg.norm(A0)
+        else:
+            Sh = S.view(real_t)[:K].double().cpu().numpy()
+            assert np.all(Sh[rank:] == 0)
+            assert np.abs(Sh[:rank] - want[:rank]).max() <= 10 * max(eps, storage_eps) * want[0]
+            err = L.hyacinCheckNorm(C.byref(h), opA.encode(), M, N, pA, lda, rank, C.c_void_p(V.data_ptr()), N, at)
+            nrm = L.hyacinCheckNorm(C.byref(h), opA.encode(), M, N, pA, lda, 0, None, N, at)
+            assert abs(nrm - (np.abs(A0) ** 2).sum() * reps) <= 1e-9 * nrm
+            assert err <= (10 * max(eps, storage_eps)) ** 2 * nrm, (err, nrm)
+    finally:
+        h.GramMatrixAlgorithm = b"A"
