@@ -366,6 +366,16 @@ def main():
         dbytes = cP * lP * stride * 8 + N * N * gb.value
         stages["dequantize"] = {"ms": t, "bytes": dbytes, "GB/s": dbytes / t / 1e6, "frac_of_hbm_peak": dbytes / t / 1e6 / HBM_PEAK_GBS}
         del G
+        # what plain streams reach on this device in the same run: a 1 GiB -> 1 GiB copy (half reads, half writes) and a 2 GiB fill
+        src = torch.ones(2 ** 27, dtype=torch.float64, device="cuda")
+        dst = torch.empty(2 ** 28, dtype=torch.float64, device="cuda")
+        t = timed_ms(lambda: L.hykMatcopy(stream, b"A", 2 ** 20, 128, 0, C.c_void_p(src.data_ptr()), 2 ** 20, 0, C.c_void_p(dst.data_ptr()), 2 ** 20))
+        copy_gbs = 2 * 2 ** 30 / t / 1e6
+        t = timed_ms(lambda: L.hykGramWorkspaceClear(stream, C.c_void_p(dst.data_ptr()), 2 ** 31))
+        fill_gbs = 2 ** 31 / t / 1e6
+        stages["device_streams"] = {"copy_GB/s": copy_gbs, "fill_GB/s": fill_gbs, "what": "copy_kernel 1 GiB -> 1 GiB and fill_zero_kernel 2 GiB in this run: a mixed read / write stream does not reach what a read-only stream does"}
+        stages["quantize"]["frac_of_copy_stream"] = stages["quantize"]["GB/s"] / copy_gbs
+        del src, dst
 
     fit_ms, fit_rank = None, None
     if not a.no_fit:

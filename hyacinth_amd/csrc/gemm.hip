@@ -8,8 +8,9 @@
  * copy; here: the interleaved operands are multiplied directly with FP32
  * accumulation, which is at least as accurate as the reference's FP16
  * accumulation).  FP64 types accumulate in FP64, FP32 / FP16 types in FP32.
- * General kernel: LDS-tiled 64 x 64 x 16, 256 threads, a 4 x 4 register tile per thread (vector ALU).  The FP16 products
- * C = op(A) B, the shape of matmul_cf16_{cn,tn,nn}, run on the matrix cores (second kernel below).
+ * General kernel: LDS-tiled 64 x 64 x 16, 256 threads, a 4 x 4 register tile per thread (vector ALU).  The FP16 and FP32
+ * products C = op(A) B, the shape of matmul_cf16_{cn,tn,nn} and of the stage products of the segmented fit, run on the
+ * matrix cores (the two kernels below).
  */
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
@@ -133,7 +134,8 @@ __device__ __forceinline__ uint4 load_piece_strided(const char* X, int64_t ldx, 
     for (int i = 0; i < PE; ++i) {
       if (k + i < K) {
         const char* src = X + (q + (k + i) * ldx) * E;
-        if constexpr (E == 4) { w[i] = *reinterpret_cast<const uint32_t*>(src); } else { w[i >> 1] |= (uint32_t)*reinterpret_cast<const uint16_t*>(src) << (16 * (i & 1)); }
+        if constexpr (E == 8) { const uint2 v = *reinterpret_cast<const uint2*>(src); w[2 * i] = v.x; w[2 * i + 1] = v.y; }
+        else if constexpr (E == 4) { w[i] = *reinterpret_cast<const uint32_t*>(src); } else { w[i >> 1] |= (uint32_t)*reinterpret_cast<const uint16_t*>(src) << (16 * (i & 1)); }
       }
     }
   }
@@ -234,6 +236,113 @@ __global__ __launch_bounds__(256) void gemm_f16_mfma_kernel(int32_t M, int32_t N
   }
 }
 
+/* ------------------------------------------------------------------ FP32 products on the matrix cores
+ * The same tiling with `v_mfma_f32_32x32x2_f32` (C = op(A) B, real and complex FP32, FP32 accumulation): the stage products
+ * of the column-segmented fit for FP32 storage (reference: the GemmEx calls of src/lra.cpp:90-93,102-105).  A 16-byte piece
+ * of an LDS row holds four consecutive contraction indices (two complex numbers); the lanes 0..31 take the even pieces and
+ * the lanes 32..63 the odd ones, and the four MFMA steps of a piece use its four floats in turn: both operands follow the
+ * same assignment, so every index is contracted once.  Complex as a real product of twice the depth, as above: B's
+ * interleaved storage is the real (2 K) x N operand, op(A) expands to (Ar, -Ai) / (Ai, Ar) (conjugated: (Ar, Ai) /
+ * (-Ai, Ar)) in registers. */
+template <bool CPLX, int OPA>   /* OPA: 0 'N', 1 'T', 2 'C' */
+__global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(int32_t M, int32_t N, int32_t K, const char* __restrict__ A, int64_t lda, const char* __restrict__ B, int64_t ldb, char* __restrict__ C, int64_t ldc) {
+  constexpr int E = CPLX ? 8 : 4, PE = 16 / E, KS = HROW / E;
+  __shared__ __attribute__((aligned(16))) char lds[2][2][HTILE];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, wm = wave & 1, wn = wave >> 1;
+  const int64_t m0 = (int64_t)blockIdx.x * HT, n0 = (int64_t)blockIdx.y * HT;
+  uint4 ra[4], rb[4];
+  auto fetch = [&](int64_t k0) {
+    #pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      if constexpr (OPA == 0) { const int row = tid & 127, p = (tid >> 7) + 2 * r; ra[r] = load_piece_strided<E>(A, lda, m0 + row, M, k0 + p * PE, K); }
+      else { const int row = (tid >> 3) + 32 * r, p = tid & 7; ra[r] = load_piece_contiguous<E>(A, lda, m0 + row, M, k0 + p * PE, K); }
+      { const int row = (tid >> 3) + 32 * r, p = tid & 7; rb[r] = load_piece_contiguous<E>(B, ldb, n0 + row, N, k0 + p * PE, K); }
+    }
+  };
+  auto park = [&](int buf) {
+    #pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      { const int row = OPA == 0 ? (tid & 127) : (tid >> 3) + 32 * r, p = OPA == 0 ? (tid >> 7) + 2 * r : (tid & 7);
+        *reinterpret_cast<uint4*>(&lds[buf][0][row * HROW + ((p ^ h_swz(row)) << 4)]) = ra[r]; }
+      { const int row = (tid >> 3) + 32 * r, p = tid & 7; *reinterpret_cast<uint4*>(&lds[buf][1][row * HROW + ((p ^ h_swz(row)) << 4)]) = rb[r]; }
+    }
+  };
+  constexpr int SETS = CPLX ? 2 : 1;
+  float16_t acc[SETS][2][2];   /* [re | im][block of n][block of m] */
+  #pragma unroll
+  for (int s = 0; s < SETS; ++s) {
+    #pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      #pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        #pragma unroll
+        for (int e = 0; e < 16; ++e) { acc[s][i][j][e] = 0.f; }
+      }
+    }
+  }
+  const int slabs = (K + KS - 1) / KS;
+  const int rowM = (wm * 64 + (lane & 31)) * HROW, rowN = (wn * 64 + (lane & 31)) * HROW, sw = h_swz(lane & 31), hi = lane >> 5;
+  if (slabs > 0) { fetch(0); park(0); }
+  __syncthreads();
+  for (int it = 0; it < slabs; ++it) {
+    const int buf = it & 1;
+    if (it + 1 < slabs) { fetch((int64_t)(it + 1) * KS); }
+    #pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int slot = ((2 * s + hi) ^ sw) << 4;
+      float4 fm[2], fn[2];
+      #pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        fm[b] = *reinterpret_cast<const float4*>(&lds[buf][0][rowM + b * 32 * HROW + slot]);
+        fn[b] = *reinterpret_cast<const float4*>(&lds[buf][1][rowN + b * 32 * HROW + slot]);
+      }
+      #pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const float a[4] = { fm[j].x, fm[j].y, fm[j].z, fm[j].w };
+        float are[4], aim[4];
+        if constexpr (CPLX) {   /* a = (Ar0, Ai0, Ar1, Ai1) */
+          are[0] = a[0]; are[1] = OPA == 2 ? a[1] : -a[1]; are[2] = a[2]; are[3] = OPA == 2 ? a[3] : -a[3];
+          aim[0] = OPA == 2 ? -a[1] : a[1]; aim[1] = a[0]; aim[2] = OPA == 2 ? -a[3] : a[3]; aim[3] = a[2];
+        } else { are[0] = a[0]; are[1] = a[1]; are[2] = a[2]; are[3] = a[3]; aim[0] = aim[1] = aim[2] = aim[3] = 0.f; }
+        #pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          const float b[4] = { fn[i].x, fn[i].y, fn[i].z, fn[i].w };
+          #pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            acc[0][i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(b[e], are[e], acc[0][i][j], 0, 0, 0);
+            if constexpr (CPLX) { acc[1][i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(b[e], aim[e], acc[1][i][j], 0, 0, 0); }
+          }
+        }
+      }
+    }
+    if (it + 1 < slabs) { park(buf ^ 1); }
+    __syncthreads();
+  }
+  /* lane: row m of the block; register e: column n = 8 (e / 4) + 4 (lane / 32) + e % 4 of the block */
+  #pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    #pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int64_t m = m0 + wm * 64 + j * 32 + (lane & 31); if (m >= M) { continue; }
+      #pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int64_t n = n0 + wn * 64 + i * 32 + ((e >> 2) << 3) + (hi << 2) + (e & 3); if (n >= N) { continue; }
+        char* dst = C + (m + n * ldc) * E;
+        if constexpr (CPLX) { *reinterpret_cast<float2*>(dst) = make_float2(acc[0][i][j][e], acc[1][i][j][e]); }
+        else { *reinterpret_cast<float*>(dst) = acc[0][i][j][e]; }
+      }
+    }
+  }
+}
+
+template <bool CPLX> int run_f32_mfma(hipStream_t stream, char opA, int32_t M, int32_t N, int32_t K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C, int64_t ldc) {
+  dim3 grid((M + HT - 1) / HT, (N + HT - 1) / HT); const char* a = (const char*)A; const char* b = (const char*)B; char* c = (char*)C;
+  if (opA == 'N') { gemm_f32_mfma_kernel<CPLX, 0><<<grid, 256, 0, stream>>>(M, N, K, a, lda, b, ldb, c, ldc); }
+  else if (opA == 'T' || !CPLX) { gemm_f32_mfma_kernel<CPLX, 1><<<grid, 256, 0, stream>>>(M, N, K, a, lda, b, ldb, c, ldc); }
+  else { gemm_f32_mfma_kernel<CPLX, 2><<<grid, 256, 0, stream>>>(M, N, K, a, lda, b, ldb, c, ldc); }
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
 template <bool CPLX> int run_f16_mfma(hipStream_t stream, char opA, int32_t M, int32_t N, int32_t K, const void* A, int64_t lda, const void* B, int64_t ldb, void* C, int64_t ldc) {
   dim3 grid((M + HT - 1) / HT, (N + HT - 1) / HT); const char* a = (const char*)A; const char* b = (const char*)B; char* c = (char*)C;
   if (opA == 'N') { gemm_f16_mfma_kernel<CPLX, 0><<<grid, 256, 0, stream>>>(M, N, K, a, lda, b, ldb, c, ldc); }
@@ -242,10 +351,10 @@ template <bool CPLX> int run_f16_mfma(hipStream_t stream, char opA, int32_t M, i
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
-/* the matrix-core kernel covers C = op(A) B (alpha 1, beta 0, B as stored) on 16-byte aligned operands */
-bool f16_mfma_applies(char opB, double alpha, double beta, int32_t type, const void* A, int64_t lda, const void* B, int64_t ldb, const void* C, int32_t N) {
-  if ((type != HYK_F16 && type != HYK_F16C) || opB != 'N' || alpha != 1.0 || beta != 0.0 || (N + HT - 1) / HT > 65535) { return false; }
-  const int64_t e = type == HYK_F16C ? 4 : 2;
+/* the matrix-core kernels cover C = op(A) B (alpha 1, beta 0, B as stored) on 16-byte aligned operands, FP16 and FP32 storage */
+bool mfma_applies(char opB, double alpha, double beta, int32_t type, const void* A, int64_t lda, const void* B, int64_t ldb, const void* C, int32_t N) {
+  if ((type != HYK_F16 && type != HYK_F16C && type != HYK_F32 && type != HYK_F32C) || opB != 'N' || alpha != 1.0 || beta != 0.0 || (N + HT - 1) / HT > 65535) { return false; }
+  const int64_t e = type == HYK_F16C ? 4 : (type == HYK_F16 ? 2 : (type == HYK_F32 ? 4 : 8));
   return ((uintptr_t)A % 16 == 0) && ((uintptr_t)B % 16 == 0) && ((uintptr_t)C % e == 0) && (lda * e) % 16 == 0 && (ldb * e) % 16 == 0;
 }
 
@@ -257,8 +366,13 @@ extern "C" int hykGemm(hipStream_t stream, char opA, char opB, int32_t M, int32_
   if (M <= 0 || N <= 0) { return 0; }
   if (K < 0 || (N + GT - 1) / GT > 65535) { return -1; }
   opA = norm_op(opA); opB = norm_op(opB);
-  if (K > 0 && f16_mfma_applies(opB, alpha, beta, type, A, lda, B, ldb, C, N)) {
-    return type == HYK_F16C ? run_f16_mfma<true>(stream, opA, M, N, K, A, lda, B, ldb, C, ldc) : run_f16_mfma<false>(stream, opA, M, N, K, A, lda, B, ldb, C, ldc);
+  if (K > 0 && mfma_applies(opB, alpha, beta, type, A, lda, B, ldb, C, N)) {
+    switch (type) {
+      case HYK_F16C: return run_f16_mfma<true>(stream, opA, M, N, K, A, lda, B, ldb, C, ldc);
+      case HYK_F16: return run_f16_mfma<false>(stream, opA, M, N, K, A, lda, B, ldb, C, ldc);
+      case HYK_F32C: return run_f32_mfma<true>(stream, opA, M, N, K, A, lda, B, ldb, C, ldc);
+      default: return run_f32_mfma<false>(stream, opA, M, N, K, A, lda, B, ldb, C, ldc);
+    }
   }
   switch (type) {
     case HYK_F64: return run<double, false>(stream, opA, opB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc);

@@ -151,8 +151,9 @@ int hykMatmulCf16(hipStream_t stream, char opA, int32_t M, int32_t N, int32_t K,
 
 /* Real / complex matrix product C = op(A) B in the storage type (FP64, FP32, FP16 and complex FP64 / FP32), used by the
  * column-segmented fit and the residual check.  Replaces the cuBLAS gemm calls of src/lra.cpp:86-105,202-203.
- * alpha/beta are real scalars. opA 'N' | 'T' | 'C', opB 'N' | 'T' | 'C'.  FP16 and complex FP16 calls of the form
- * C = op(A) B (alpha 1, beta 0, opB 'N') run on the matrix cores like hykMatmulCf16. */
+ * alpha/beta are real scalars. opA 'N' | 'T' | 'C', opB 'N' | 'T' | 'C'.  FP16 and FP32 calls (real and complex) of the
+ * form C = op(A) B (alpha 1, beta 0, opB 'N') with 16-byte aligned operands and leading dimensions run on the matrix cores
+ * (v_mfma_f32_32x32x16_f16, v_mfma_f32_32x32x2_f32, FP32 accumulation); everything else on the vector ALU. */
 int hykGemm(hipStream_t stream, char opA, char opB, int32_t M, int32_t N, int32_t K, double alpha, int32_t type, const void* A, int64_t lda, const void* B, int64_t ldb, double beta, void* C, int64_t ldc);
 
 /* V (N x r, FP64 or complex FP64, interleaved) is overwritten by an orthonormal basis of its column space (one-sided

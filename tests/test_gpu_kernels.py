@@ -379,6 +379,40 @@ def test_f16_products(gl, cplx, opA, M, N, K, pad):
 
 
 @pytest.mark.parametrize("cplx", [0, 1])
+@pytest.mark.parametrize("opA", ["N", "T", "C"])
+@pytest.mark.parametrize("M,N,K,pad", [(300, 70, 45, 0), (128, 128, 64, 0), (1000, 260, 333, 4), (257, 129, 1, 0), (96, 40, 200, 3), (2048, 512, 2048, 0)])
+def test_f32_products(gl, cplx, opA, M, N, K, pad):
+    """hykGemm on FP32 / complex FP32 operands in the form C = op(A) B (the stage products of the column-segmented fit, the
+    GemmEx calls of src/lra.cpp:90-93,102-105) against numpy in FP64 on the same inputs, at the bound of test_gemm_fp64 with
+    the FP32 unit roundoff: 2^-24 / 2^-53 times its 1e-13.  Ragged tiles, K tails inside a 16-byte piece, padded leading
+    dimensions; pad = 3 makes the leading dimensions unaligned, which takes the vector-ALU kernel."""
+    from gpu_util import dev, zeros, ptr, stream, sync, host
+    rng = np.random.default_rng(177 + cplx)
+    comps = 2 if cplx else 1
+    rowsA, colsA = (M, K) if opA == "N" else (K, M)
+    lda, ldb, ldc = rowsA + (4 - rowsA % 4) % 4 + pad, K + (4 - K % 4) % 4 + pad, M + pad
+    def rand(rows, cols, ld):
+        buf = np.zeros((cols, ld, comps), np.float32)
+        buf[:, :rows, :] = rng.standard_normal((cols, rows, comps)).astype(np.float32)
+        v = buf[:, :rows, :].astype(np.float64)
+        m = (v[..., 0] + 1j * v[..., 1]).T if cplx else v[..., 0].T        # rows x cols
+        return buf, m
+    bufA, mA = rand(rowsA, colsA, lda)
+    bufB, mB = rand(K, N, ldb)
+    want = (mA if opA == "N" else (mA.T if opA == "T" else mA.conj().T)) @ mB
+    Cd = zeros(N * ldc * comps * 4)
+    dA, dB = dev(bufA), dev(bufB)
+    rc = gl.L.hykGemm(stream(), opA.encode(), b"N", M, N, K, C.c_double(1.0), 3 if cplx else 2, ptr(dA), C.c_int64(lda), ptr(dB), C.c_int64(ldb), C.c_double(0.0), ptr(Cd), C.c_int64(ldc))
+    assert rc == 0
+    sync()
+    full = host(Cd, np.float32, (N, ldc, comps))
+    got = full[:, :M, :].astype(np.float64)
+    got = (got[..., 0] + 1j * got[..., 1]).T if cplx else got[..., 0].T
+    assert np.abs(got - want).max() <= 1e-13 * 2.0**29 * np.abs(want).max() * max(1, K) ** 0.5
+    assert not full[:, M:, :].any()                                        # nothing written into the padding
+
+
+@pytest.mark.parametrize("cplx", [0, 1])
 @pytest.mark.parametrize("N,K", [(40, 7), (150, 32), (300, 75), (700, 257)])
 def test_interp_solve(gl, cplx, N, K):
     """hykInterpSolve (cuBLAS trsm of src/gram_id.cpp:40-46): T = R11^-1 R12 for a factor given column-wise in pivot order,
