@@ -90,7 +90,7 @@ int hykDequantize(hipStream_t stream, int32_t N, int32_t orderC, const uint64_t*
  * Rt: zero-initialised, column-wise factor Rt[c * ldr + k] = R[k, c] in the type of G, ldr >= min(N, K + 1).
  * jpiv: N 1-based pivots in the reference's swap order.  rankOut: device-visible int32 (pinned host memory); -1 when the
  * workgroups of the run lost each other (a bounded wait inside the kernel gave up).
- * hykPotrfp runs the blocked right-looking kernel (panels of 16 columns, one rank-16 update of the trailing matrix per
+ * hykPotrfp runs the blocked right-looking kernel (panels of 32 columns, 16 for complex matrices, one rank-32 or rank-16 update of the trailing matrix per
  * panel) for N <= 8192 when computeUnits >= ceil(N / 64), else the left-looking kernel, which hykPotrfpLeftLooking
  * always runs (it leaves G untouched).  Same pivots, same rank; factor entries equal to rounding. */
 size_t hykPotrfpWorkspaceBytes(int32_t N, int32_t Gtype);
@@ -99,7 +99,7 @@ int hykPotrfpLeftLooking(hipStream_t stream, int32_t computeUnits, double eps, i
 
 /* hykPotrfp for callers that cannot allocate device memory (code under HIP graph capture, serving loops, harnesses that
  * forbid hipMalloc).  No counterpart in the reference.  The workspace of hykPotrfp (diagonal, position table, exchange
- * records; 194 KB) is a device array built into the library, one copy per device, so the call allocates nothing; inputs
+ * records; 197 120 bytes) is a device array built into the library, one copy per device, so the call allocates nothing; inputs
  * and outputs are the caller's as in hykPotrfp.  N <= hykPotrfpStaticMaxN() (8192), larger N returns -2 with a message on
  * stderr.  All calls on one device share the array: calls that overlap on one device (two streams, two threads) race. */
 int32_t hykPotrfpStaticMaxN(void);
