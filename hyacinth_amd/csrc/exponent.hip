@@ -71,13 +71,13 @@ __global__ __launch_bounds__(EXP_THREADS) void column_exponent_kernel(int32_t se
  * slice, so every load instruction of a wavefront covers 1 KB of one stored row; the per-chunk results meet in mexp (filled
  * with INT_MAX before) through an integer minimum: u - e is smallest where the magnitude is largest.  Replaces the
  * transposing copy of src/lra.cpp:63-69 followed by src/fp_exponent.cu:23-51. */
-constexpr int EXP_T_ROWS = 64;
+constexpr int EXP_T_ROWS = 64;    /* rows per workgroup: a multiple of this, chosen on the host so that the launch still has a few thousand workgroups */
 template <typename SCALAR>
-__global__ __launch_bounds__(EXP_THREADS) void column_exponent_transposed_kernel(int32_t segM, int32_t lastM, int32_t comps, const SCALAR* __restrict__ S, int64_t lda_scalars, int32_t u, int32_t N, int32_t* __restrict__ mexp) {
+__global__ __launch_bounds__(EXP_THREADS) void column_exponent_transposed_kernel(int32_t segM, int32_t lastM, int32_t comps, const SCALAR* __restrict__ S, int64_t lda_scalars, int32_t u, int32_t N, int32_t* __restrict__ mexp, int32_t rowsPerBlock) {
   constexpr int VEC = 16 / sizeof(SCALAR); constexpr SCALAR ABS = (SCALAR)(~(SCALAR)0) >> 1;
   const int32_t b = blockIdx.y; const int64_t rows = (b + 1 == (int32_t)gridDim.y) ? lastM : segM;
-  const int64_t r0 = (int64_t)blockIdx.x * EXP_T_ROWS; if (r0 >= rows) { return; }
-  const int64_t r1 = r0 + EXP_T_ROWS < rows ? r0 + EXP_T_ROWS : rows, width = (int64_t)N * comps;
+  const int64_t r0 = (int64_t)blockIdx.x * rowsPerBlock; if (r0 >= rows) { return; }
+  const int64_t r1 = r0 + rowsPerBlock < rows ? r0 + rowsPerBlock : rows, width = (int64_t)N * comps;
   const int64_t c0 = ((int64_t)blockIdx.z * EXP_THREADS + threadIdx.x) * VEC; if (c0 >= width) { return; }
   const SCALAR* base = S + ((int64_t)b * segM + r0) * lda_scalars + c0;
   SCALAR mx[VEC];
@@ -179,11 +179,13 @@ extern "C" int hykColumnExponentsOp(hipStream_t stream, char opA, int32_t batche
   } else {
     const int64_t cells = (int64_t)batches * N; exponent_fill_kernel<<<(uint32_t)((cells + 255) / 256), 256, 0, stream>>>((int32_t)cells, &vexp[N]);
     const int scalarBytes = (Atype & ~1) == HYK_F64 ? 8 : ((Atype & ~1) == HYK_F32 ? 4 : 2); const int64_t perBlock = (int64_t)EXP_THREADS * (16 / scalarBytes);
-    dim3 grid((uint32_t)((segM + EXP_T_ROWS - 1) / EXP_T_ROWS), (uint32_t)batches, (uint32_t)(((int64_t)N * comps + perBlock - 1) / perBlock));
+    const int64_t across = ((int64_t)N * comps + perBlock - 1) / perBlock, at64 = (int64_t)((segM + EXP_T_ROWS - 1) / EXP_T_ROWS) * batches * across;
+    const int32_t rowsPerBlock = EXP_T_ROWS * (int32_t)std::min<int64_t>(16, std::max<int64_t>(1, at64 / 4096));   /* fewer atomic minima per column while 4096 workgroups remain */
+    dim3 grid((uint32_t)((segM + rowsPerBlock - 1) / rowsPerBlock), (uint32_t)batches, (uint32_t)across);
     switch (Atype & ~1) {
-      case HYK_F64: column_exponent_transposed_kernel<uint64_t><<<grid, EXP_THREADS, 0, stream>>>(segM, lastM, comps, (const uint64_t*)A, lda * comps, u, N, &vexp[N]); break;
-      case HYK_F32: column_exponent_transposed_kernel<uint32_t><<<grid, EXP_THREADS, 0, stream>>>(segM, lastM, comps, (const uint32_t*)A, lda * comps, u, N, &vexp[N]); break;
-      default: column_exponent_transposed_kernel<uint16_t><<<grid, EXP_THREADS, 0, stream>>>(segM, lastM, comps, (const uint16_t*)A, lda * comps, u, N, &vexp[N]); break;
+      case HYK_F64: column_exponent_transposed_kernel<uint64_t><<<grid, EXP_THREADS, 0, stream>>>(segM, lastM, comps, (const uint64_t*)A, lda * comps, u, N, &vexp[N], rowsPerBlock); break;
+      case HYK_F32: column_exponent_transposed_kernel<uint32_t><<<grid, EXP_THREADS, 0, stream>>>(segM, lastM, comps, (const uint32_t*)A, lda * comps, u, N, &vexp[N], rowsPerBlock); break;
+      default: column_exponent_transposed_kernel<uint16_t><<<grid, EXP_THREADS, 0, stream>>>(segM, lastM, comps, (const uint16_t*)A, lda * comps, u, N, &vexp[N], rowsPerBlock); break;
     }
   }
   exponent_min_kernel<<<(N + 255) / 256, 256, 0, stream>>>(N, batches, vexp);

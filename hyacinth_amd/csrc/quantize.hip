@@ -284,10 +284,34 @@ __global__ __launch_bounds__(Q_THREADS) void quantize_transposed_kernel(int32_t 
   extern __shared__ __attribute__((aligned(16))) unsigned char tileBytes[];
   T* tile = reinterpret_cast<T*>(tileBytes);
   const int64_t k0 = (int64_t)blockIdx.x * T_ROWS; const int32_t j0 = blockIdx.y * TJ;
-  for (int e = threadIdx.x; e < TJ * T_ROWS; e += Q_THREADS) {
-    const int jj = e % TJ, kk = e / TJ; T v = T{};
-    if (j0 + jj < N && k0 + kk < M) { v = S[(int64_t)(j0 + jj) + (k0 + kk) * lda]; if constexpr (CONJ) { v = conj_elem<E>(v); } }
-    tile[jj * PITCH + kk] = v;
+  /* whole tiles of an aligned matrix come in as 16-byte pieces along the stored rows, all loads of a thread issued before
+   * the first LDS write; ragged or unaligned tiles element by element */
+  constexpr int VE = sizeof(T) >= 16 ? 1 : 16 / (int)sizeof(T), PIECES = TJ / VE, ITER = PIECES * T_ROWS / Q_THREADS;
+  static_assert(PIECES * T_ROWS % Q_THREADS == 0, "the pieces of a tile divide evenly among the threads");
+  if ((((uintptr_t)S) & 15u) == 0 && ((lda * (int64_t)sizeof(T)) & 15) == 0 && j0 + TJ <= N) {
+    u32x4 piece[ITER];
+    #pragma unroll
+    for (int it = 0; it < ITER; ++it) {
+      const int e = threadIdx.x + it * Q_THREADS, g = e % PIECES, kk = e / PIECES;
+      piece[it] = u32x4{ 0u, 0u, 0u, 0u };
+      if (k0 + kk < M) { piece[it] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(&S[(int64_t)(j0 + g * VE) + (k0 + kk) * lda])); }
+    }
+    #pragma unroll
+    for (int it = 0; it < ITER; ++it) {
+      const int e = threadIdx.x + it * Q_THREADS, g = e % PIECES, kk = e / PIECES;
+      #pragma unroll
+      for (int c = 0; c < VE; ++c) {
+        T v; __builtin_memcpy(&v, reinterpret_cast<const char*>(&piece[it]) + c * sizeof(T), sizeof(T));
+        if constexpr (CONJ) { v = conj_elem<E>(v); }
+        tile[(g * VE + c) * PITCH + kk] = v;
+      }
+    }
+  } else {
+    for (int e = threadIdx.x; e < TJ * T_ROWS; e += Q_THREADS) {
+      const int jj = e % TJ, kk = e / TJ; T v = T{};
+      if (j0 + jj < N && k0 + kk < M) { v = S[(int64_t)(j0 + jj) + (k0 + kk) * lda]; if constexpr (CONJ) { v = conj_elem<E>(v); } }
+      tile[jj * PITCH + kk] = v;
+    }
   }
   __syncthreads();
   constexpr int GROUPS = T_ROWS / Q_ROWS;   /* 32 row groups per column: a wavefront covers two columns */
