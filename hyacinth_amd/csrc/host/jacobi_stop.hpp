@@ -40,17 +40,18 @@ inline bool jacobi_sweeps_done(int rotations, double cosine2, double lastCosine2
  * A noise floor of hundreds of nearly equal small columns, which a cyclic Jacobi method needs ten and more sweeps to resolve
  * and which is never handed out, then no longer decides when the sweeps end.  With nothing left outside (kept = all columns
  * and a zero cut) rule (ii) never holds and the rules above decide alone.
- * before / after: the column norms (not squared) at the start and at the end of the sweep, in the same column order. */
-inline bool jacobi_output_settled(const std::vector<double>& before, const std::vector<double>& after, int kept, double eps) {
+ * before / after: the column norms (not squared) at the start and at the end of the sweep, in the same column order.
+ * seen (optional): { largest move of a kept value, what the kept columns gained, what is left outside } for the log. */
+inline bool jacobi_output_settled(const std::vector<double>& before, const std::vector<double>& after, int kept, double eps, double* seen = nullptr) {
   const size_t r = after.size(); if (before.size() != r || r == 0 || kept <= 0 || (size_t)kept >= r) { return false; }
   std::vector<double> a(before), b(after);
   std::sort(a.begin(), a.end(), std::greater<double>()); std::sort(b.begin(), b.end(), std::greater<double>());
   double moved = 0.; for (int i = 0; i < kept; ++i) { moved = std::max(moved, std::fabs(b[(size_t)i] - a[(size_t)i])); }
-  if (!(moved <= 0.25 * eps * b[0])) { return false; }
   double outsideBefore = 0., outsideAfter = 0.;   /* summed from the small end: no cancellation against the large values */
   for (size_t i = r; i-- > (size_t)kept;) { outsideBefore += a[i] * a[i]; outsideAfter += b[i] * b[i]; }
   const double gained = outsideBefore - outsideAfter;
-  return gained <= outsideAfter / 32.;
+  if (seen) { seen[0] = moved; seen[1] = gained; seen[2] = outsideAfter; }
+  return moved <= 0.25 * eps * b[0] && gained <= outsideAfter / 32.;
 }
 
 /* Columns a sweep may leave alone.  Let nu be the K-th largest column norm and b = max(nu^2, eps^2 sum of all squared norms).

@@ -103,7 +103,11 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
       if (!hyh::ok()) { return 0; }
       if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: %d rotations, largest cosine %.2le%s\n", used, seen.rotations, std::sqrt(seen.cosine2), top < rank ? " (floor of small columns left alone)" : ""); }
       if (hyh::jacobi_sweeps_done(seen.rotations, seen.cosine2, lastCosine2, rotateAbove)) { break; }
-      if (watchOutput && hyh::jacobi_output_settled(before, after, K, eps)) { if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ: the %d values handed out have settled\n", K); } break; }
+      if (watchOutput) {
+        double moved[3] = { 0., 0., 0. }; const bool settled = hyh::jacobi_output_settled(before, after, K, eps, moved);
+        if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: the %d values handed out moved by at most %.2le, their columns gained %.2le of %.2le outside%s\n", used, K, moved[0], moved[1], moved[2], settled ? ": settled" : ""); }
+        if (settled) { break; }
+      }
       lastCosine2 = seen.cosine2; before.swap(after);
     }
     HYH_KERNEL(hykColumnNorms(s, Complex, N, rank, B.as<double>(), sigma.as<double>()));

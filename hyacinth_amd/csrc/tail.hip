@@ -388,15 +388,46 @@ __global__ __launch_bounds__(THREADS) void jacobi_block_round_kernel(int32_t N, 
  * step kernel; the cross products of later steps come out of the updated Gram matrix instead of fresh dot products (both
  * carry rounding noise of the size eps |x_i| |x_j|; the next round starts from fresh sums again). */
 struct RotRec { double cs, sn, a, b; };   /* x_c0' = cs x_c0 - a x_c1,  x_c1' = sn x_c0 + b x_c1;  sn == 0: no rotation */
-/* The same rotation on columns kept as scale x vector (x_c = s_c u_c): u_c0' = u_c0 - t1 u_c1, u_c1' = u_c1 + t2 u_c0 with
- * t1 = a s_c1 / (cs s_c0), t2 = sn s_c0 / (b s_c1), and s_c0' = cs s_c0, s_c1' = b s_c1: two multiply-adds per row instead of
- * two products and two multiply-adds; the scales (within 2^-8 .. 1 over the at most 15 rotations a column meets in a round)
- * are multiplied in once, before the columns are stored.  t1 == t2 == 0: no rotation. */
+/* The same rotation on columns kept as scale x vector (x_c = s_c u_c), as two shears in sequence: u_c0' = u_c0 - t1 u_c1, then
+ * u_c1' = u_c1 + t2 u_c0' with t1 = a s_c1 / (cs s_c0), t2 = a cs s_c0 / s_c1, and s_c0' = cs s_c0, s_c1' = b s_c1 / cs^2: two
+ * multiply-adds per row, in place, instead of two products and two multiply-adds; the scales (within 2^-8 .. 2^8 over the at
+ * most 15 rotations a column meets in a round) are multiplied in once, before the columns are stored.  t1 == t2 == 0: no
+ * rotation. */
 struct FastRot { double t1, t2; };
+
+/* 1 / z and 1 / sqrt(z) for z of ordinary size (no scaling, no fix-up of special values): hardware approximation, two
+ * Newton steps; the result is within an ulp or two of the exact one. */
+__device__ __forceinline__ double rcp_newton(double z) {
+  double y = __builtin_amdgcn_rcp(z);
+  y = fma(y, fma(-z, y, 1.), y); y = fma(y, fma(-z, y, 1.), y);
+  return y;
+}
+__device__ __forceinline__ double rsqrt_newton(double z) {
+  double y = __builtin_amdgcn_rsq(z);
+  y = fma(0.5 * y, fma(-z * y, y, 1.), y); y = fma(0.5 * y, fma(-z * y, y, 1.), y);
+  return y;
+}
 
 __device__ __forceinline__ void wave_lds_sync() {   /* LDS operations of one wavefront complete in order: only the compiler must not move them */
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
+
+/* Phase timing of the real Gram-space round (measurement builds only, -DHYK_JACOBI_TIMING): workgroup 1's first thread
+ * stamps the 100 MHz counter between the phases and adds the differences to the six 64-bit words behind the 16 bytes of
+ * `rotations` that the sweep uses. */
+#ifdef HYK_JACOBI_TIMING
+#define HYK_JDECL() long long hyk_t0 = 0, hyk_t1 = 0, hyk_t2 = 0, hyk_t3 = 0, hyk_t4 = 0, hyk_t5 = 0, hyk_t6 = 0
+#define HYK_JSTAMP(i) if (blockIdx.x == 1 && threadIdx.x == 0) { hyk_t##i = (long long)__builtin_readcyclecounter(); }
+#define HYK_JWAIT() asm volatile("s_waitcnt vmcnt(0)" ::: "memory")
+#define HYK_JREPORT() if (blockIdx.x == 1 && threadIdx.x == 0) { unsigned long long* w = reinterpret_cast<unsigned long long*>(rotations) + 2; \
+  atomicAdd(&w[0], (unsigned long long)(hyk_t1 - hyk_t0)); atomicAdd(&w[1], (unsigned long long)(hyk_t2 - hyk_t1)); atomicAdd(&w[2], (unsigned long long)(hyk_t3 - hyk_t2)); \
+  atomicAdd(&w[3], (unsigned long long)(hyk_t4 - hyk_t3)); atomicAdd(&w[4], (unsigned long long)(hyk_t5 - hyk_t4)); atomicAdd(&w[5], (unsigned long long)(hyk_t6 - hyk_t5)); }
+#else
+#define HYK_JDECL()
+#define HYK_JSTAMP(i)
+#define HYK_JWAIT()
+#define HYK_JREPORT()
+#endif
 
 /* CARRY: the products inside a block (x_i . x_j, i < j in the same block of BC columns) travel with the block from round
  * to round in `carry` (BC (BC - 1) / 2 doubles per block) instead of being summed again: the first round of a sweep (FULL)
@@ -426,10 +457,15 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
   __shared__ RotRec rot[STEPS][BC];
   __shared__ FastRot fast[STEPS][BC];
   __shared__ double scale[NC];
+  __shared__ double iscale[NC];
   __shared__ double fixed[BC][2];
   __shared__ int32_t pairCol[BC][2];
   __shared__ int32_t appliedAll;
-  const int i = blockIdx.x; int P, Q;
+  __shared__ int32_t stepsReady;
+  /* Workgroups go to the 8 XCDs in turn.  Pair i of a round takes its blocks over from the pairs i - 1 and i + 1 of the round
+   * before: with the pairs numbered so that neighbours run on the same XCD, most of what a workgroup loads was written
+   * through the L2 it sits behind. */
+  const int pairs = gridDim.x, i = (pairs % 8 == 0) ? (int)(blockIdx.x % 8) * (pairs / 8) + (int)(blockIdx.x / 8) : (int)blockIdx.x; int P, Q;
   if (i == 0) { P = nb - 1; Q = round; } else { P = (round + i) % (nb - 1); Q = (round - i + (nb - 1)) % (nb - 1); }
   if (P > Q) { const int t = P; P = Q; Q = t; }
   int col[NC]; bool live[NC];
@@ -440,20 +476,56 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
    * in the tail has nothing to do, except in the first round of a sweep, which also refreshes the carried products. */
   if (!FULL && col[0] >= top) { return; }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  HYK_JDECL(); HYK_JSTAMP(0);
   [[maybe_unused]] double carried = 0.;
   if constexpr (SLIM) { if (wave == 0 && lane < 2 * NW) { carried = carry[(int64_t)(lane < NW ? P : Q) * NW + lane % NW]; } }
   static_assert(PASSES == 1 || PASSES == 2, "all rows at once or in two halves");
   double x[NC][ROWS];
+  /* a thread owns pairs of adjacent rows: 16-byte loads and stores where the columns are 16-byte aligned (N even) */
+  static_assert(ROWS % 2 == 0, "rows are owned in adjacent pairs");
+  const bool vec2 = (N & 1) == 0 && (reinterpret_cast<uintptr_t>(B) & 15u) == 0;
+  auto row_of = [&](int pass, int m) { return 2 * (int)threadIdx.x + (m & 1) + (m >> 1) * 2 * THREADS + pass * ROWS * THREADS; };
   auto load_rows = [&](int pass) {
-    #pragma unroll
-    for (int c = 0; c < NC; ++c) {
+    if (vec2) {
       #pragma unroll
-      for (int m = 0; m < ROWS; ++m) { const int k = threadIdx.x + (pass * ROWS + m) * THREADS; x[c][m] = (live[c] && k < N) ? B[(int64_t)col[c] * N + k] : 0.; }
+      for (int c = 0; c < NC; ++c) {
+        #pragma unroll
+        for (int m = 0; m < ROWS; m += 2) {
+          const int k = row_of(pass, m); double2 v = { 0., 0. };
+          if (live[c] && k < N) { v = *reinterpret_cast<const double2*>(&B[(int64_t)col[c] * N + k]); }
+          x[c][m] = v.x; x[c][m + 1] = v.y;
+        }
+      }
+    } else {
+      #pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        #pragma unroll
+        for (int m = 0; m < ROWS; ++m) { const int k = row_of(pass, m); x[c][m] = (live[c] && k < N) ? B[(int64_t)col[c] * N + k] : 0.; }
+      }
+    }
+  };
+  auto store_rows = [&](int pass) {
+    if (vec2) {
+      #pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        #pragma unroll
+        for (int m = 0; m < ROWS; m += 2) {
+          const int k = row_of(pass, m);
+          if (live[c] && k < N) { *reinterpret_cast<double2*>(&B[(int64_t)col[c] * N + k]) = double2{ x[c][m], x[c][m + 1] }; }
+        }
+      }
+    } else {
+      #pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        #pragma unroll
+        for (int m = 0; m < ROWS; ++m) { const int k = row_of(pass, m); if (live[c] && k < N) { B[(int64_t)col[c] * N + k] = x[c][m]; } }
+      }
     }
   };
   #pragma unroll
   for (int pass = 0; pass < PASSES; ++pass) {
   load_rows(pass);
+  HYK_JWAIT(); HYK_JSTAMP(1);
   /* products numbered by diagonal: p = d NC + c stands for (c, (c + d) % NC), d = 0 .. NC / 2 (the last diagonal only for
    * c < NC / 2): every unordered pair once, and p splits back into the pair by shifts.  Summed over the wavefront 32 at a time. */
   #pragma unroll
@@ -464,7 +536,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
       int c0 = 0, c1 = 0; pair_of(chunk * CH + q, c0, c1);
       double sum = 0.;
       #pragma unroll
-      for (int m = 0; m < ROWS; ++m) { sum += x[c0][m] * x[c1][m]; }
+      for (int m = 0; m < ROWS; ++m) { sum = fma(x[c0][m], x[c1][m], sum); }
       v[q] = sum;
     }
     const double tot = wave_sum_swap<CH>(v);
@@ -477,14 +549,20 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
       int c0 = 0, c1 = 0; pair_of((NP / CH) * CH + q, c0, c1);
       double sum = 0.;
       #pragma unroll
-      for (int m = 0; m < ROWS; ++m) { sum += x[c0][m] * x[c1][m]; }
+      for (int m = 0; m < ROWS; ++m) { sum = fma(x[c0][m], x[c1][m], sum); }
       v[q] = sum;
     }
     const double tot = wave_sum_swap<TAIL>(v);
     if ((lane & (64 / TAIL - 1)) == 0) { double* slot = &part[wave][(NP / CH) * CH + lane / (64 / TAIL)]; *slot = pass == 0 ? tot : *slot + tot; }
   }
   }   /* passes */
+  HYK_JSTAMP(2);
+  if (threadIdx.x == 0) { stepsReady = 0; }
   __syncthreads();
+  HYK_JSTAMP(3);
+  /* From here on the wavefronts meet through `stepsReady` only: the first wavefront publishes the number of steps whose
+   * rotations are in `fast` (and STEPS + 1 once the scales and the rotation count are there as well), the others replay
+   * a step on their rows as soon as it is out, while the first one works on the next. */
   if (wave == 0) {
     for (int idx = lane; idx < NP; idx += 64) {
       double tot = 0.;
@@ -496,100 +574,148 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
     if constexpr (SLIM) {
       if (lane < 2 * NW) { int ci, cj; carried_pair<BC>(lane % NW, ci, cj); const int base = lane < NW ? 0 : BC; Gs[(base + ci) * GS + base + cj] = carried; Gs[(base + cj) * GS + base + ci] = carried; }
     }
-    if (lane < NC) { scale[lane] = 1.; }
+    if (lane < NC) { scale[lane] = 1.; iscale[lane] = 1.; }
     wave_lds_sync();
     int applied = 0; double worst = 0.;
-    for (int step = 0; step < STEPS; ++step) {
-      if (lane < BC) {
-        const int j = lane;
-        int c0, c1;
-        if constexpr (FULL) {
+    /* One rotation from the 2 x 2 Gram block (alpha, gre; gre, beta) of two columns that are kept as scale x vector
+     * (x = s u; s and 1 / s travel together).  rr is the plain rotation for the small matrix; fr the same rotation on the
+     * vectors as two shears in sequence, u0 <- u0 - t1 u1, then u1 <- u1 + t2 u0 with the new u0: t1 = sigma tan s1 / s0,
+     * t2 = sigma sin cos s0 / s1, and the scales become cos s0 and sigma s1 / cos (sigma = sign of gre).  Everything on
+     * this chain holds up the whole workgroup: reciprocal square roots from the hardware approximation and two Newton
+     * steps (operands within [1/4, 2]), no division (1 / cos and 1 / (1 + |d| / rho) come out of the second root). */
+    auto rotation = [&](double alpha, double beta, double gre, bool pairLive, bool counted, double& s0, double& is0, double& s1, double& is1, RotRec& rr, FastRot& fr, double& na, double& nbeta, bool mine) {
+      const double g2 = gre * gre, ab = alpha * beta;
+      if (mine && pairLive && counted && g2 > 0.) { worst = fmax(worst, fmin(g2 * __builtin_amdgcn_rcp(ab), 1.)); }   /* an indicator: the approximate reciprocal will do */
+      const bool rotate = pairLive && g2 > tol * tol * ab && g2 > 0.;
+      rr = RotRec{ 1., 0., 0., 1. }; fr = FastRot{ 0., 0. }; na = alpha; nbeta = beta;
+      if (rotate) {
+        /* d = beta - alpha, h = 2 |g|, both scaled by one power of two so that rho^2 = d^2 + h^2 lies in [1/4, 2):
+         * cos^2 = (1 + |d| / rho) / 2 >= 1/2, sin = sign(d) h / (2 rho cos), tan = sin / cos */
+        const double gabs = fabs(gre), d = beta - alpha, h = 2. * gabs;
+        const int e = __builtin_amdgcn_frexp_exp(fmax(fabs(d), h));
+        const double ds = ldexp(fabs(d), -e), hs = ldexp(h, -e);
+        const double q = rsqrt_newton(fma(ds, ds, hs * hs)), c2 = fma(0.5 * ds, q, 0.5), w = rsqrt_newton(c2);   /* w = 1 / cos */
+        const double cs = c2 * w, sn = copysign(0.5 * hs * q * w, d), tn = sn * w;
+        rr.cs = cs; rr.sn = sn; rr.a = gre < 0. ? -sn : sn; rr.b = gre < 0. ? -cs : cs;
+        const double shift = tn * gabs; na = alpha - shift; nbeta = beta + shift;
+        if (sn != 0.) {
+          if (mine) { ++applied; }
+          const double sw = gre < 0. ? -w : w;
+          fr.t1 = (sw * sn) * (s1 * is0); fr.t2 = (rr.a * cs) * (s0 * is1);
+          s0 = cs * s0; is0 = w * is0; s1 = sw * s1; is1 = rr.b * is1;
+        }
+      }
+    };
+    if constexpr (FULL) {
+      for (int step = 0; step < STEPS; ++step) {
+        if (lane < BC) {
+          const int j = lane;
           const int fa = (j == 0) ? NC - 1 : (step + j) % (NC - 1), fb = (j == 0) ? step : (step - j + (NC - 1)) % (NC - 1);
-          c0 = fa < fb ? fa : fb; c1 = fa < fb ? fb : fa;
-        } else { c0 = j; c1 = BC + (j + step) % BC; }
-        const double alpha = Gs[c0 * GS + c0], beta = Gs[c1 * GS + c1], gre = Gs[c0 * GS + c1];
-        const int i0 = (c0 < BC ? P : Q) * BC + (c0 % BC), i1 = (c1 < BC ? P : Q) * BC + (c1 % BC);
-        const bool pairLive = i0 < r && i1 < r && (i0 < top || i1 < top), counted = i0 < head || i1 < head;
-        const double g2 = gre * gre;
-        if (pairLive && counted) {
-          const double ab = alpha * beta;
-          if (ab > 0.) { if (g2 > worst * ab) { worst = g2 / ab; } } else if (g2 > 0.) { worst = fmax(worst, 1.); }
+          const int c0 = fa < fb ? fa : fb, c1 = fa < fb ? fb : fa;
+          const int i0 = (c0 < BC ? P : Q) * BC + (c0 % BC), i1 = (c1 < BC ? P : Q) * BC + (c1 % BC);
+          RotRec rr; FastRot fr; double na, nbeta, s0 = scale[c0], s1 = scale[c1], is0 = iscale[c0], is1 = iscale[c1];
+          rotation(Gs[c0 * GS + c0], Gs[c1 * GS + c1], Gs[c0 * GS + c1], i0 < r && i1 < r && (i0 < top || i1 < top), i0 < head || i1 < head, s0, is0, s1, is1, rr, fr, na, nbeta, true);
+          scale[c0] = s0; scale[c1] = s1; iscale[c0] = is0; iscale[c1] = is1;
+          rot[step][j] = rr; fast[step][j] = fr; fixed[j][0] = na; fixed[j][1] = nbeta; pairCol[j][0] = c0; pairCol[j][1] = c1;
         }
-        const bool rotate = pairLive && g2 > tol * tol * alpha * beta && g2 > 0.;
-        RotRec rr = { 1., 0., 0., 1. }; FastRot fr = { 0., 0. }; double na = alpha, nbeta = beta;
-        if (rotate) {
-          /* t = sign(d) h / (|d| + sqrt(d^2 + h^2)), d = beta - alpha, h = 2 |g|, scaled by one power of two (see the step kernel) */
-          const double gabs = fabs(gre), d = beta - alpha, h = 2. * gabs;
-          const int e = __builtin_amdgcn_frexp_exp(fmax(fabs(d), h));
-          const double ds = ldexp(fabs(d), -e), hs = ldexp(h, -e);
-          const double t = copysign(hs / (ds + sqrt(ds * ds + hs * hs)), d);
-          const double cs = rsqrt(1. + t * t), sn = cs * t, shift = t * gabs;
-          rr.cs = cs; rr.sn = sn; rr.a = gre < 0. ? -sn : sn; rr.b = gre < 0. ? -cs : cs;
-          na = alpha - shift; nbeta = beta + shift;
-          if (sn != 0.) {
-            ++applied;
-            const double s0 = scale[c0], s1 = scale[c1], n0 = cs * s0, n1 = rr.b * s1;
-            fr.t1 = rr.a * s1 / n0; fr.t2 = sn * s0 / n1; scale[c0] = n0; scale[c1] = n1;
-          }
+        wave_lds_sync();
+        /* G <- J^T G J, one lane per pair of pairs: the 2 x 2 block (rows of pair jr, columns of pair jc) takes the column
+         * rotation of jc and the row rotation of jr at once; the blocks are disjoint, so one pass does the step.  What a
+         * rotation fixes (its own block: alpha - t gamma, beta + t gamma, 0) is written as such. */
+        if (lane < BC * BC) {
+          const int jr = lane / BC, jc = lane % BC, r0 = pairCol[jr][0], r1 = pairCol[jr][1], k0 = pairCol[jc][0], k1 = pairCol[jc][1];
+          const RotRec rw = rot[step][jr], cl = rot[step][jc];
+          const double g00 = Gs[r0 * GS + k0], g01 = Gs[r0 * GS + k1], g10 = Gs[r1 * GS + k0], g11 = Gs[r1 * GS + k1];
+          const double h00 = cl.cs * g00 - cl.a * g01, h01 = cl.sn * g00 + cl.b * g01, h10 = cl.cs * g10 - cl.a * g11, h11 = cl.sn * g10 + cl.b * g11;
+          double y00 = rw.cs * h00 - rw.a * h10, y10 = rw.sn * h00 + rw.b * h10, y01 = rw.cs * h01 - rw.a * h11, y11 = rw.sn * h01 + rw.b * h11;
+          if (jr == jc && rw.sn != 0.) { y00 = fixed[jr][0]; y11 = fixed[jr][1]; y01 = 0.; y10 = 0.; }
+          Gs[r0 * GS + k0] = y00; Gs[r0 * GS + k1] = y01; Gs[r1 * GS + k0] = y10; Gs[r1 * GS + k1] = y11;
         }
-        rot[step][j] = rr; fast[step][j] = fr; fixed[j][0] = na; fixed[j][1] = nbeta; pairCol[j][0] = c0; pairCol[j][1] = c1;
+        wave_lds_sync();
       }
-      wave_lds_sync();
-      /* G <- J^T G J, one lane per pair of pairs: the 2 x 2 block (rows of pair jr, columns of pair jc) takes the column
-       * rotation of jc and the row rotation of jr at once; the blocks are disjoint, so one pass does the step.  What a
-       * rotation fixes (its own block: alpha - t gamma, beta + t gamma, 0) is written as such. */
-      if (lane < BC * BC) {
-        const int jr = lane / BC, jc = lane % BC, r0 = pairCol[jr][0], r1 = pairCol[jr][1], k0 = pairCol[jc][0], k1 = pairCol[jc][1];
-        const RotRec rw = rot[step][jr], cl = rot[step][jc];
-        const double g00 = Gs[r0 * GS + k0], g01 = Gs[r0 * GS + k1], g10 = Gs[r1 * GS + k0], g11 = Gs[r1 * GS + k1];
-        const double h00 = cl.cs * g00 - cl.a * g01, h01 = cl.sn * g00 + cl.b * g01, h10 = cl.cs * g10 - cl.a * g11, h11 = cl.sn * g10 + cl.b * g11;
-        double y00 = rw.cs * h00 - rw.a * h10, y10 = rw.sn * h00 + rw.b * h10, y01 = rw.cs * h01 - rw.a * h11, y11 = rw.sn * h01 + rw.b * h11;
-        if (jr == jc && rw.sn != 0.) { y00 = fixed[jr][0]; y11 = fixed[jr][1]; y01 = 0.; y10 = 0.; }
-        Gs[r0 * GS + k0] = y00; Gs[r0 * GS + k1] = y01; Gs[r1 * GS + k0] = y10; Gs[r1 * GS + k1] = y11;
+    } else {
+      /* Cross pairs only (step s pairs column j of the first block with column (j + s) % BC of the second): the small
+       * matrix lives in registers.  Lane (jr, jc) holds the 2 x 2 block rows {jr, BC + (jr + s) % BC} x columns
+       * {jc, BC + (jc + s) % BC}; the diagonal lanes (j, j) hold alpha, gamma, beta of pair j and work out its rotation,
+       * which the lanes of row j and of column j fetch by lane index (sigma cos and sin: two values say it all); after the
+       * update three of the four entries move one lane on to where the next step's pairing wants them.  No LDS memory on
+       * the chain from one step to the next. */
+      const int jr = (lane / BC) % BC, jc = lane % BC; const bool diag = jr == jc && lane < BC * BC;
+      double y00 = Gs[jr * GS + jc], y01 = Gs[jr * GS + BC + jc], y10 = Gs[(BC + jr) * GS + jc], y11 = Gs[(BC + jr) * GS + BC + jc];
+      double s0 = 1., is0 = 1., s1 = 1., is1 = 1.;
+      const int rowSrc = jr * (BC + 1), colSrc = jc * (BC + 1);
+      const int next01 = jr * BC + (jc + 1) % BC, next10 = ((jr + 1) % BC) * BC + jc, next11 = ((jr + 1) % BC) * BC + (jc + 1) % BC;
+      const int i0 = P * BC + jr;
+      for (int step = 0; step < STEPS; ++step) {
+        const int i1 = Q * BC + (jr + step) % BC;
+        RotRec rr; FastRot fr; double na, nbeta;
+        rotation(y00, y11, y01, i0 < r && i1 < r && (i0 < top || i1 < top), i0 < head || i1 < head, s0, is0, s1, is1, rr, fr, na, nbeta, diag);
+        if (diag) { fast[step][jr] = fr; }
+        const double rb = __shfl(rr.b, rowSrc, 64), rs = __shfl(rr.sn, rowSrc, 64), cb = __shfl(rr.b, colSrc, 64), cn = __shfl(rr.sn, colSrc, 64);
+        const double rc = fabs(rb), ra = rb < 0. ? -rs : rs, cc = fabs(cb), ca = cb < 0. ? -cn : cn;   /* b = sigma cos, a = sigma sin */
+        const double h00 = fma(cc, y00, -(ca * y01)), h01 = fma(cn, y00, cb * y01), h10 = fma(cc, y10, -(ca * y11)), h11 = fma(cn, y10, cb * y11);
+        double z00 = fma(rc, h00, -(ra * h10)), z10 = fma(rs, h00, rb * h10), z01 = fma(rc, h01, -(ra * h11)), z11 = fma(rs, h01, rb * h11);
+        if (diag && rr.sn != 0.) { z00 = na; z11 = nbeta; z01 = 0.; z10 = 0.; }
+        y00 = z00; y01 = __shfl(z01, next01, 64); y10 = __shfl(z10, next10, 64); y11 = __shfl(z11, next11, 64); s1 = __shfl(s1, next11, 64); is1 = __shfl(is1, next11, 64);
+        if (lane == 0) { __hip_atomic_store(&stepsReady, step + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP); }
       }
-      wave_lds_sync();
+      /* after BC steps every entry is back where it started */
+      if (lane < BC * BC) { Gs[jr * GS + jc] = y00; Gs[(BC + jr) * GS + BC + jc] = y11; }
+      if (diag) { scale[jr] = s0; scale[BC + jr] = s1; }
     }
     #pragma unroll
-    for (int off = BC / 2; off > 0; off >>= 1) { worst = fmax(worst, __shfl_xor(worst, off, 64)); applied += __shfl_xor(applied, off, 64); }
+    for (int off = 32; off > 0; off >>= 1) { worst = fmax(worst, __shfl_xor(worst, off, 64)); applied += __shfl_xor(applied, off, 64); }
     if (lane == 0) { report_cosine(rotations, worst); appliedAll = applied; if (applied > 0) { atomicAdd(rotations, applied); } }
+    wave_lds_sync();
     if constexpr (CARRY) {   /* the products inside the two blocks as the steps have left them */
       if (lane < 2 * NW) { int ci, cj; carried_pair<BC>(lane % NW, ci, cj); const int base = lane < NW ? 0 : BC; carry[(int64_t)(lane < NW ? P : Q) * NW + lane % NW] = Gs[(base + ci) * GS + base + cj]; }
     }
+    if (lane == 0) { __hip_atomic_store(&stepsReady, STEPS + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP); }
   }
-  __syncthreads();
-  if (appliedAll == 0) { return; }
+  HYK_JSTAMP(4);
+  auto wait_steps = [&](int want) {
+    if (wave != 0) { while (__hip_atomic_load(&stepsReady, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < want) { __builtin_amdgcn_s_sleep(1); } }
+  };
   /* replay the rotations on the rows of this thread (records fetched one ahead); the half in registers first */
   #pragma unroll
   for (int pass = PASSES - 1; pass >= 0; --pass) {
   if (pass != PASSES - 1) { load_rows(pass); }
-  FastRot cur = fast[0][0];
   #pragma unroll
-  for (int n = 0; n < STEPS * BC; ++n) {
-    const int step = n / BC, j = n % BC;
-    const FastRot fr = cur;
-    if (n + 1 < STEPS * BC) { cur = fast[(n + 1) / BC][(n + 1) % BC]; }
-    const int fa = (j == 0) ? NC - 1 : (step + j) % (NC - 1), fb = (j == 0) ? step : (step - j + (NC - 1)) % (NC - 1);
-    const int c0 = FULL ? (fa < fb ? fa : fb) : j, c1 = FULL ? (fa < fb ? fb : fa) : BC + (j + step) % BC;
-    if (fr.t1 != 0. || fr.t2 != 0.) {
+  for (int step = 0; step < STEPS; ++step) {
+    if (pass == PASSES - 1) { wait_steps(FULL ? STEPS + 1 : step + 1); }
+    /* Nothing of the compiler's moves across this point: not the records of later steps (fetched ahead they would wait in
+     * scratch memory), and not the arithmetic of this thread's rows either (it is needed only when the rows are stored, and
+     * would otherwise sink behind the waits for all later steps, which takes the overlap away). */
+    #pragma unroll
+    for (int c = 0; c < NC; ++c) {
       #pragma unroll
-      for (int m = 0; m < ROWS; ++m) {
-        const double pv = x[c0][m], qv = x[c1][m];
-        x[c0][m] = fma(-fr.t1, qv, pv); x[c1][m] = fma(fr.t2, pv, qv);
-      }
+      for (int m = 0; m < ROWS; ++m) { asm volatile("" : "+v"(x[c][m]) : : "memory"); }
+    }
+    FastRot recs[BC];   /* the records of a step come in together: one LDS latency per step, not one per rotation */
+    #pragma unroll
+    for (int j = 0; j < BC; ++j) { recs[j] = fast[step][j]; }
+    #pragma unroll
+    for (int j = 0; j < BC; ++j) {
+      const FastRot fr = recs[j];
+      const int fa = (j == 0) ? NC - 1 : (step + j) % (NC - 1), fb = (j == 0) ? step : (step - j + (NC - 1)) % (NC - 1);
+      const int c0 = FULL ? (fa < fb ? fa : fb) : j, c1 = FULL ? (fa < fb ? fb : fa) : BC + (j + step) % BC;
+      #pragma unroll
+      for (int m = 0; m < ROWS; ++m) { x[c0][m] = fma(-fr.t1, x[c1][m], x[c0][m]); x[c1][m] = fma(fr.t2, x[c0][m], x[c1][m]); }   /* t1 = t2 = 0: no rotation */
     }
   }
+  if (pass == PASSES - 1) { wait_steps(STEPS + 1); }
+  if (appliedAll == 0) { return; }   /* uniform over the workgroup: nothing was rotated, the columns stay as they are */
   #pragma unroll
   for (int c = 0; c < NC; ++c) {
     const double sc = scale[c];
     #pragma unroll
     for (int m = 0; m < ROWS; ++m) { x[c][m] *= sc; }
   }
-  #pragma unroll
-  for (int c = 0; c < NC; ++c) {
-    #pragma unroll
-    for (int m = 0; m < ROWS; ++m) { const int k = threadIdx.x + (pass * ROWS + m) * THREADS; if (live[c] && k < N) { B[(int64_t)col[c] * N + k] = x[c][m]; } }
-  }
+  HYK_JSTAMP(5);
+  store_rows(pass);
+  HYK_JWAIT(); HYK_JSTAMP(6);
   }   /* passes */
+  HYK_JREPORT();
 }
 
 /* The same round for complex factors.  The Gram matrix is Hermitian, G[c0][c1] = x_c0^H x_c1: NC (NC + 1) / 2 real parts

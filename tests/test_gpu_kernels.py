@@ -480,13 +480,14 @@ def test_gemm_fp64(gl, cplx, opA, opB, M, N, K):
 
 
 @pytest.mark.parametrize("variant,carry", [(0, 0), (0, 1), (1, 0), (2, 0), (2, 1)])
-@pytest.mark.parametrize("cplx,N,r", [(0, 300, 40), (0, 1000, 130), (0, 2048, 96), (0, 2500, 70), (0, 4096, 40), (1, 600, 50), (1, 2048, 40), (1, 3000, 24), (1, 4096, 36), (0, 64, 64), (0, 700, 20)])
+@pytest.mark.parametrize("cplx,N,r", [(0, 300, 40), (0, 1000, 130), (0, 2048, 96), (0, 2500, 70), (0, 4096, 40), (1, 600, 50), (1, 2048, 40), (1, 3000, 24), (1, 4096, 36), (0, 64, 64), (0, 700, 20), (0, 701, 40), (0, 1023, 64), (0, 2047, 33), (0, 2048, 256)])
 def test_jacobi_sweep_kernels(gl, variant, carry, cplx, N, r):
     """One-sided Jacobi sweeps on a graded N x r factor: every kernel behind hykJacobiSweep / hykJacobiSweepCarry (Gram-space
     rounds with blocks of 8 and of 4 columns, with and without the products inside a block carried from round to round in
     memory that starts as NaN, the step kernel, the pair kernel for few columns) must leave orthogonal columns whose norms are
     the singular values numpy finds, to 32 sqrt(r) eps of the largest (a column takes part in a few hundred rotations), and
-    whose span is unchanged."""
+    whose span is unchanged.  Odd N takes the kernels' element-wise loads (columns not 16-byte aligned); r = 256 gives the 16
+    block pairs of a round that are numbered by XCD."""
     from gpu_util import dev, host, ptr, stream, sync, zeros
     rng = np.random.default_rng(1000 * N + r + cplx)
     B = rng.standard_normal((N, r)) + (1j * rng.standard_normal((N, r)) if cplx else 0)
