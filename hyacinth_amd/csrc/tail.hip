@@ -747,7 +747,8 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t
   __shared__ double fixed[BC][2];
   __shared__ int32_t pairCol[BC][2];
   __shared__ int32_t appliedAll;
-  const int i = blockIdx.x; int P, Q;
+  __shared__ int32_t stepsReady;
+  const int pairs = gridDim.x, i = (pairs % 8 == 0) ? (int)(blockIdx.x % 8) * (pairs / 8) + (int)(blockIdx.x / 8) : (int)blockIdx.x; int P, Q;   /* neighbouring pairs on one XCD, as in the real kernel */
   if (i == 0) { P = nb - 1; Q = round; } else { P = (round + i) % (nb - 1); Q = (round - i + (nb - 1)) % (nb - 1); }
   if (P > Q) { const int t = P; P = Q; Q = t; }
   int col[NC]; bool live[NC];
@@ -771,6 +772,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t
     }
   };
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  HYK_JDECL(); HYK_JSTAMP(0);
   [[maybe_unused]] double carried = 0.;
   if constexpr (SLIM) { if (wave == 0 && lane < 4 * NW) { carried = carry[(int64_t)(lane < 2 * NW ? P : Q) * 2 * NW + lane % (2 * NW)]; } }
   /* sum q < NG: real part of pair p = q; q >= NG: imaginary part of pair p = q - NG + NC (the diagonal has none); pairs
@@ -779,6 +781,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t
   for (int pass = 0; pass < PASSES; ++pass) {
   if (pass > 0) { asm volatile("" ::: "memory"); }   /* the second half is loaded when the first is done with, not before */
   load_rows(pass);
+  HYK_JWAIT(); HYK_JSTAMP(1);
   #pragma unroll
   for (int chunk = 0; chunk < NP / CH + (TAIL > 0 ? 1 : 0); ++chunk) {
     constexpr int dummy = 0; (void)dummy;
@@ -789,8 +792,8 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t
       double sum = 0.;
       #pragma unroll
       for (int m = 0; m < ROWS; ++m) {
-        if (isIm) { sum += x[c0][m][0] * x[c1][m][1] - x[c0][m][1] * x[c1][m][0]; }
-        else { sum += x[c0][m][0] * x[c1][m][0] + x[c0][m][1] * x[c1][m][1]; }
+        if (isIm) { sum = fma(x[c0][m][0], x[c1][m][1], fma(-x[c0][m][1], x[c1][m][0], sum)); }
+        else { sum = fma(x[c0][m][0], x[c1][m][0], fma(x[c0][m][1], x[c1][m][1], sum)); }
       }
       v[e] = sum;
     }
@@ -798,7 +801,12 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t
     if ((lane & (64 / CH - 1)) == 0 && chunk * CH + lane / (64 / CH) < NP) { double* slot = &part[wave][chunk * CH + lane / (64 / CH)]; *slot = pass == 0 ? tot : *slot + tot; }
   }
   }   /* passes */
+  HYK_JSTAMP(2);
+  if (threadIdx.x == 0) { stepsReady = 0; }
   __syncthreads();
+  HYK_JSTAMP(3);
+  /* from here on the wavefronts meet through stepsReady only, as in the real kernel: the first wavefront publishes the
+   * number of steps whose rotations are in `rot`, the others replay a step while the next is worked out */
   if (wave == 0) {
     for (int idx = lane; idx < NP; idx += 64) {
       double tot = 0.;
@@ -829,18 +837,16 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t
         const int i0 = (c0 < BC ? P : Q) * BC + (c0 % BC), i1 = (c1 < BC ? P : Q) * BC + (c1 % BC);
         const bool pairLive = i0 < r && i1 < r && (i0 < top || i1 < top), counted = i0 < head || i1 < head;
         const double g2 = gre * gre + gim * gim;
-        if (pairLive && counted) {
-          const double ab = alpha * beta;
-          if (ab > 0.) { if (g2 > worst * ab) { worst = g2 / ab; } } else if (g2 > 0.) { worst = fmax(worst, 1.); }
-        }
+        if (pairLive && counted && g2 > 0.) { worst = fmax(worst, fmin(g2 * __builtin_amdgcn_rcp(alpha * beta), 1.)); }   /* an indicator: the approximate reciprocal will do */
         const bool rotate = pairLive && g2 > tol * tol * alpha * beta && g2 > 0.;
         RotRecC rr = { 1., 0., 0., 0., 1., 0. }; double na = alpha, nbeta = beta;
         if (rotate) {
-          const double gabs = sqrt(g2), inv = 1. / gabs, er = gre * inv, ei = gim * inv, d = beta - alpha, h = 2. * gabs;
+          /* as in the real kernel: no division and no library square root on the chain every wavefront waits for */
+          const double inv = rsqrt_newton(g2), gabs = g2 * inv, er = gre * inv, ei = gim * inv, d = beta - alpha, h = 2. * gabs;
           const int e = __builtin_amdgcn_frexp_exp(fmax(fabs(d), h));
           const double ds = ldexp(fabs(d), -e), hs = ldexp(h, -e);
-          const double t = copysign(hs / (ds + sqrt(ds * ds + hs * hs)), d);
-          const double cs = rsqrt(1. + t * t), sn = cs * t, shift = t * gabs;
+          const double q = rsqrt_newton(fma(ds, ds, hs * hs)), c2 = fma(0.5 * ds, q, 0.5), w = rsqrt_newton(c2);
+          const double cs = c2 * w, sn = copysign(0.5 * hs * q * w, d), shift = sn * w * gabs;
           rr.cs = cs; rr.sn = sn; rr.ar = sn * er; rr.ai = -sn * ei; rr.br = cs * er; rr.bi = -cs * ei;
           na = alpha - shift; nbeta = beta + shift;
           if (sn != 0.) { ++applied; }
@@ -866,6 +872,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t
         Gre[r1 * GS + k0] = y10.re; Gim[r1 * GS + k0] = y10.im; Gre[r1 * GS + k1] = y11.re; Gim[r1 * GS + k1] = y11.im;
       }
       wave_lds_sync();
+      if (lane == 0) { __hip_atomic_store(&stepsReady, step + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP); }
     }
     #pragma unroll
     for (int off = BC / 2; off > 0; off >>= 1) { worst = fmax(worst, __shfl_xor(worst, off, 64)); applied += __shfl_xor(applied, off, 64); }
@@ -876,29 +883,46 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t
         carry[(int64_t)(lane < 2 * NW ? P : Q) * 2 * NW + lane % (2 * NW)] = im ? Gim[(base + ci) * GS + base + cj] : Gre[(base + ci) * GS + base + cj];
       }
     }
+    wave_lds_sync();
+    if (lane == 0) { __hip_atomic_store(&stepsReady, STEPS + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP); }
   }
-  __syncthreads();
-  if (appliedAll == 0) { return; }
+  HYK_JSTAMP(4);
+  auto wait_steps = [&](int want) {
+    if (wave != 0) { while (__hip_atomic_load(&stepsReady, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) < want) { __builtin_amdgcn_s_sleep(1); } }
+  };
   #pragma unroll
   for (int pass = PASSES - 1; pass >= 0; --pass) {   /* the half in registers first */
   if (pass != PASSES - 1) { asm volatile("" ::: "memory"); load_rows(pass); }
-  RotRecC cur = rot[0][0];
   #pragma unroll
-  for (int n = 0; n < STEPS * BC; ++n) {
-    const int step = n / BC, j = n % BC;
-    const RotRecC rr = cur;
-    if (n + 1 < STEPS * BC) { cur = rot[(n + 1) / BC][(n + 1) % BC]; }
-    const int fa = (j == 0) ? NC - 1 : (step + j) % (NC - 1), fb = (j == 0) ? step : (step - j + (NC - 1)) % (NC - 1);
-    const int c0 = FULL ? (fa < fb ? fa : fb) : j, c1 = FULL ? (fa < fb ? fb : fa) : BC + (j + step) % BC;
-    if (rr.sn != 0.) {
+  for (int step = 0; step < STEPS; ++step) {
+    if (pass == PASSES - 1) { wait_steps(step + 1); }
+    /* nothing of the compiler's moves across this point (see the real kernel) */
+    #pragma unroll
+    for (int c = 0; c < NC; ++c) {
       #pragma unroll
-      for (int m = 0; m < ROWS; ++m) {
-        const double pr = x[c0][m][0], pi = x[c0][m][1]; const Cx q = { x[c1][m][0], x[c1][m][1] };
-        const Cx aq = cmul(rr.ar, rr.ai, q), bq = cmul(rr.br, rr.bi, q);
-        x[c0][m][0] = rr.cs * pr - aq.re; x[c0][m][1] = rr.cs * pi - aq.im; x[c1][m][0] = rr.sn * pr + bq.re; x[c1][m][1] = rr.sn * pi + bq.im;
+      for (int m = 0; m < ROWS; ++m) { asm volatile("" : "+v"(x[c][m][0]), "+v"(x[c][m][1]) : : "memory"); }
+    }
+    RotRecC recs[BC];   /* the records of a step come in together */
+    #pragma unroll
+    for (int j = 0; j < BC; ++j) { recs[j] = rot[step][j]; }
+    #pragma unroll
+    for (int j = 0; j < BC; ++j) {
+      const RotRecC rr = recs[j];
+      const int fa = (j == 0) ? NC - 1 : (step + j) % (NC - 1), fb = (j == 0) ? step : (step - j + (NC - 1)) % (NC - 1);
+      const int c0 = FULL ? (fa < fb ? fa : fb) : j, c1 = FULL ? (fa < fb ? fb : fa) : BC + (j + step) % BC;
+      if (rr.sn != 0.) {
+        #pragma unroll
+        for (int m = 0; m < ROWS; ++m) {
+          const double pr = x[c0][m][0], pi = x[c0][m][1], qr = x[c1][m][0], qi = x[c1][m][1];
+          x[c0][m][0] = fma(rr.cs, pr, fma(rr.ai, qi, -(rr.ar * qr))); x[c0][m][1] = fma(rr.cs, pi, fma(-rr.ar, qi, -(rr.ai * qr)));
+          x[c1][m][0] = fma(rr.sn, pr, fma(rr.br, qr, -(rr.bi * qi))); x[c1][m][1] = fma(rr.sn, pi, fma(rr.br, qi, rr.bi * qr));
+        }
       }
     }
   }
+  if (pass == PASSES - 1) { wait_steps(STEPS + 1); }
+  if (appliedAll == 0) { return; }   /* uniform over the workgroup: nothing was rotated */
+  HYK_JSTAMP(5);
   #pragma unroll
   for (int c = 0; c < NC; ++c) {
     #pragma unroll
@@ -907,7 +931,9 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t
       if (live[c] && k < N) { B[((int64_t)col[c] * N + k) * 2] = x[c][m][0]; B[((int64_t)col[c] * N + k) * 2 + 1] = x[c][m][1]; }
     }
   }
+  HYK_JWAIT(); HYK_JSTAMP(6);
   }   /* passes */
+  HYK_JREPORT();
 }
 
 template <bool CPLX>
