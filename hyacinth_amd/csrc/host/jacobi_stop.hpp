@@ -54,6 +54,16 @@ inline bool jacobi_output_settled(const std::vector<double>& before, const std::
   return moved <= 0.25 * eps * b[0] && gained <= outsideAfter / 32.;
 }
 
+/* The columns whose pairs the caller waits for: one past the last index among the `kept` largest column norms.  Pairs of two
+ * columns from there on are never handed out; what their cosines are says nothing about the vectors that are. */
+inline int jacobi_head(const std::vector<double>& norm, int kept) {
+  const int r = (int)norm.size(); if (kept <= 0 || kept >= r) { return r; }
+  std::vector<double> v(norm); std::nth_element(v.begin(), v.begin() + (kept - 1), v.end(), std::greater<double>());
+  const double nu = v[(size_t)(kept - 1)]; int head = 0;
+  for (int i = 0; i < r; ++i) { if (norm[(size_t)i] >= nu) { head = i + 1; } }
+  return head;
+}
+
 /* Columns a sweep may leave alone.  Let nu be the K-th largest column norm and b = max(nu^2, eps^2 sum of all squared norms).
  * The tail is the longest index range [top, r) whose squared norms sum to at most b / 1024; it is used only when it holds
  * at least half of the columns (a few large columns in front of a broad floor of small ones: a low-rank matrix plus noise),

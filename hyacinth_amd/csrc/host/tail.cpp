@@ -96,12 +96,13 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
       if (watchOutput) { HYH_CHECK(hipStreamSynchronize(s)); if (!hyh::ok()) { return 0; } }   /* `before` is on the host now */
       const int32_t top = watchOutput ? hyh::jacobi_tail_start(before, K, eps) : rank;   /* a broad floor of small columns is left alone */
       HYH_KERNEL(hykGramWorkspaceClear(s, counter.p, 64));
-      HYH_KERNEL(hykJacobiSweepTop(s, Complex, N, rank, top, top, B.as<double>(), rotateAbove, counter.as<int32_t>(), carry.as<double>())); ++used;
+      const int32_t headCols = watchOutput ? std::min(top, hyh::jacobi_head(before, K)) : rank;   /* cosines are watched on the pairs that involve a column that can be handed out */
+      HYH_KERNEL(hykJacobiSweepTop(s, Complex, N, rank, headCols, top, B.as<double>(), rotateAbove, counter.as<int32_t>(), carry.as<double>())); ++used;
       if (watchOutput) { fetch_norms(after); }
       struct { int32_t rotations, pad; double cosine2; } seen = { 0, 0, 0. };
       HYH_CHECK(hipMemcpyAsync(&seen, counter.p, sizeof(seen), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
       if (!hyh::ok()) { return 0; }
-      if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: %d rotations, largest cosine %.2le%s\n", used, seen.rotations, std::sqrt(seen.cosine2), top < rank ? " (floor of small columns left alone)" : ""); }
+      if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: %d rotations, largest cosine %.2le among pairs with a column before %d%s\n", used, seen.rotations, std::sqrt(seen.cosine2), headCols, top < rank ? " (floor of small columns left alone)" : ""); }
       if (hyh::jacobi_sweeps_done(seen.rotations, seen.cosine2, lastCosine2, rotateAbove)) { break; }
       if (watchOutput) {
         double moved[3] = { 0., 0., 0. }; const bool settled = hyh::jacobi_output_settled(before, after, K, eps, moved);

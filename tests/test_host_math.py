@@ -27,6 +27,8 @@ def hm():
     L.hm_jacobi_tail_start.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_double]
     L.hm_jacobi_tail_start.restype = C.c_int
     L.hm_jacobi_settled.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_double]
+    L.hm_jacobi_head.argtypes = [C.c_void_p, C.c_int, C.c_int]
+    L.hm_jacobi_head.restype = C.c_int
     L.hm_jacobi_settled.restype = C.c_int
     return L
 
@@ -233,6 +235,18 @@ def test_jacobi_output_settled_rule(hm):
     # a flat floor that keeps mixing (its norms move among themselves, their sum stays) does not hold the end back
     floor = np.concatenate([s[:10], np.full(30, 1e-9)]); mixed = floor.copy(); mixed[10:] = 1e-9 * np.sqrt(np.linspace(0.5, 1.5, 30))
     assert abs((mixed[10:] ** 2).sum() - (floor[10:] ** 2).sum()) < 1e-30 and settled(floor, mixed, 10, 1e-12) == 1
+
+
+def test_jacobi_head(hm):
+    """The columns whose cosines the host watches (host/jacobi_stop.hpp): one past the last index among the K largest norms."""
+    def head(norm, K):
+        a = np.ascontiguousarray(norm, dtype=np.float64)
+        return hm.hm_jacobi_head(_p(a), len(a), K)
+    s = 2.0 ** -np.arange(12.0)
+    assert head(s, 4) == 4 and head(s, 12) == 12 and head(s, 0) == 12 and head(s, 20) == 12
+    t = s.copy(); t[[3, 9]] = t[[9, 3]]                       # the fourth largest sits at index 9
+    assert head(t, 4) == 10 and head(t, 3) == 3
+    assert head(np.ones(6), 2) == 6                           # ties: every column that could be handed out counts
 
 
 def test_jacobi_tail_rule(hm):
