@@ -64,7 +64,7 @@ __device__ __forceinline__ void fetch_rows(const T* __restrict__ src, int valid,
 }
 
 __device__ __forceinline__ void store_panel(int8_t* dst, uint32_t packed, int valid, bool aligned) {
-  if (aligned && valid == Q_ROWS) { *reinterpret_cast<uint32_t*>(dst) = packed; }
+  if (aligned && valid == Q_ROWS) { __builtin_nontemporal_store(packed, reinterpret_cast<uint32_t*>(dst)); }   /* written once, read by another kernel: past the caches */
   else { for (int r = 0; r < valid; ++r) { dst[r] = (int8_t)(packed >> (8 * r)); } }
 }
 
