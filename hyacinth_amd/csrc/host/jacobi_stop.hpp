@@ -64,6 +64,26 @@ inline int jacobi_head(const std::vector<double>& norm, int kept) {
   return head;
 }
 
+/* How many leading columns of B (rows of the Cholesky factor, in pivot order) the SVD needs when only the K largest values
+ * and their vectors are handed out.  G = R^H R is the sum over the rows of R of their outer products, so leaving the rows
+ * from t on out of the SVD takes a positive semidefinite matrix of trace tau_t = sum_{j >= t} |row j|^2 off G: no eigenvalue
+ * moves up and none moves down by more than tau_t, hence 0 <= sigma_i - sigma'_i <= tau_t / (sigma_i + sigma'_i) <=
+ * tau_t / (2 sigma'_i) for the values sigma' of the truncated factor.  With tau_t <= eps sigma'_1 sigma'_K every value that is
+ * handed out is within eps sigma_1 / 2 of the true one, and the residual |A - A V V^H|^2 grows by at most tau_t.
+ * jacobi_columns_needed guesses t from the column norms (largest norm for sigma_1, K-th largest norm for sigma_K, a quarter of
+ * the bound for the guess: the norms of the columns are not the singular values); jacobi_truncation_holds is the test with
+ * the values the sweeps have found, and the caller goes on with all columns when it fails.  A noise floor under the wanted
+ * values, which costs a cyclic Jacobi method the most sweeps, is what this leaves out. */
+inline int jacobi_columns_needed(const std::vector<double>& norm, int K, double eps) {
+  const int r = (int)norm.size(); if (K < 1 || K >= r) { return r; }
+  std::vector<double> v(norm); std::nth_element(v.begin(), v.begin() + (K - 1), v.end(), std::greater<double>());
+  const double nuK = v[(size_t)(K - 1)], nu1 = *std::max_element(norm.begin(), norm.end()), bound = 0.25 * eps * nu1 * nuK;
+  double sum = 0.; int t = r;
+  while (t > K && sum + norm[(size_t)(t - 1)] * norm[(size_t)(t - 1)] <= bound) { sum += norm[(size_t)(t - 1)] * norm[(size_t)(t - 1)]; --t; }
+  return t;
+}
+inline bool jacobi_truncation_holds(double dropped2, double sigma1, double sigmaK, double eps) { return dropped2 <= eps * sigma1 * sigmaK; }
+
 /* Columns a sweep may leave alone.  Let nu be the K-th largest column norm and b = max(nu^2, eps^2 sum of all squared norms).
  * The tail is the longest index range [top, r) whose squared norms sum to at most b / 1024; it is used only when it holds
  * at least half of the columns (a few large columns in front of a broad floor of small ones: a low-rank matrix plus noise),

@@ -84,42 +84,63 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
      * below it costs sweeps and leaves the orthogonality where it was.  Nor below a sixteenth of the accuracy asked for:
      * cosines of that size move a singular value by less than eps / 2 of the largest one. */
     const double rotateAbove = std::max(std::max(machineEps, std::sqrt((double)N) * 2.220446049250313e-16), eps / 16.);
-    double lastCosine2 = 0.;
-    std::vector<double> before((size_t)rank), after((size_t)rank);
-    auto fetch_norms = [&](std::vector<double>& v) {
-      HYH_KERNEL(hykColumnNorms(s, Complex, N, rank, B.as<double>(), sigma.as<double>()));
-      HYH_CHECK(hipMemcpyAsync(v.data(), sigma.p, sizeof(double) * (size_t)rank, hipMemcpyDeviceToHost, s));
+    std::vector<double> before((size_t)rank), after, sig;
+    auto fetch_norms = [&](std::vector<double>& v, int32_t cols) {
+      v.resize((size_t)cols);
+      HYH_KERNEL(hykColumnNorms(s, Complex, N, cols, B.as<double>(), sigma.as<double>()));
+      HYH_CHECK(hipMemcpyAsync(v.data(), sigma.p, sizeof(double) * (size_t)cols, hipMemcpyDeviceToHost, s));
     };
-    const bool watchOutput = K < rank;   /* with every column handed out only the cosines can end the sweeps */
-    if (watchOutput && rank > 1) { fetch_norms(before); }
-    for (int32_t sw = 0; sw < maxSweeps && rank > 1; ++sw) {
-      if (watchOutput) { HYH_CHECK(hipStreamSynchronize(s)); if (!hyh::ok()) { return 0; } }   /* `before` is on the host now */
-      const int32_t top = watchOutput ? hyh::jacobi_tail_start(before, K, eps) : rank;   /* a broad floor of small columns is left alone */
-      HYH_KERNEL(hykGramWorkspaceClear(s, counter.p, 64));
-      const int32_t headCols = watchOutput ? std::min(top, hyh::jacobi_head(before, K)) : rank;   /* cosines are watched on the pairs that involve a column that can be handed out */
-      HYH_KERNEL(hykJacobiSweepTop(s, Complex, N, rank, headCols, top, B.as<double>(), rotateAbove, counter.as<int32_t>(), carry.as<double>())); ++used;
-      if (watchOutput) { fetch_norms(after); }
-      struct { int32_t rotations, pad; double cosine2; } seen = { 0, 0, 0. };
-      HYH_CHECK(hipMemcpyAsync(&seen, counter.p, sizeof(seen), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
-      if (!hyh::ok()) { return 0; }
-      if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: %d rotations, largest cosine %.2le among pairs with a column before %d%s\n", used, seen.rotations, std::sqrt(seen.cosine2), headCols, top < rank ? " (floor of small columns left alone)" : ""); }
-      if (hyh::jacobi_sweeps_done(seen.rotations, seen.cosine2, lastCosine2, rotateAbove)) { break; }
-      if (watchOutput) {
-        double moved[3] = { 0., 0., 0. }; const bool settled = hyh::jacobi_output_settled(before, after, K, eps, moved);
-        if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: the %d values handed out moved by at most %.2le, their columns gained %.2le of %.2le outside%s\n", used, K, moved[0], moved[1], moved[2], settled ? ": settled" : ""); }
-        if (settled) { break; }
-      }
-      lastCosine2 = seen.cosine2; before.swap(after);
+    /* Only the K largest values and their vectors are handed out.  Leaving the last rows of the Cholesky factor (the last
+     * columns of B) out of the SVD takes a positive semidefinite matrix of trace tau (the sum of their squared norms) off
+     * G: every eigenvalue moves down by at most tau, a singular value by at most tau / (2 sigma'), sigma' being the value
+     * found without them.  The columns of a noise floor under the values that are wanted are not worth their rotations:
+     * jacobi_columns_needed picks the prefix from the column norms, and what the sweeps then find must confirm it
+     * (jacobi_truncation_holds with the values themselves), or the sweeps go on with all columns. */
+    int32_t cols = rank; double dropped2 = 0.;
+    if (K < rank && rank > 1) {
+      fetch_norms(before, rank); HYH_CHECK(hipStreamSynchronize(s)); if (!hyh::ok()) { return 0; }
+      cols = hyh::jacobi_columns_needed(before, K, eps);
+      for (int32_t j = rank - 1; j >= cols; --j) { dropped2 = std::fma(before[(size_t)j], before[(size_t)j], dropped2); }
+      before.resize((size_t)cols);
+      if (handle->logger && cols < rank) { std::fprintf((FILE*)handle->logger, "GESVJ: the last %d of %d columns (squared norms %.2le in all) are left out of the sweeps\n", rank - cols, rank, dropped2); }
     }
-    HYH_KERNEL(hykColumnNorms(s, Complex, N, rank, B.as<double>(), sigma.as<double>()));
-    std::vector<double> sig((size_t)rank); HYH_CHECK(hipMemcpyAsync(sig.data(), sigma.p, sizeof(double) * (size_t)rank, hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
-    if (!hyh::ok()) { return 0; }
-    std::vector<int32_t> order((size_t)rank); std::iota(order.begin(), order.end(), 0);
+    for (;;) {
+      double lastCosine2 = 0.;
+      const bool watchOutput = K < cols;   /* with every column handed out only the cosines can end the sweeps */
+      for (int32_t sw = 0; sw < maxSweeps && cols > 1; ++sw) {
+        const int32_t top = watchOutput ? hyh::jacobi_tail_start(before, K, eps) : cols;   /* a broad floor of small columns is left alone */
+        HYH_KERNEL(hykGramWorkspaceClear(s, counter.p, 64));
+        const int32_t headCols = watchOutput ? std::min(top, hyh::jacobi_head(before, K)) : cols;   /* cosines are watched on the pairs that involve a column that can be handed out */
+        HYH_KERNEL(hykJacobiSweepTop(s, Complex, N, cols, headCols, top, B.as<double>(), rotateAbove, counter.as<int32_t>(), carry.as<double>())); ++used;
+        if (watchOutput) { fetch_norms(after, cols); }
+        struct { int32_t rotations, pad; double cosine2; } seen = { 0, 0, 0. };
+        HYH_CHECK(hipMemcpyAsync(&seen, counter.p, sizeof(seen), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
+        if (!hyh::ok()) { return 0; }
+        if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: %d rotations, largest cosine %.2le among pairs with a column before %d%s\n", used, seen.rotations, std::sqrt(seen.cosine2), headCols, top < cols ? " (floor of small columns left alone)" : ""); }
+        if (hyh::jacobi_sweeps_done(seen.rotations, seen.cosine2, lastCosine2, rotateAbove)) { break; }
+        if (watchOutput) {
+          double moved[3] = { 0., 0., 0. }; const bool settled = hyh::jacobi_output_settled(before, after, K, eps, moved);
+          if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: the %d values handed out moved by at most %.2le, their columns gained %.2le of %.2le outside%s\n", used, K, moved[0], moved[1], moved[2], settled ? ": settled" : ""); }
+          if (settled) { break; }
+        }
+        lastCosine2 = seen.cosine2; before.swap(after);
+      }
+      fetch_norms(sig, cols); HYH_CHECK(hipStreamSynchronize(s));
+      if (!hyh::ok()) { return 0; }
+      if (cols == rank) { break; }
+      std::vector<double> top(sig); std::nth_element(top.begin(), top.begin() + (K - 1), top.end(), std::greater<double>());
+      const double sigmaK = top[(size_t)(K - 1)], sigma1 = *std::max_element(sig.begin(), sig.end());
+      if (hyh::jacobi_truncation_holds(dropped2, sigma1, sigmaK, eps)) { break; }
+      if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ: value %d is %.2le: the columns left out weigh too much, the sweeps go on with all %d\n", K, sigmaK, rank); }
+      cols = rank; dropped2 = 0.; fetch_norms(before, rank); HYH_CHECK(hipStreamSynchronize(s)); if (!hyh::ok()) { return 0; }
+    }
+    std::vector<int32_t> order((size_t)cols); std::iota(order.begin(), order.end(), 0);
     std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return sig[a] > sig[b]; });
-    /* rank cut (reference: find_srank_kernel, src/gram_evd.cu:44-70): keep i < K while sum_{j>=i} sigma_j^2 > eps^2 sum_j sigma_j^2 */
-    std::vector<double> suffix((size_t)rank + 1, 0.); for (int32_t i = rank - 1; i >= 0; --i) { const double v = sig[order[i]]; suffix[i] = std::fma(v, v, suffix[i + 1]); }
+    /* rank cut (reference: find_srank_kernel, src/gram_evd.cu:44-70): keep i < K while sum_{j>=i} sigma_j^2 > eps^2 sum_j sigma_j^2;
+     * the columns left out count with what they weigh (the sum over all values is the trace of G either way) */
+    std::vector<double> suffix((size_t)cols + 1, dropped2); for (int32_t i = cols - 1; i >= 0; --i) { const double v = sig[order[i]]; suffix[i] = std::fma(v, v, suffix[i + 1]); }
     const double resid = eps * eps * suffix[0]; std::vector<double> Sout((size_t)K, 0.); int32_t kept = 0;
-    for (int32_t i = 0; i < K; ++i) { if (i < rank && resid < suffix[i]) { Sout[i] = sig[order[i]]; ++kept; } }
+    for (int32_t i = 0; i < K; ++i) { if (i < cols && resid < suffix[i]) { Sout[i] = sig[order[i]]; ++kept; } }
     const int32_t svdRank = kept; rank = std::min(rank, kept);
     hyh::Scratch dS(handle, sizeof(double) * (size_t)K), dOrder(handle, sizeof(int32_t) * (size_t)std::max(1, rank));
     if (!hyh::ok()) { return 0; }

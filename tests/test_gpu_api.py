@@ -254,3 +254,53 @@ def test_timer_segments(oracle):
     ha.lib().hyacinSync_TimerSegments(C.byref(h), ms, 4)
     assert ms[0] > 0 and ms[1] > 0 and ms[2] == 0 and ms[3] == 0
     ha.destroy_handle(h)
+
+
+def _kahan(n, c):
+    s = np.sqrt(1.0 - c * c)
+    return (s ** np.arange(n))[:, None] * (np.triu(-c * np.ones((n, n)), 1) + np.eye(n)) * (1.0 - 1e-3 * np.arange(n))[None, :]
+
+
+@pytest.mark.parametrize("case", ["floor left out", "floor taken back in"])
+def test_gevd_leaves_out_floor_columns(case, capfd, monkeypatch):
+    """hyacinXGevd (src/gram_evd.cu:94-142) with fewer values wanted than the Cholesky factor has rows: the rows of a noise
+    floor are left out of the Jacobi sweeps when what they weigh is below eps sigma_1 sigma_K (first case: the log says so,
+    and the values still agree with numpy's to 10 eps sigma_1).  The choice is made from the row norms; in the second case
+    they mislead (a Kahan matrix: its last singular value is 3e-5 of its last row's norm), the test with the values found
+    fails, and the sweeps must go on with all rows: value K is then the floor's, not the Kahan block's."""
+    import hyacinth_amd as ha
+    from gpu_util import dev, zeros, ptr, stream, sync, host
+    rng = np.random.default_rng(8)
+    if case == "floor left out":
+        N, K, eps = 300, 20, 1e-8
+        V = haar(rng, N, N, False)
+        R = (np.concatenate([10.0 ** -np.linspace(0, 6, 40), np.full(N - 40, 1e-8)])[:, None]) * V.T     # singular values: 40 graded ones over a floor
+    else:
+        N, K, eps = 64, 24, 1e-6
+        R = np.zeros((N, N))
+        R[:24, :24] = _kahan(24, 0.6)
+        R[24:, 24:] = 1e-5 * np.eye(N - 24)
+    G = R.T @ R
+    want = np.linalg.svd(R, compute_uv=False)
+    monkeypatch.setenv("HYACIN_VERBOSE", "1")
+    h = ha.create_handle(stream=stream().value)
+    try:
+        dG, dS, dX = dev(np.ascontiguousarray(G.T)), zeros(8 * K), zeros(8 * N * K)
+        capfd.readouterr()
+        rank = ha.lib().hyacinXGevd(C.byref(h), eps, N, K, 0, ptr(dX), N, ptr(dS), 0, ptr(dG), N)
+        sync()
+        C.CDLL(None).fflush(None)                       # the log goes through the C library's buffered stdout
+        log = capfd.readouterr().out
+    finally:
+        ha.destroy_handle(h)
+    S = host(dS, np.float64, (K,))
+    X = host(dX, np.float64, (K, N))[:rank]
+    assert "are left out of the sweeps" in log
+    assert ("go on with all" in log) == (case == "floor taken back in")
+    assert 0 < rank <= K and np.abs(S[:rank] - want[:rank]).max() <= 10 * eps * want[0]
+    assert np.abs(X @ X.T - np.eye(rank)).max() <= max(1e-12, eps)            # rotations stop at cosines of eps / 16
+    if case == "floor taken back in":
+        assert rank >= 23 and abs(S[rank - 1] - want[rank - 1]) <= 1e-11 and (rank < 24 or abs(S[23] - 1e-5) <= 1e-11)
+    # the basis captures the matrix up to the values that are not handed out
+    resid2 = (R ** 2).sum() - ((R @ X.T) ** 2).sum()
+    assert abs(resid2 - (want[rank:] ** 2).sum()) <= (10 * eps) ** 2 * (want ** 2).sum() + 1e-6 * (want[rank:] ** 2).sum()

@@ -29,6 +29,10 @@ def hm():
     L.hm_jacobi_settled.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_double]
     L.hm_jacobi_head.argtypes = [C.c_void_p, C.c_int, C.c_int]
     L.hm_jacobi_head.restype = C.c_int
+    L.hm_jacobi_columns_needed.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_double]
+    L.hm_jacobi_columns_needed.restype = C.c_int
+    L.hm_jacobi_truncation_holds.argtypes = [C.c_double, C.c_double, C.c_double, C.c_double]
+    L.hm_jacobi_truncation_holds.restype = C.c_int
     L.hm_jacobi_settled.restype = C.c_int
     return L
 
@@ -247,6 +251,31 @@ def test_jacobi_head(hm):
     t = s.copy(); t[[3, 9]] = t[[9, 3]]                       # the fourth largest sits at index 9
     assert head(t, 4) == 10 and head(t, 3) == 3
     assert head(np.ones(6), 2) == 6                           # ties: every column that could be handed out counts
+
+
+def test_jacobi_columns_needed(hm):
+    """Which prefix of the factor's columns the SVD works on (host/jacobi_stop.hpp): the trailing columns whose squared norms
+    sum to at most eps nu_1 nu_K / 4 are left out, never fewer than K columns kept.  The bound behind it, checked on an
+    explicit matrix: dropping rows of R of squared Frobenius norm tau moves every singular value down, by at most
+    tau / (2 sigma') (sigma' the value without them)."""
+    rng = np.random.default_rng(11)
+    def need(norm, K, eps):
+        a = np.ascontiguousarray(norm, dtype=np.float64)
+        return hm.hm_jacobi_columns_needed(_p(a), len(a), K, eps)
+    floor = np.concatenate([10.0 ** -np.arange(8.0), np.full(100, 1e-9)])        # 8 graded columns over a floor of 100
+    # K = 4: nu_1 = 1, nu_4 = 1e-3; eps = 1e-6 allows 2.5e-10: all of the floor (1e-16) and the columns below it
+    t = need(floor, 4, 1e-6)
+    assert 4 <= t <= 8 and (floor[t:] ** 2).sum() <= 0.25e-6 * 1.0 * 1e-3 < (floor[t - 1:] ** 2).sum()
+    assert need(floor, 4, 1e-16) == 108                                          # nothing is small enough: 2.5e-20 < 1e-18
+    assert need(floor, 4, 4.1e-12) == 8                                          # exactly the floor (100 x 1e-18 = 1e-16 <= 1.025e-15 ... and 1e-14 more is too much)
+    assert need(floor, 108, 1.0) == 108 and need(floor, 0, 1.0) == 108           # every column wanted / no K: all
+    assert need(np.full(20, 1.0), 5, 1.0) >= 5                                   # never fewer than K
+    # the perturbation bound on an explicit factor: rows of R in pivot order, graded, the last 30 small
+    R = rng.standard_normal((40, 60)) * np.concatenate([2.0 ** -np.arange(10.0), np.full(30, 1e-6)])[:, None]
+    full = np.linalg.svd(R, compute_uv=False); cut = np.linalg.svd(R[:10], compute_uv=False); tau = (R[10:] ** 2).sum()
+    assert np.all(full[:10] >= cut * (1 - 1e-15)) and np.all(full[:10] - cut <= tau / (2 * cut) * (1 + 1e-9))
+    assert hm.hm_jacobi_truncation_holds(tau, cut[0], cut[9], tau / (cut[0] * cut[9]) * 1.01) == 1
+    assert hm.hm_jacobi_truncation_holds(tau, cut[0], cut[9], tau / (cut[0] * cut[9]) * 0.99) == 0
 
 
 def test_jacobi_tail_rule(hm):
