@@ -465,7 +465,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
   /* Workgroups go to the 8 XCDs in turn.  Pair i of a round takes its blocks over from the pairs i - 1 and i + 1 of the round
    * before: with the pairs numbered so that neighbours run on the same XCD, most of what a workgroup loads was written
    * through the L2 it sits behind. */
-  const int pairs = gridDim.x, i = (pairs % 8 == 0) ? (int)(blockIdx.x % 8) * (pairs / 8) + (int)(blockIdx.x / 8) : (int)blockIdx.x; int P, Q;
+  const int pairs = gridDim.x, xcd = blockIdx.x % 8, i = xcd * (pairs / 8) + (xcd < pairs % 8 ? xcd : pairs % 8) + (int)(blockIdx.x / 8); int P, Q;   /* XCD x takes a contiguous range of pairs */
   if (i == 0) { P = nb - 1; Q = round; } else { P = (round + i) % (nb - 1); Q = (round - i + (nb - 1)) % (nb - 1); }
   if (P > Q) { const int t = P; P = Q; Q = t; }
   int col[NC]; bool live[NC];
@@ -748,7 +748,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_cplx_kernel(int32_t
   __shared__ int32_t pairCol[BC][2];
   __shared__ int32_t appliedAll;
   __shared__ int32_t stepsReady;
-  const int pairs = gridDim.x, i = (pairs % 8 == 0) ? (int)(blockIdx.x % 8) * (pairs / 8) + (int)(blockIdx.x / 8) : (int)blockIdx.x; int P, Q;   /* neighbouring pairs on one XCD, as in the real kernel */
+  const int pairs = gridDim.x, xcd = blockIdx.x % 8, i = xcd * (pairs / 8) + (xcd < pairs % 8 ? xcd : pairs % 8) + (int)(blockIdx.x / 8); int P, Q;   /* neighbouring pairs on one XCD, as in the real kernel */
   if (i == 0) { P = nb - 1; Q = round; } else { P = (round + i) % (nb - 1); Q = (round - i + (nb - 1)) % (nb - 1); }
   if (P > Q) { const int t = P; P = Q; Q = t; }
   int col[NC]; bool live[NC];
