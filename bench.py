@@ -9,6 +9,8 @@ take the storage order of A) on a synthetic matrix that is already resident in H
              reports them for what it launched) / time against the dense INT8 MFMA peak; board power and shader clock
              sampled while that kernel runs back to back
   tsvd_fit_ms  the fit the configuration names, wall clock, median of 5 after 2 warm-ups
+  fit_gaussian_matrix, other_workloads  (default workload only) the same fit on the Gaussian matrix of the same shape, and the
+             other configurations in short: step time, TFLOP/s, share of the INT8 peak, their fit
   cpu_baseline  the same limb / CRT algorithm compiled for the host (the oracle), timed on a row sample of the same matrix,
              with OpenBLAS DSYRK / ZHERK on the same sample and LAPACK syevd / heevd on its N x N Gram beside it
 
@@ -223,6 +225,58 @@ class Telemetry:
                 "sclk_mhz_sysfs": (sum(self.mhz) / len(self.mhz)) if self.mhz else None}
 
 
+def brief(torch, ha, L, name, steps, warmup):
+    """The other workloads in short, for the same record: Gram-build step time, effective TFLOP/s, the contraction kernel's
+    share of the INT8 peak, and the fit the configuration names (median of 5 after 2 warm-ups)."""
+    num, at, opA, M, N, K, eps, alg, fit_name, desc = WORKLOADS[name]
+    cplx = at & 1
+    h = ha.create_handle(stream=torch.cuda.current_stream().cuda_stream, GramMatrixAlgorithm=alg)
+    try:
+        A, lda = make_workload(torch, name)
+        op = opA.encode()
+        u, cP, lP, stride = ha.herk_batch_init(h, eps, M, N, at)
+        seg = min(h.GramSegmentK, M) if h.GramSegmentK > 0 else M
+        batches, lastM = (M + seg - 1) // seg, M - (M - 1) // seg * seg
+        vexp = torch.zeros((batches + 1) * N, dtype=torch.int32, device="cuda")
+        Cq = torch.zeros(cP * lP * stride, dtype=torch.int64, device="cuda")
+        pA, pV, pC = C.c_void_p(A.data_ptr()), C.c_void_p(vexp.data_ptr()), C.c_void_p(Cq.data_ptr())
+
+        def step():
+            L.hykQuantizeScaleBatchOp(C.byref(h), op, batches, seg, lastM, N, at, pA, lda, u, pV)
+            L.hykHerkBatchOp(C.byref(h), op, batches, seg, lastM, N, at, pA, lda, u, pV, 0, lP, pC)
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        L.hykGramProfile(1)
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+        kms, kn = C.c_double(), C.c_int32()
+        L.hykGramProfileRead(C.byref(kms), C.byref(kn))
+        L.hykGramProfile(0)
+        plan = ha.HerkPlan()
+        assert L.hykLastHerkPlan(C.byref(plan)) == 0 and L.hykLastStatus() == 0
+        t_kernel = kms.value / 1e3 / steps
+        real = torch.float64 if at in (0, 1) else (torch.float32 if at in (2, 3) else torch.float16)
+        S = torch.zeros(max(K, N), dtype=torch.float64, device="cuda")
+        V = torch.zeros(N * K * (2 if cplx else 1), dtype=real, device="cuda")
+        times, rank = [], 0
+        for _ in range(7):
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            rank = getattr(L, fit_name)(C.byref(h), eps, op, M, N, K, pA, lda, C.c_void_p(S.data_ptr()), C.c_void_p(V.data_ptr()), N, 0, at)
+            torch.cuda.synchronize()
+            times.append((time.perf_counter() - t1) * 1e3)
+        assert L.hykLastStatus() == 0
+        return {"workload": "%s: %s" % (name, desc), "ms_per_step": dt * 1e3, "value": M * N * (N + 1) * (4 if cplx else 1) / dt / 1e12, "unit": "TFLOP/s",
+                "pct_int8_mfma_peak": 100.0 * (plan.int8Ops / t_kernel / 1e12 if t_kernel > 0 else 0.0) / INT8_PEAK_TOPS, "contraction_calls": plan.gramCalls,
+                "fit": {"call": fit_name, "K": K, "rank": rank, "ms": sorted(times[2:])[len(times[2:]) // 2]}}
+    finally:
+        ha.destroy_handle(h)
+
+
 def measured_traffic(workload):
     """HBM bytes per launch of the contraction kernel from the rocprofv3 counter summary under profiles/, if that summary was
     made from the kernel source as it is now (it records the SHA-256 of gram_mfma.hip); None otherwise."""
@@ -247,6 +301,7 @@ def main():
     ap.add_argument("--no-fit", action="store_true", help="skip the end-to-end fit timing")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-stages", action="store_true", help="skip the separate timing of the HBM-bound stages (exponents, quantize, dequantize)")
+    ap.add_argument("--no-others", action="store_true", help="skip the short measurements of the other workloads (configurations 1 to 5) that the default run appends")
     ap.add_argument("--no-ceiling", action="store_true", help="skip the register-only MFMA ceiling and the power / clock sampling")
     ap.add_argument("--cpu-rows", type=int, default=65536, help="rows of the workload the CPU baseline is timed on (about 15 s of host work)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -434,6 +489,7 @@ def main():
     }
     if fit_gauss:
         out["fit_gaussian_matrix"] = fit_gauss
+    sample = None
     if not a.no_cpu:
         rows = min(a.cpu_rows, M)
         if opA == "N":
@@ -447,8 +503,24 @@ def main():
             import numpy as np
             sample = sample[..., 0] + 1j * sample[..., 1]
             sample = sample.astype(np.complex128 if at == 1 else np.complex64)
+    if a.workload == "target" and not a.no_others and not a.no_fit:
+        # configurations 1 to 5 in short, so that one record holds every workload (about half a minute in all)
+        del A, vexp, Cq
+        S = V = None
+        ha.destroy_handle(h)
+        h = None
+        others = []
+        for name in ("cfg1", "cfg2", "cfg3", "cfg4", "cfg5"):
+            torch.cuda.empty_cache()
+            try:
+                others.append(brief(torch, ha, L, name, a.steps, a.warmup))
+            except Exception as e:   # the headline must not be lost over one of them
+                others.append({"workload": name, "error": repr(e)})
+        out["other_workloads"] = others
+    if sample is not None:
         out["cpu_baseline"] = cpu_baseline(sample, at, plan_alg, order, u)
-    ha.destroy_handle(h)
+    if h is not None:
+        ha.destroy_handle(h)
     print(json.dumps(out))
 
 
