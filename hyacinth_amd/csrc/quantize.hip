@@ -18,6 +18,7 @@
  * One thread quantizes four consecutive rows of one column and stores one
  * packed dword per panel (byte stores when B + row is not 4-byte aligned).
  */
+#include <type_traits>
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 #include "hyk_common.h"
@@ -74,24 +75,62 @@ template <typename E>
 __device__ __forceinline__ void limbs_rows(int32_t order, int32_t expon, const typename E::T (&raw)[Q_ROWS], int valid, int8_t* out, bool aligned, int64_t strideB) {
   constexpr int GROUPS = E::cplx ? 3 : 1;
   if (expon == HYK_INT_MAX) { for (int p = 0; p < order * GROUPS; ++p) { store_panel(out + p * strideB, 0u, valid, aligned); } return; }
-  hyk::I96 q[GROUPS][Q_ROWS];
-  #pragma unroll
-  for (int r = 0; r < Q_ROWS; ++r) {
-    hyk::Dec re{ 0, 0, 0 }, im{ 0, 0, 0 }; E::load(&raw[r], re, im);
-    if constexpr (E::cplx) { hyk::I96 a = hyk::round_scaled(re, expon), b = hyk::round_scaled(im, expon); q[0][r] = hyk::i96_add(a, b); q[1][r] = a; q[2][r] = b; }
-    else { q[0][r] = hyk::round_scaled(re, expon); }
-  }
-  #pragma unroll
-  for (int g = 0; g < GROUPS; ++g) {
-    uint32_t carry[Q_ROWS] = { 0, 0, 0, 0 };
+  /* Small values first: q = rint(x 2^expon) is exact in a double while |q| < 2^50 (every plan for FP16 / FP32 storage, and
+   * FP64 up to six digits), and its two's complement bytes then come from a 32-bit integer (|q| < 2^29: FP16 storage, three
+   * digits) or a 64-bit one instead of the 96-bit path. */
+  { double re[Q_ROWS], im[Q_ROWS]; double big = 0.;
     #pragma unroll
-    for (int l = 0; l < 12; ++l) {
-      if (l < order) {
-        uint32_t packed = 0;
+    for (int r = 0; r < Q_ROWS; ++r) {
+      double a = 0., b = 0.; E::load_f64(&raw[r], a, b);
+      re[r] = __builtin_rint(__builtin_ldexp(a, expon)); im[r] = __builtin_rint(__builtin_ldexp(b, expon));
+      big = __builtin_fmax(big, __builtin_fmax(__builtin_fabs(re[r]), __builtin_fabs(im[r])));
+      if (!(re[r] == re[r]) || !(im[r] == im[r])) { big = __builtin_inf(); }   /* a NaN goes the long way like anything else out of range */
+    }
+    /* one group at a time (a rolled loop: unrolled, the 3 x order panel addresses and digit words of a complex element cost
+     * more registers, and with them resident wavefronts, than the loop costs instructions); the digits of a group unrolled */
+    auto digits = [&](auto zero, auto signShift, auto bytes) {
+      using Q = decltype(zero);
+      #pragma unroll 1
+      for (int g = 0; g < GROUPS; ++g) {
+        Q q[Q_ROWS];
         #pragma unroll
-        for (int r = 0; r < Q_ROWS; ++r) { uint32_t t = hyk::i96_byte(q[g][r], l) + carry[r]; packed |= (t & 0xffu) << (8 * r); carry[r] = (t >> 8) + ((t >> 7) & 1u); }
-        store_panel(out + (int64_t)(g * order + l) * strideB, packed, valid, aligned);
+        for (int r = 0; r < Q_ROWS; ++r) { const Q a = (Q)re[r]; if constexpr (E::cplx) { const Q b = (Q)im[r]; q[r] = g == 0 ? a + b : (g == 1 ? a : b); } else { q[r] = a; } }
+        uint32_t carry[Q_ROWS] = { 0, 0, 0, 0 }; int8_t* dst = out + (int64_t)(g * order) * strideB;
+        #pragma unroll
+        for (int l = 0; l < 12; ++l) {
+          if (l < order) {
+            uint32_t packed = 0;
+            #pragma unroll
+            for (int r = 0; r < Q_ROWS; ++r) {
+              const uint32_t t = (uint32_t)((q[r] >> (l < bytes() ? 8 * l : signShift())) & 0xff) + carry[r];
+              packed |= (t & 0xffu) << (8 * r); carry[r] = (t >> 8) + ((t >> 7) & 1u);
+            }
+            store_panel(dst, packed, valid, aligned); dst += strideB;
+          }
+        }
       }
+    };
+    if (big < 0x1p29) { digits((int32_t)0, std::integral_constant<int, 31>{}, std::integral_constant<int, 4>{}); return; }
+    if (big < 0x1p50) { digits((long long)0, std::integral_constant<int, 63>{}, std::integral_constant<int, 8>{}); return; }
+  }
+  /* the long way: 96-bit integers, one group at a time (the values are worked out again per group: this path is rare, and
+   * holding all three groups would set the register count of the whole kernel) */
+  #pragma unroll 1
+  for (int g = 0; g < GROUPS; ++g) {
+    hyk::I96 q[Q_ROWS];
+    #pragma unroll
+    for (int r = 0; r < Q_ROWS; ++r) {
+      hyk::Dec re{ 0, 0, 0 }, im{ 0, 0, 0 }; E::load(&raw[r], re, im);
+      if constexpr (E::cplx) { q[r] = g == 0 ? hyk::i96_add(hyk::round_scaled(re, expon), hyk::round_scaled(im, expon)) : hyk::round_scaled(g == 1 ? re : im, expon); }
+      else { q[r] = hyk::round_scaled(re, expon); }
+    }
+    uint32_t carry[Q_ROWS] = { 0, 0, 0, 0 };
+    #pragma unroll 1
+    for (int l = 0; l < order; ++l) {
+      uint32_t packed = 0;
+      #pragma unroll
+      for (int r = 0; r < Q_ROWS; ++r) { uint32_t t = hyk::i96_byte(q[r], l) + carry[r]; packed |= (t & 0xffu) << (8 * r); carry[r] = (t >> 8) + ((t >> 7) & 1u); }
+      store_panel(out + (int64_t)(g * order + l) * strideB, packed, valid, aligned);
     }
   }
 }
@@ -270,8 +309,11 @@ __global__ __launch_bounds__(Q_THREADS) void quantize_kernel(int32_t M, int32_t 
  * run along j, whole rows of the stored matrix; the quantized bytes leave along k, 128 per panel and column), then every
  * thread quantizes groups of Q_ROWS rows exactly as in the column-major kernel.  Replaces the transposing copy of the
  * reference (src/lra.cpp:63-69, src/matcopy.cu:36-43) together with the kernel that followed it. */
-constexpr int T_ROWS = 128;
-template <typename T> struct TileCols { static constexpr int value = sizeof(T) >= 8 ? 32 : 64; };
+/* tile shape by element size: the stored rows of a tile are TJ elements long (at least 128 bytes), a column of it leaves as
+ * T_ROWS panel bytes per panel; 256 rows (one wavefront per column, 256-byte runs as in the column-major kernel) where 33 KB
+ * of LDS hold them */
+template <typename T> struct TileCols { static constexpr int value = sizeof(T) >= 4 ? 32 : 64; };
+template <typename T> struct TileRows { static constexpr int value = sizeof(T) == 4 ? 256 : 128; };
 template <typename E> __device__ __forceinline__ typename E::T conj_elem(typename E::T v) {
   if constexpr (!E::cplx) { return v; }
   else if constexpr (sizeof(typename E::T) == 16) { v.y ^= 0x8000000000000000ull; return v; }
@@ -280,14 +322,15 @@ template <typename E> __device__ __forceinline__ typename E::T conj_elem(typenam
 }
 template <typename E, typename ROWS, bool CONJ>
 __global__ __launch_bounds__(Q_THREADS) void quantize_transposed_kernel(int32_t M, int32_t N, int32_t order, const typename E::T* __restrict__ S, int64_t lda, const int32_t* __restrict__ vexp, int8_t* __restrict__ B, int64_t ldb, int64_t strideB) {
-  using T = typename E::T; constexpr int TJ = TileCols<T>::value, PITCH = T_ROWS + 1;
+  using T = typename E::T; constexpr int TJ = TileCols<T>::value, T_ROWS = TileRows<T>::value, PITCH = T_ROWS + 1;
   extern __shared__ __attribute__((aligned(16))) unsigned char tileBytes[];
   T* tile = reinterpret_cast<T*>(tileBytes);
-  const int64_t k0 = (int64_t)blockIdx.x * T_ROWS; const int32_t j0 = blockIdx.y * TJ;
-  /* whole tiles of an aligned matrix come in as 16-byte pieces along the stored rows, all loads of a thread issued before
-   * the first LDS write; ragged or unaligned tiles element by element */
+  const int32_t j0 = blockIdx.y * TJ;
+  /* Whole tiles of an aligned matrix come in as 16-byte pieces along the stored rows, all requested before the first is
+   * used; ragged or unaligned tiles element by element. */
   constexpr int VE = sizeof(T) >= 16 ? 1 : 16 / (int)sizeof(T), PIECES = TJ / VE, ITER = PIECES * T_ROWS / Q_THREADS;
   static_assert(PIECES * T_ROWS % Q_THREADS == 0, "the pieces of a tile divide evenly among the threads");
+  const int64_t k0 = (int64_t)blockIdx.x * T_ROWS;
   if ((((uintptr_t)S) & 15u) == 0 && ((lda * (int64_t)sizeof(T)) & 15) == 0 && j0 + TJ <= N) {
     u32x4 piece[ITER];
     #pragma unroll
@@ -314,7 +357,7 @@ __global__ __launch_bounds__(Q_THREADS) void quantize_transposed_kernel(int32_t 
     }
   }
   __syncthreads();
-  constexpr int GROUPS = T_ROWS / Q_ROWS;   /* 32 row groups per column: a wavefront covers two columns */
+  constexpr int GROUPS = T_ROWS / Q_ROWS;   /* row groups per column */
   for (int e = threadIdx.x; e < TJ * GROUPS; e += Q_THREADS) {
     const int kg = e % GROUPS, jj = e / GROUPS; const int32_t j = j0 + jj; const int64_t i0 = k0 + (int64_t)kg * Q_ROWS;
     if (j >= N || i0 >= M) { continue; }
@@ -341,7 +384,7 @@ int launch_quantize(hipStream_t stream, char op, int32_t M, int32_t N, int32_t o
     dim3 grid((uint32_t)((M + Q_THREADS * Q_ROWS - 1) / (Q_THREADS * Q_ROWS)), (uint32_t)N);
     quantize_kernel<E, ROWS><<<grid, Q_THREADS, 0, stream>>>(M, order, (const T*)A, lda, vexp, B, ldb, strideB);
   } else {
-    constexpr int TJ = TileCols<T>::value; const size_t lds = (size_t)TJ * (T_ROWS + 1) * sizeof(T);
+    constexpr int TJ = TileCols<T>::value, T_ROWS = TileRows<T>::value; const size_t lds = (size_t)TJ * (T_ROWS + 1) * sizeof(T);
     dim3 grid((uint32_t)((M + T_ROWS - 1) / T_ROWS), (uint32_t)((N + TJ - 1) / TJ));
     if (op == 'C' && E::cplx) {
       if (lds > 65536 && hipFuncSetAttribute(reinterpret_cast<const void*>(&quantize_transposed_kernel<E, ROWS, true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) { return -3; }
