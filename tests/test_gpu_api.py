@@ -304,3 +304,59 @@ def test_gevd_leaves_out_floor_columns(case, capfd, monkeypatch):
     # the basis captures the matrix up to the values that are not handed out
     resid2 = (R ** 2).sum() - ((R @ X.T) ** 2).sum()
     assert abs(resid2 - (want[rank:] ** 2).sum()) <= (10 * eps) ** 2 * (want ** 2).sum() + 1e-6 * (want[rank:] ** 2).sum()
+
+
+def test_two_handles_on_two_threads():
+    """Two handles, each on a stream and a host thread of its own, fit different matrices at the same time: every result
+    equals, bit for bit, what the same handle gives when it runs alone.  (The reference keeps all state on the handle,
+    include/hyacin.h:20-53; a handle itself is used by one thread at a time.)"""
+    import threading
+    import torch
+    import hyacinth_amd as ha
+    from gpu_util import zeros, ptr
+    from oracle import ho
+    L = ha.lib()
+    rng = np.random.default_rng(77)
+    jobs = []
+    for (M, N, K, cplx, eps) in ((2048, 192, 96, False, 1e-10), (1536, 128, 128, True, 1e-8)):
+        A, _ = low_rank(rng, M, N, 0.9, cplx, noise=1e-13)
+        A = to_storage(A, 1 if cplx else 0)
+        at = ho.atype_of(A)
+        dA, lda = dev_matrix(A, "N")
+        eb = 16 if cplx else 8
+        st = torch.cuda.Stream()
+        jobs.append(dict(M=M, N=N, K=K, eps=eps, at=at, dA=dA, lda=lda, S=zeros(8 * K), V=zeros(eb * N * K), stream=st,
+                         h=ha.create_handle(stream=st.cuda_stream)))
+    torch.cuda.synchronize()
+
+    def fit(j):
+        j["S"].zero_(); j["V"].zero_(); torch.cuda.synchronize()
+        rank = L.hyacinTsvdFit(C.byref(j["h"]), j["eps"], b"N", j["M"], j["N"], j["K"], ptr(j["dA"]), j["lda"], ptr(j["S"]), ptr(j["V"]), j["N"], 0, j["at"])
+        j["stream"].synchronize()
+        return rank, L.hykLastStatus(), j["S"].cpu().numpy().copy(), j["V"].cpu().numpy().copy()
+
+    try:
+        alone = [fit(j) for j in jobs]
+        assert all(r[0] > 0 and r[1] == 0 for r in alone)
+        together = [[], []]
+        start = threading.Barrier(2)
+
+        def worker(i):
+            start.wait()
+            for _ in range(4):
+                together[i].append(fit(jobs[i]))
+
+        threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        for i in range(2):
+            assert len(together[i]) == 4
+            for rank, status, S, V in together[i]:
+                assert status == 0 and rank == alone[i][0]
+                assert np.array_equal(S, alone[i][2]) and np.array_equal(V, alone[i][3])
+    finally:
+        torch.cuda.synchronize()
+        for j in jobs:
+            ha.destroy_handle(j["h"])
