@@ -365,7 +365,7 @@ def main():
     t_kernel = kms.value / 1e3 / a.steps            # contraction kernel time per step
     achieved = ops / t_kernel / 1e12 if t_kernel > 0 else 0.0
 
-    ceiling, board = None, None
+    ceiling, board, quiet = None, None, None
     if not a.no_ceiling:
         # what a register-only MFMA loop sustains on this device with random operands (power-limited clock)
         tops, ghz = C.c_double(), C.c_double()
@@ -381,6 +381,32 @@ def main():
                 torch.cuda.synchronize()
         board = tel.summary()
         board["what"] = "hwmon power and pp_dpm_sclk sampled every 5 ms while the Gram stage (exponents, quantization, contraction, reconstruction) runs back to back for 1 s"
+        if a.workload == "target":
+            # the same launch on operands that draw almost no power (one non-zero row per row slice, all other residues zero):
+            # what the kernel's instruction stream reaches when the board's power cap does not set the clock
+            Aq = torch.zeros_like(A)
+            Aq[:, ::seg] = 1.0
+            pq = C.c_void_p(Aq.data_ptr())
+            def quiet_step():
+                L.hykQuantizeScaleBatchOp(C.byref(h), op, batches, seg, lastM, N, at, pq, lda, u, pV)
+                L.hykHerkBatchOp(C.byref(h), op, batches, seg, lastM, N, at, pq, lda, u, pV, 0, lP, pC)
+            quiet_step()
+            torch.cuda.synchronize()
+            L.hykGramProfile(1)
+            for _ in range(3):
+                quiet_step()
+            torch.cuda.synchronize()
+            qms, qn = C.c_double(), C.c_int32()
+            L.hykGramProfileRead(C.byref(qms), C.byref(qn))
+            L.hykGramProfile(0)
+            qplan = ha.HerkPlan()
+            assert L.hykLastHerkPlan(C.byref(qplan)) == 0 and qplan.int8Ops == ops and qn.value == 3 * launches_per_step, "the quiet operands must take the same plan"
+            quiet = {"achieved": ops / (qms.value / 1e3 / 3) / 1e12, "unit": "TFLOP/s", "avg_launch_ms": qms.value / qn.value,
+                     "what": "the same contraction launches on a matrix with one non-zero row per row slice: same instruction stream, operands that barely toggle, clock not held down by the power cap"}
+            quiet["frac"] = quiet["achieved"] / INT8_PEAK_TOPS
+            del Aq
+            step()   # vexp and C back to the workload's own
+            torch.cuda.synchronize()
 
     # HBM-bound stages on their own (HIP events on the launch stream, outside the timed region): algorithmic bytes / time
     def timed_ms(fn, reps=3):
@@ -475,6 +501,8 @@ def main():
     if board:
         roofline.update({k: board[k] for k in ("power_w", "power_w_max", "power_cap_w", "sclk_mhz_sysfs")})
         roofline["power_note"] = board["what"]
+    if quiet:
+        roofline["on_quiet_operands"] = quiet
     out = {
         "metric": "Gram-build effective TFLOPS (+ % INT8 MFMA peak; hyacinTsvdFit wall ms)",
         "value": feff / dt / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
