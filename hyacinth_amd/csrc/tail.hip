@@ -440,7 +440,12 @@ template <int BC> __device__ __forceinline__ void carried_pair(int t, int& i, in
 /* PASSES = 2: factors with twice the rows that fit the registers.  The rows are taken in two halves: the sums of the first
  * half, then of the second (which stays in registers), the steps, and the replay on the second half and then on the first,
  * loaded again: three loads and two stores of half the rows instead of one each of all, for blocks twice as wide. */
-template <int ROWS, int BC, bool FULL, int THREADS, bool CARRY, int PASSES>
+/* SPLIT: two workgroups per block pair, partners on one XCD.  Both load all rows, form the same sums in the same order and
+ * therefore work out the same rotations, bit for bit; each replays them on one half of the rows only (the first or the last
+ * two of a thread's four) and stores that half: no word passes between the two, the second read of the pair's rows comes
+ * out of the L2 the partner filled, and the replay of the first wavefront and the stores, which end a round, are half as
+ * long.  For the launches that leave half of the compute units idle otherwise. */
+template <int ROWS, int BC, bool FULL, int THREADS, bool CARRY, int PASSES, bool SPLIT = false>
 __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, int32_t nb, int32_t r, int32_t head, int32_t top, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations, double* __restrict__ carry) {
   constexpr int NC = 2 * BC, NG = NC * (NC + 1) / 2, WAVES = THREADS / 64, STEPS = FULL ? NC - 1 : BC, GS = NC + 1;
   constexpr bool SLIM = CARRY && !FULL;                    /* norms and cross products only */
@@ -465,7 +470,11 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
   /* Workgroups go to the 8 XCDs in turn.  Pair i of a round takes its blocks over from the pairs i - 1 and i + 1 of the round
    * before: with the pairs numbered so that neighbours run on the same XCD, most of what a workgroup loads was written
    * through the L2 it sits behind. */
-  const int pairs = gridDim.x, xcd = blockIdx.x % 8, i = xcd * (pairs / 8) + (xcd < pairs % 8 ? xcd : pairs % 8) + (int)(blockIdx.x / 8); int P, Q;   /* XCD x takes a contiguous range of pairs */
+  static_assert(!SPLIT || (!FULL && PASSES == 1 && ROWS == 4), "the split round halves the four rows of a thread");
+  const int pairs = nb / 2, xcd = blockIdx.x % 8, slot = (int)(blockIdx.x / 8), half = SPLIT ? (slot & 1) : 0;   /* XCD x takes a contiguous range of pairs */
+  if (SPLIT && (slot >> 1) >= pairs / 8 + (xcd < pairs % 8 ? 1 : 0)) { return; }   /* the grid is rounded up to whole XCD rows */
+  const int i = xcd * (pairs / 8) + (xcd < pairs % 8 ? xcd : pairs % 8) + (SPLIT ? (slot >> 1) : slot); int P, Q;
+  constexpr int RROWS = SPLIT ? ROWS / 2 : ROWS;   /* rows of a thread that this workgroup rotates and stores: registers x[c][0 .. RROWS) once the sums are done */
   if (i == 0) { P = nb - 1; Q = round; } else { P = (round + i) % (nb - 1); Q = (round - i + (nb - 1)) % (nb - 1); }
   if (P > Q) { const int t = P; P = Q; Q = t; }
   int col[NC]; bool live[NC];
@@ -509,8 +518,8 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
       #pragma unroll
       for (int c = 0; c < NC; ++c) {
         #pragma unroll
-        for (int m = 0; m < ROWS; m += 2) {
-          const int k = row_of(pass, m);
+        for (int m = 0; m < RROWS; m += 2) {
+          const int k = row_of(pass, m + half * RROWS);
           if (live[c] && k < N) { *reinterpret_cast<double2*>(&B[(int64_t)col[c] * N + k]) = double2{ x[c][m], x[c][m + 1] }; }
         }
       }
@@ -518,7 +527,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
       #pragma unroll
       for (int c = 0; c < NC; ++c) {
         #pragma unroll
-        for (int m = 0; m < ROWS; ++m) { const int k = row_of(pass, m); if (live[c] && k < N) { B[(int64_t)col[c] * N + k] = x[c][m]; } }
+        for (int m = 0; m < RROWS; ++m) { const int k = row_of(pass, m + half * RROWS); if (live[c] && k < N) { B[(int64_t)col[c] * N + k] = x[c][m]; } }
       }
     }
   };
@@ -557,6 +566,17 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
   }
   }   /* passes */
   HYK_JSTAMP(2);
+  if constexpr (SPLIT) {   /* the rows of this workgroup's half into the first registers; the others are done with */
+    #pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      #pragma unroll
+      for (int m = 0; m < RROWS; ++m) {
+        double lo = x[c][m], hi = x[c][m + RROWS];
+        asm volatile("" : "+v"(lo), "+v"(hi));   /* two values, not one element picked by a run-time index (which would put the rows into scratch memory) */
+        x[c][m] = half ? hi : lo;
+      }
+    }
+  }
   if (threadIdx.x == 0) { stepsReady = 0; }
   __syncthreads();
   HYK_JSTAMP(3);
@@ -665,10 +685,10 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
     }
     #pragma unroll
     for (int off = 32; off > 0; off >>= 1) { worst = fmax(worst, __shfl_xor(worst, off, 64)); applied += __shfl_xor(applied, off, 64); }
-    if (lane == 0) { report_cosine(rotations, worst); appliedAll = applied; if (applied > 0) { atomicAdd(rotations, applied); } }
+    if (lane == 0) { appliedAll = applied; if (half == 0) { report_cosine(rotations, worst); if (applied > 0) { atomicAdd(rotations, applied); } } }
     wave_lds_sync();
     if constexpr (CARRY) {   /* the products inside the two blocks as the steps have left them */
-      if (lane < 2 * NW) { int ci, cj; carried_pair<BC>(lane % NW, ci, cj); const int base = lane < NW ? 0 : BC; carry[(int64_t)(lane < NW ? P : Q) * NW + lane % NW] = Gs[(base + ci) * GS + base + cj]; }
+      if (lane < 2 * NW && half == 0) { int ci, cj; carried_pair<BC>(lane % NW, ci, cj); const int base = lane < NW ? 0 : BC; carry[(int64_t)(lane < NW ? P : Q) * NW + lane % NW] = Gs[(base + ci) * GS + base + cj]; }
     }
     if (lane == 0) { __hip_atomic_store(&stepsReady, STEPS + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP); }
   }
@@ -689,7 +709,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
     #pragma unroll
     for (int c = 0; c < NC; ++c) {
       #pragma unroll
-      for (int m = 0; m < ROWS; ++m) { asm volatile("" : "+v"(x[c][m]) : : "memory"); }
+      for (int m = 0; m < RROWS; ++m) { asm volatile("" : "+v"(x[c][m]) : : "memory"); }
     }
     FastRot recs[BC];   /* the records of a step come in together: one LDS latency per step, not one per rotation */
     #pragma unroll
@@ -700,7 +720,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
       const int fa = (j == 0) ? NC - 1 : (step + j) % (NC - 1), fb = (j == 0) ? step : (step - j + (NC - 1)) % (NC - 1);
       const int c0 = FULL ? (fa < fb ? fa : fb) : j, c1 = FULL ? (fa < fb ? fb : fa) : BC + (j + step) % BC;
       #pragma unroll
-      for (int m = 0; m < ROWS; ++m) { x[c0][m] = fma(-fr.t1, x[c1][m], x[c0][m]); x[c1][m] = fma(fr.t2, x[c0][m], x[c1][m]); }   /* t1 = t2 = 0: no rotation */
+      for (int m = 0; m < RROWS; ++m) { x[c0][m] = fma(-fr.t1, x[c1][m], x[c0][m]); x[c1][m] = fma(fr.t2, x[c0][m], x[c1][m]); }   /* t1 = t2 = 0: no rotation */
     }
   }
   if (pass == PASSES - 1) { wait_steps(STEPS + 1); }
@@ -709,7 +729,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
   for (int c = 0; c < NC; ++c) {
     const double sc = scale[c];
     #pragma unroll
-    for (int m = 0; m < ROWS; ++m) { x[c][m] *= sc; }
+    for (int m = 0; m < RROWS; ++m) { x[c][m] *= sc; }
   }
   HYK_JSTAMP(5);
   store_rows(pass);
@@ -1042,9 +1062,24 @@ extern "C" int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t
 /* one sweep = every pair of the r columns of B (N x r, FP64, complex interleaved) once; rotations counts the rotations applied */
 static thread_local int g_jacobiVariant = 0;   /* 0: Gram-space rounds, 8-column blocks for real factors where they fit (default); 1: the step kernel everywhere; 2: Gram-space rounds, 4-column blocks */
 
+static int compute_units() {   /* of the device current on this thread */
+  int dev = 0, n = 0;
+  if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) { return n; }
+  return 0;
+}
+
 template <int ROWS, int BC, int THREADS = T_THREADS, int PASSES = 1>
 static int gram_sweep(hipStream_t stream, int32_t N, int32_t r, int32_t head, int32_t top, double* B, double tol, int32_t* rotations, double* carry) {
   const int blocks = (r + BC - 1) / BC, nb = (blocks + 1) & ~1;
+  if constexpr (ROWS == 4 && PASSES == 1 && THREADS == 512) {
+    /* two workgroups per pair (one per compute unit: 512 threads with their rows in registers) while all of them still run side by side */
+    const int splitGrid = 16 * ((nb / 2 + 7) / 8);
+    if (carry && splitGrid <= compute_units()) {
+      jacobi_gram_round_kernel<ROWS, BC, true, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, tol, rotations, carry);
+      for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, true, PASSES, true><<<splitGrid, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, tol, rotations, carry); }
+      return hipGetLastError() == hipSuccess ? 0 : -3;
+    }
+  }
   if (carry) {
     jacobi_gram_round_kernel<ROWS, BC, true, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, tol, rotations, carry);
     for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, tol, rotations, carry); }
