@@ -1071,7 +1071,7 @@ static int compute_units() {   /* of the device current on this thread */
 template <int ROWS, int BC, int THREADS = T_THREADS, int PASSES = 1>
 static int gram_sweep(hipStream_t stream, int32_t N, int32_t r, int32_t head, int32_t top, double* B, double tol, int32_t* rotations, double* carry) {
   const int blocks = (r + BC - 1) / BC, nb = (blocks + 1) & ~1;
-  if constexpr (ROWS == 4 && PASSES == 1 && THREADS == 512) {
+  if constexpr (ROWS == 4 && PASSES == 1 && BC == 8) {
     /* two workgroups per pair (one per compute unit: 512 threads with their rows in registers) while all of them still run side by side */
     const int splitGrid = 16 * ((nb / 2 + 7) / 8);
     if (carry && splitGrid <= compute_units()) {
@@ -1126,6 +1126,8 @@ extern "C" int hykJacobiSweepTop(hipStream_t stream, int32_t Complex, int32_t N,
   /* real factors: Gram-space rounds; blocks of 8 columns where the rows of 16 columns fit the registers of 512 threads
    * (half as many rounds, each 1.4 times as long at N = 2048; up to 4096 rows in two halves), blocks of 4 otherwise */
   if (!Complex && r >= 32 && g_jacobiVariant == 0) {
+    /* up to 1024 rows: four rows per thread on 256 threads, so that a round can go to two workgroups per pair (gram_sweep), while they all run side by side */
+    if (N <= 4 * 256 && carry && 16 * ((((r + 7) / 8 + 1) / 2 + 7) / 8) <= compute_units()) { return gram_sweep<4, 8, 256>(stream, N, r, head, top, B, tol, rotations, carry); }
     if (N <= 2 * 512) { return gram_sweep<2, 8, 512>(stream, N, r, head, top, B, tol, rotations, carry); }
     if (N <= 4 * 512) { return gram_sweep<4, 8, 512>(stream, N, r, head, top, B, tol, rotations, carry); }
     if (N <= 8 * 512) { return gram_sweep<4, 8, 512, 2>(stream, N, r, head, top, B, tol, rotations, carry); }
