@@ -87,6 +87,36 @@ def test_quantize_panels_bit_exact(gl, oracle, kind):
     assert np.array_equal(got[:, :, 7:57], want) and not got[:, :, :7].any() and not got[:, :, 57:].any()
 
 
+@pytest.mark.parametrize("cplx", [False, True])
+def test_limb_digits_at_the_integer_width_limits(gl, oracle, cplx):
+    """The limb encoder takes the digits of small values from 32- and 64-bit integers (below 2^29 and 2^50) and of the rest
+    from the 96-bit path: integers on both sides of the two limits, of both signs, alone in their group of four rows and
+    mixed with small ones, must give the oracle's digits (reference: src/quantize_limbs.cu:14-58)."""
+    edge = [2 ** 29 - 1, 2 ** 29, 2 ** 29 + 1, 2 ** 50 - 1, 2 ** 50, 2 ** 50 + 1, 2 ** 52 + 1, 3, 0, 1]
+    vals = []
+    for e in edge:
+        vals += [e, 0, 0, 0, -e, 1, -1, 2, 5, e, -7, 100, -e, -e, e, e]          # groups of four rows
+    vals += [2 ** 28, 2 ** 28, 2 ** 28, 2 ** 28, -(2 ** 49), 2 ** 49, 2 ** 49, -(2 ** 49)]
+    col = np.array(vals, dtype=np.float64)
+    M = len(col)
+    A = np.zeros((M, 3), dtype=np.complex128 if cplx else np.float64)
+    A[:, 0] = col
+    A[:, 1] = col[::-1]
+    A[:, 2] = np.roll(col, 5)
+    if cplx:
+        A[:, 0] += 1j * np.roll(col, 3)          # re + im reaches 2^53: the sum's own carry into the next width
+        A[:, 1] -= 1j * col
+    A[0, :] = 2.0 ** 60                          # the column maximum: with u = 61 the exponent is 0 and q = x
+    vexp = oracle.quantize_scale_batch(A, 1, M, M, 61)
+    assert not vexp[:3].any()
+    for order in (4, 8, 11):
+        want = oracle.quantize("limbs", A, order, vexp, ldb=M + 4)
+        got = gl.quantize("limbs", A, order, vexp, ldb=M + 4)
+        assert np.array_equal(got, want), order
+        got_t = gl.quantize_op("limbs", A, "C" if cplx else "T", order, vexp, ldb=M + 4)
+        assert np.array_equal(got_t, want), order
+
+
 @pytest.mark.parametrize("op", ["T", "C"])
 @pytest.mark.parametrize("kind", ALL_KINDS)
 def test_transposed_storage_bit_exact(gl, oracle, kind, op):
