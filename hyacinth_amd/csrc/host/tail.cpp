@@ -8,7 +8,8 @@
  *  - an FP32 Gram is widened to FP64 before the Cholesky (the reference factors it in FP32);
  *  - the SVD always runs in FP64, also for FP32 / FP16 storage (the reference uses FP32 there);
  *  - the Jacobi iteration stops as soon as a sweep applies no rotation, or leaves only cosines that the quadratic
- *    contraction measured over the last two sweeps puts within 8 thresholds; a sweep here is one plain round-robin pass over all
+ *    contraction measured over the last two sweeps puts within 8 thresholds, or once the values that are handed out have
+ *    stopped moving and their columns are orthogonal to sqrt(eps); a sweep here is one plain round-robin pass over all
  *    column pairs, which does less work than a sweep of the vendor's blocked solver, so the cap is 5 x |JacobiSVDSweeps|
  *    plain sweeps (15 by default); JacobiSVDSweeps == 0 (the reference's "bidiagonalization backend") caps at 30.
  * G is working storage, as in the reference (which overwrites it with the factor): the Cholesky keeps the trailing matrix
@@ -90,6 +91,27 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
       HYH_KERNEL(hykColumnNorms(s, Complex, N, cols, B.as<double>(), sigma.as<double>()));
       HYH_CHECK(hipMemcpyAsync(v.data(), sigma.p, sizeof(double) * (size_t)cols, hipMemcpyDeviceToHost, s));
     };
+    /* How far the columns that can be handed out (the K largest norms) are from orthogonal: the largest cosine among them,
+     * from their Gram matrix.  The sweeps may end on the values alone (jacobi_output_settled), which settle with the square
+     * of what the vectors still lack: singular values 2 % apart leave their vectors several per cent away from orthogonal
+     * when the values have long stopped moving.  What is handed out as singular vectors is held to sqrt(eps): the
+     * projector V V^H is then right to eps. */
+    auto handed_out_defect = [&](const std::vector<double>& norm, int32_t ncols) -> double {
+      std::vector<int32_t> order((size_t)ncols), mark((size_t)ncols, 0); std::iota(order.begin(), order.end(), 0);
+      const int32_t kept = std::min(K, ncols);
+      std::nth_element(order.begin(), order.begin() + (kept - 1), order.end(), [&](int32_t a, int32_t b) { return norm[(size_t)a] > norm[(size_t)b]; });
+      for (int32_t i = 0; i < kept; ++i) { mark[(size_t)order[(size_t)i]] = 1; }
+      hyh::Scratch gram(handle, (size_t)ncols * ncols * 8 * (1 + Complex)), dMark(handle, sizeof(int32_t) * (size_t)ncols), dOut(handle, 64);
+      if (!hyh::ok()) { return 0.; }
+      double cos2 = 0.;
+      HYH_CHECK(hipMemcpyAsync(dMark.p, mark.data(), sizeof(int32_t) * (size_t)ncols, hipMemcpyHostToDevice, s));
+      HYH_KERNEL(hykGramWorkspaceClear(s, dOut.p, 64));
+      HYH_KERNEL(hykGemm(s, 'C', 'N', ncols, ncols, N, 1., HYACIN_F64 + Complex, B.p, N, B.p, N, 0., gram.p, ncols));
+      HYH_KERNEL(hykMaxCosine(s, Complex, ncols, gram.as<double>(), ncols, dMark.as<int32_t>(), dOut.as<double>()));
+      HYH_CHECK(hipMemcpyAsync(&cos2, dOut.p, sizeof(double), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
+      return std::sqrt(cos2);
+    };
+    const double orthogonalTo = std::sqrt(eps);
     /* Only the K largest values and their vectors are handed out.  Leaving the last rows of the Cholesky factor (the last
      * columns of B) out of the SVD takes a positive semidefinite matrix of trace tau (the sum of their squared norms) off
      * G: every eigenvalue moves down by at most tau, a singular value by at most tau / (2 sigma'), sigma' being the value
@@ -121,7 +143,11 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
         if (watchOutput) {
           double moved[3] = { 0., 0., 0. }; const bool settled = hyh::jacobi_output_settled(before, after, K, eps, moved);
           if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: the %d values handed out moved by at most %.2le, their columns gained %.2le of %.2le outside%s\n", used, K, moved[0], moved[1], moved[2], settled ? ": settled" : ""); }
-          if (settled) { break; }
+          if (settled) {
+            const double defect = handed_out_defect(after, cols); if (!hyh::ok()) { return 0; }
+            if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: largest cosine among the columns that can be handed out %.2le (wanted: %.2le)\n", used, defect, orthogonalTo); }
+            if (defect <= orthogonalTo) { break; }
+          }
         }
         lastCosine2 = seen.cosine2; before.swap(after);
       }

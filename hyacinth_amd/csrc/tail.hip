@@ -1166,6 +1166,36 @@ extern "C" int hykColumnNorms(hipStream_t stream, int32_t Complex, int32_t N, in
   return 0;
 }
 
+/* the largest squared cosine among the marked columns, from their Gram matrix: G column-major n x n (complex interleaved),
+ * mark[p] != 0 for the columns that count; out: one double, zero before the call, raised by an integer maximum on its bits */
+template <bool CPLX>
+__global__ __launch_bounds__(T_THREADS) void max_cosine_kernel(int32_t n, const double* __restrict__ G, int64_t ldg, const int32_t* __restrict__ mark, double* __restrict__ out) {
+  __shared__ double scratch[T_THREADS / 64]; constexpr int W = CPLX ? 2 : 1;
+  const int q = blockIdx.x; double worst = 0.;
+  if (mark[q]) {
+    const double gqq = G[((int64_t)q + (int64_t)q * ldg) * W];
+    for (int p = threadIdx.x; p < q; p += T_THREADS) {
+      if (!mark[p]) { continue; }
+      const double* g = &G[((int64_t)p + (int64_t)q * ldg) * W]; double g2 = g[0] * g[0]; if constexpr (CPLX) { g2 = fma(g[1], g[1], g2); }
+      worst = fmax(worst, squared_cosine(g2, G[((int64_t)p + (int64_t)p * ldg) * W], gqq));
+    }
+  }
+  for (int off = 32; off > 0; off >>= 1) { worst = fmax(worst, __shfl_xor(worst, off, 64)); }
+  if ((threadIdx.x & 63) == 0) { scratch[threadIdx.x >> 6] = worst; }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < T_THREADS / 64; ++w) { worst = fmax(worst, scratch[w]); }
+    if (worst > 0.) { atomicMax(reinterpret_cast<unsigned long long*>(out), (unsigned long long)__double_as_longlong(worst)); }
+  }
+}
+
+extern "C" int hykMaxCosine(hipStream_t stream, int32_t Complex, int32_t n, const double* G, int64_t ldg, const int32_t* mark, double* out) {
+  if (n <= 1) { return 0; }
+  if (ldg < n) { return -1; }
+  if (Complex) { max_cosine_kernel<true><<<n, T_THREADS, 0, stream>>>(n, G, ldg, mark, out); } else { max_cosine_kernel<false><<<n, T_THREADS, 0, stream>>>(n, G, ldg, mark, out); }
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
 extern "C" int hykBasisOut(hipStream_t stream, int32_t N, int32_t rank, int32_t Atype, const double* B, const double* sigma, const int32_t* order, void* X, int64_t ldx) {
   if (N <= 0 || rank <= 0) { return 0; }
   dim3 grid((N + T_THREADS - 1) / T_THREADS, rank);

@@ -127,6 +127,12 @@ int hykJacobiSweepTop(hipStream_t stream, int32_t Complex, int32_t N, int32_t r,
  * pairs in the same order; kept selectable so that tests cover every kernel.  The setting is per host thread. */
 int hykJacobiSetVariant(int32_t variant);
 int hykColumnNorms(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, const double* B, double* sigma);
+
+/* How far a set of columns is from orthogonal, from their Gram matrix (no counterpart in the reference, which takes what
+ * gesvdj returns after its sweep budget, src/gram_evd.cu:9-42): G is n x n column-major FP64 (complex interleaved when
+ * Complex), mark[p] != 0 selects the columns that count; *out (device, zero before the call) receives the largest
+ * |G[p, q]|^2 / (G[p, p] G[q, q]) over the marked pairs p < q. */
+int hykMaxCosine(hipStream_t stream, int32_t Complex, int32_t n, const double* G, int64_t ldg, const int32_t* mark, double* out);
 int hykBasisOut(hipStream_t stream, int32_t N, int32_t rank, int32_t Atype, const double* B, const double* sigma, const int32_t* order, void* X, int64_t ldx);
 int hykValuesOut(hipStream_t stream, int32_t K, int32_t Atype, const double* S, void* out);
 

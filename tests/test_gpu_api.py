@@ -306,6 +306,23 @@ def test_gevd_leaves_out_floor_columns(case, capfd, monkeypatch):
     assert abs(resid2 - (want[rank:] ** 2).sum()) <= (10 * eps) ** 2 * (want ** 2).sum() + 1e-6 * (want[rank:] ** 2).sum()
 
 
+@pytest.mark.parametrize("at", [0, 3])
+def test_fit_hands_out_orthogonal_vectors(env, at):
+    """Singular values 2 % apart: the values stop moving several sweeps before their vectors are orthogonal.  What
+    hyacinTsvdFit hands out as singular vectors is orthonormal to sqrt(eps) all the same (the reference takes what three
+    sweeps of gesvdj leave, src/gram_evd.cu:148-150), or to the rounding of the storage type where that is coarser."""
+    rng = np.random.default_rng(90 + at)
+    M, N, K, eps = 1500, 256, 128, 1e-5
+    cplx = bool(at & 1)
+    U, W = haar(rng, M, N, cplx), haar(rng, N, N, cplx)
+    A = to_storage((U * 2.0 ** (-np.arange(N) / 32.0)) @ W.conj().T, at)
+    rank, S, V, err, nrm = run_tsvd(env, A, eps, K, "N")
+    assert rank == K
+    defect = np.abs(V.conj().T @ V - np.eye(rank)).max()
+    print("orthogonality", at, defect, flush=True)
+    assert defect <= max(np.sqrt(eps), 1e-5 if at >= 2 else 0.0)
+
+
 def test_two_handles_on_two_threads():
     """Two handles, each on a stream and a host thread of its own, fit different matrices at the same time: every result
     equals, bit for bit, what the same handle gives when it runs alone.  (The reference keeps all state on the handle,

@@ -189,3 +189,34 @@ def test_orthonormalize(L, cplx, N, r):
     Qr, _ = np.linalg.qr(V)
     assert np.abs(Q - Qr @ (Qr.conj().T @ Q)).max() <= 1e-12       # nothing of Q lies outside span(V)
     assert L.hykOrthonormalize(stream(), cplx, N, r, ptr(dV), N + 1, ptr(work)) == -1
+
+
+@pytest.mark.parametrize("cplx", [0, 1])
+@pytest.mark.parametrize("n,pad", [(2, 0), (37, 3), (300, 0)])
+def test_max_cosine(L, cplx, n, pad):
+    """hykMaxCosine: the largest |G[p, q]|^2 / (G[p, p] G[q, q]) over the marked pairs of a Gram matrix, against numpy;
+    unmarked columns do not count, a zero diagonal entry under a non-zero product counts as 1."""
+    from gpu_util import dev, zeros, ptr, stream, sync, host
+    rng = np.random.default_rng(70 + n)
+    X = rng.standard_normal((2 * n, n)) + (1j * rng.standard_normal((2 * n, n)) if cplx else 0)
+    X[:, 0] *= 1e-9
+    G = X.conj().T @ X
+    ld = n + pad
+    buf = np.full((n, ld, 2) if cplx else (n, ld), np.nan)          # [column][row]: column-major with padding rows
+    if cplx:
+        buf[:, :n, 0] = G.real.T
+        buf[:, :n, 1] = G.imag.T
+    else:
+        buf[:, :n] = G.T
+    mark = (rng.random(n) < 0.7).astype(np.int32)
+    mark[:2] = 1
+    dG, dM, out = dev(buf), dev(mark), zeros(8)
+    assert L.hykMaxCosine(stream(), cplx, n, ptr(dG), ld, ptr(dM), ptr(out)) == 0
+    sync()
+    d = np.real(np.diag(G))
+    c2 = np.abs(G) ** 2 / np.outer(d, d)
+    keep = np.outer(mark, mark).astype(bool) & ~np.eye(n, dtype=bool)
+    want = c2[keep].max()
+    got = host(out, np.float64)[0]
+    assert abs(got - want) <= 1e-12 * want
+    assert L.hykMaxCosine(stream(), cplx, n, ptr(dG), n - 1, ptr(dM), ptr(out)) == -1
