@@ -190,7 +190,9 @@ extern "C" int32_t hyacinXGinterp(const hyacinHandle_t* handle, double eps, int3
   hipStream_t s = handle->hipStream; hyh::timer_mark(handle, hyh::Segment::rep_kernel);
   const int Complex = (int)Atype & 1; eps = std::min(std::max(std::fabs(eps), storage_eps((int)Atype)), 1.);
   Factor f(handle, N, K, (int)Gtype, G, ldg);
-  const int32_t rank = run_potrfp(handle, f, eps, K, N, jpiv);
+  /* The factorization counts a single remaining column in (src/hyacin_potrfp.cu:271), so K = N - 1 can come back as N; the
+   * reference then writes N columns into an X that the caller sized for K (src/gram_id.cpp:41).  Never more than K here. */
+  const int32_t rank = std::min(K, run_potrfp(handle, f, eps, K, N, jpiv));
   if (rank <= 0 || !hyh::ok()) { return 0; }
   if (rank >= N) { HYH_KERNEL(hykInterpOut(s, N, N, (int32_t)Atype, jpiv, nullptr, X, ldx)); return hyh::ok() ? N : 0; }
   hyh::Scratch Rp(handle, (size_t)rank * rank * 8 * (1 + Complex)), Tt(handle, (size_t)rank * (N - rank) * 8 * (1 + Complex));

@@ -192,6 +192,28 @@ def test_interpolate_fit(env, oracle, at, opA):
     assert resid <= 2 * resid_o + 50 * max(eps, storage_eps) * np.linalg.norm(Ac)
 
 
+def test_interpolate_fit_never_writes_past_k_columns(env):
+    """K = N - 1 on a matrix of full rank: the reference's factorization counts the single remaining column in
+    (src/hyacin_potrfp.cu:271) and its interpolation then writes N columns into an X sized for K (src/gram_id.cpp:41).
+    Here the rank comes back as K and the memory behind the K columns of X stays as it was."""
+    from gpu_util import dev, zeros, ptr, sync, host
+    ha, h = env
+    rng = np.random.default_rng(45)
+    M, N, K = 700, 12, 11
+    A = rng.standard_normal((M, N))
+    dA, lda = dev_matrix(A, "N")
+    X = dev(np.full(N * (K + 2), 7.5))                 # two guard columns behind the K the caller asked for
+    jp = zeros(4 * N)
+    rank = ha.lib().hyacinInterpolateFit(C.byref(h), 1e-10, b"N", M, N, K, ptr(dA), lda, ptr(jp), ptr(X), N, 0, 0)
+    sync()
+    assert rank == K and ha.lib().hykLastStatus() == 0
+    Xh = host(X, np.float64).reshape(K + 2, N).T
+    assert np.all(Xh[:, K:] == 7.5)
+    sel = host(jp, np.int32)[:K] - 1
+    assert np.allclose(Xh[sel, :K], np.eye(K), atol=1e-12)
+    assert np.linalg.norm(A - A[:, sel] @ Xh[:, :K].T) <= 1e-9 * np.linalg.norm(A) + np.linalg.svd(A, compute_uv=False)[-1] * 50
+
+
 def test_segmented_fit(env, oracle):
     ha, h = env
     rng = np.random.default_rng(44)
