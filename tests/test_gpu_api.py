@@ -345,6 +345,36 @@ def test_fit_hands_out_orthogonal_vectors(env, at):
     assert defect <= max(np.sqrt(eps), 1e-5 if at >= 2 else 0.0)
 
 
+@pytest.mark.parametrize("at,eps", [(0, 1e-12), (1, 1e-9), (2, 1e-5)])
+def test_fit_with_global_rows(env, at, eps):
+    """globalM above M (the rows of other devices, include/hyacin.h:67-113): the integer Gram gets the head-room of
+    nextpow2(globalM) (src/hyacin_herk.cpp:52,57: one 63-bit limb more in the first case) and carries the same value, so the fit
+    returns what it returns for globalM = M."""
+    from gpu_util import zeros, ptr, sync, host
+    ha, h = env
+    rng = np.random.default_rng(95 + at)
+    M, N, K = 1800, 120, 60
+    A0, _ = low_rank(rng, M, N, 0.8, cplx=bool(at & 1), noise=eps * 1e-2)
+    A = to_storage(A0, at)
+    dA, lda = dev_matrix(A, "N")
+    eb = {0: 8, 1: 16, 2: 4}[at]
+    sb = eb // (1 + (at & 1))
+    out = []
+    for globalM in (0, 1 << 40):
+        u, cP, lP, stride = ha.herk_batch_init(h, eps, globalM or M, N, at)
+        S, V = zeros(sb * K), zeros(eb * N * K)
+        rank = ha.lib().hyacinTsvdFit(C.byref(h), eps, b"N", M, N, K, ptr(dA), lda, ptr(S), ptr(V), N, globalM, at)
+        sync()
+        assert ha.lib().hykLastStatus() == 0
+        real = {8: np.float64, 4: np.float32}[sb]
+        out.append((rank, lP, host(S, real).astype(np.float64).copy(), host(V, real).astype(np.float64).copy()))
+    (r0, l0, S0, V0), (r1, l1, S1, V1) = out
+    assert l1 >= l0 + (at == 0) and r1 == r0 and r0 > 0           # the FP64 case crosses into a third limb
+    tol = 4 * {0: 2.2e-16, 1: 2.2e-16, 2: 1.2e-7}[at]
+    assert np.abs(S1 - S0).max() <= tol * S0[0]
+    assert np.abs(V1 - V0).max() <= max(1e-9, 100 * tol)
+
+
 def test_two_handles_on_two_threads():
     """Two handles, each on a stream and a host thread of its own, fit different matrices at the same time: every result
     equals, bit for bit, what the same handle gives when it runs alone.  (The reference keeps all state on the handle,
