@@ -375,6 +375,31 @@ def test_fit_with_global_rows(env, at, eps):
     assert np.abs(V1 - V0).max() <= max(1e-9, 100 * tol)
 
 
+def test_tail_options_of_the_handle(env):
+    """QRCPTruncateRank and JacobiSVDSweeps (include/hyacin.h:44, src/gram_evd.cu:148-150): without the rank cut in the
+    Cholesky (QRCPTruncateRank = 0, where the sweep count is |min(0, JacobiSVDSweeps)|, 0 standing for the backend without a
+    budget) and with other sweep budgets the fit returns the values of the default settings; a budget of one (five plain
+    sweeps here) still returns a basis whose projection residual is within a factor of the converged one."""
+    ha, h = env
+    rng = np.random.default_rng(97)
+    M, N, K, eps = 1500, 96, 40, 1e-9
+    A0, _ = low_rank(rng, M, N, 0.7, noise=1e-12)
+    A = to_storage(A0, 0)
+    base = run_tsvd(env, A, eps, K, "N")
+    try:
+        for trunc, sweeps, converged in ((0, 3, True), (0, -4, True), (1, -6, True), (1, 6, True), (1, 1, False)):
+            h.QRCPTruncateRank, h.JacobiSVDSweeps = trunc, sweeps
+            rank, S, V, err, nrm = run_tsvd(env, A, eps, K, "N")
+            assert ha.lib().hykLastStatus() == 0
+            print("tail options", trunc, sweeps, rank, err / nrm, flush=True)
+            assert abs(rank - base[0]) <= (1 if converged else 3)
+            k = min(rank, base[0])
+            assert np.abs(S[:k] - base[1][:k]).max() <= (10 * eps if converged else 1e-3) * base[1][0]
+            assert err <= (4 if converged else 100) * base[3] + (20 * eps) ** 2 * nrm
+    finally:
+        h.QRCPTruncateRank, h.JacobiSVDSweeps = 1, 3
+
+
 def test_two_handles_on_two_threads():
     """Two handles, each on a stream and a host thread of its own, fit different matrices at the same time: every result
     equals, bit for bit, what the same handle gives when it runs alone.  (The reference keeps all state on the handle,
