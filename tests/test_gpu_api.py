@@ -400,6 +400,30 @@ def test_tail_options_of_the_handle(env):
         h.QRCPTruncateRank, h.JacobiSVDSweeps = 1, 3
 
 
+def test_handle_settings_from_the_environment(monkeypatch):
+    """hyacinCreate reads its settings from the environment variables the reference reads (src/utils.cpp:64-72), with the
+    reference's defaults when they are not set."""
+    import hyacinth_amd as ha
+    from gpu_util import stream
+    fields = ("GramMatrixAlgorithm", "StrideBatchPerfPenalty", "GramSegmentK", "TCGemmTargetK", "QuantizeBitCorrection", "QRCPTruncateRank", "JacobiSVDSweeps")
+    names = ("HYACIN_GRAM_ALGORITHM", "HYACIN_STRIDE_BATCH_PERF_PENALTY", "HYACIN_GRAM_SEGMENT_K", "HYACIN_TCGEMM_TARGET_K", "HYACIN_QUANTIZE_BITS_CORR",
+             "HYACIN_QRCP_TRUNCATE_RANK", "HYACIN_JACOBI_SVD_SWEEPS")
+    for n in names:
+        monkeypatch.delenv(n, raising=False)
+    h = ha.create_handle(stream=stream().value)
+    try:
+        assert tuple(getattr(h, f) for f in fields) == (b"A", 1.3, 8192, 8192, 7, 1, 3)
+    finally:
+        ha.destroy_handle(h)
+    for n, v in zip(names, ("L", "2.5", "4096", "1024", "12", "0", "-5")):
+        monkeypatch.setenv(n, v)
+    h = ha.create_handle(stream=stream().value)
+    try:
+        assert tuple(getattr(h, f) for f in fields) == (b"L", 2.5, 4096, 1024, 12, 0, -5)
+    finally:
+        ha.destroy_handle(h)
+
+
 def test_two_handles_on_two_threads():
     """Two handles, each on a stream and a host thread of its own, fit different matrices at the same time: every result
     equals, bit for bit, what the same handle gives when it runs alone.  (The reference keeps all state on the handle,
