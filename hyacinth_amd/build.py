@@ -1,9 +1,7 @@
 """Build libhyacin.so (HIP kernels + C++ drivers) for gfx950 with hipcc.
 
-Usage: python -m hyacinth_amd.build [--jobs N] [--timing]
+Usage: python -m hyacinth_amd.build [--jobs N]
 The library lands next to this file (in-tree), which is where the loader looks.
---timing additionally builds libhyacin_timing.so: the same library with the pivoted Cholesky and the Jacobi round kernels
-compiled with their phase stamps (-DHYK_POTRFP_TIMING -DHYK_JACOBI_TIMING); hyacinth_amd/phase_timing.py reads them.
 """
 import argparse
 import concurrent.futures
@@ -35,10 +33,6 @@ def hipcc():
     raise RuntimeError("hipcc not found")
 
 
-TIMING_LIB = os.path.join(HERE, "libhyacin_timing.so")
-TIMING_SOURCES = {"potrfp.hip": "-DHYK_POTRFP_TIMING", "tail.hip": "-DHYK_JACOBI_TIMING"}
-
-
 def compile_one(src, define=None):
     out = os.path.join(OBJ, ("timing_" if define else "") + src.replace("/", "_") + ".o")
     cmd = [hipcc(), "-x", "hip", "-c", os.path.join(CSRC, src), "-o", out] + COMMON + ([define] if define else [])
@@ -68,27 +62,10 @@ def build(jobs=8, verbose=False):
     return LIB
 
 
-def build_timing(jobs=8):
-    """The measurement build: needs the objects of build() and replaces those of the stamped kernels."""
-    build(jobs)
-    stamped = []
-    for src, define in TIMING_SOURCES.items():
-        out, log = compile_one(src, define)
-        if out is None:
-            raise RuntimeError(log)
-        stamped.append(out)
-    plain = [os.path.join(OBJ, src.replace("/", "_") + ".o") for src in KERNELS + HOST if src not in TIMING_SOURCES]
-    r = subprocess.run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", TIMING_LIB] + plain + stamped, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError("link failed:\n" + r.stdout + r.stderr)
-    return TIMING_LIB
-
-
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--jobs", type=int, default=8)
     ap.add_argument("-v", "--verbose", action="store_true")
-    ap.add_argument("--timing", action="store_true", help="also build libhyacin_timing.so (kernels with phase stamps)")
     a = ap.parse_args()
-    print(build_timing(a.jobs) if a.timing else build(a.jobs, a.verbose))
+    print(build(a.jobs, a.verbose))
     sys.exit(0)

@@ -76,7 +76,7 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
     rank = run_potrfp(handle, f, lrqr ? eps : 0., N, N, jpiv.as<int32_t>());
     if (rank <= 0 || !hyh::ok()) { return 0; }
     /* B = (R P^T)^H, N x rank, FP64 */
-    hyh::Scratch B(handle, (size_t)N * rank * 8 * (1 + Complex)), sigma(handle, sizeof(double) * (size_t)rank), counter(handle, 64), carry(handle, hykJacobiCarryBytes(rank));
+    hyh::Scratch B(handle, (size_t)N * rank * 8 * (1 + Complex)), sigma(handle, sizeof(double) * (size_t)rank), counter(handle, 64), carry(handle, hykJacobiCarryBytes(N, rank));
     if (!hyh::ok()) { return 0; }
     HYH_KERNEL(hykFactorToB(s, N, rank, f.type, f.Rt.p, f.ldr, B.as<double>()));
     const int32_t maxSweeps = sweeps > 0 ? 5 * sweeps : 30; int32_t used = 0;

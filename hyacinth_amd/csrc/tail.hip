@@ -444,9 +444,15 @@ template <int BC> __device__ __forceinline__ void carried_pair(int t, int& i, in
  * therefore work out the same rotations, bit for bit; each replays them on one half of the rows only (the first or the last
  * two of a thread's four) and stores that half: no word passes between the two, the second read of the pair's rows comes
  * out of the L2 the partner filled, and the replay of the first wavefront and the stores, which end a round, are half as
- * long.  For the launches that leave half of the compute units idle otherwise. */
+ * long.  For the launches that leave half of the compute units idle otherwise.
+ * A split round is OUT OF PLACE: every workgroup reads the columns from B and writes its half of the rows to Bout, another
+ * buffer, so that no load of the launch can meet a store of the same launch, whenever the two partners are dispatched
+ * (in place, a partner that starts after the other has stored would read half-rotated columns and form other rotations).
+ * Every block is in exactly one pair of a round, and a split round writes every pair it is given: the pairs that it does
+ * not rotate (wholly in the tail that is left alone, or nothing above the threshold) are copied, so Bout holds all live
+ * columns after the launch and the host swaps the two buffers from round to round. */
 template <int ROWS, int BC, bool FULL, int THREADS, bool CARRY, int PASSES, bool SPLIT = false>
-__global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, int32_t nb, int32_t r, int32_t head, int32_t top, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations, double* __restrict__ carry) {
+__global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, int32_t nb, int32_t r, int32_t head, int32_t top, int32_t round, double* __restrict__ B, double* __restrict__ Bout, double tol, int32_t* __restrict__ rotations, double* __restrict__ carry, double* __restrict__ carryOut) {
   constexpr int NC = 2 * BC, NG = NC * (NC + 1) / 2, WAVES = THREADS / 64, STEPS = FULL ? NC - 1 : BC, GS = NC + 1;
   constexpr bool SLIM = CARRY && !FULL;                    /* norms and cross products only */
   constexpr int NW = BC * (BC - 1) / 2, NP = SLIM ? NC + BC * BC : NG;
@@ -483,7 +489,22 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
   if (!live[0]) { return; }
   /* Columns from `top` on are the tail that is left alone: pairs of two tail columns are not rotated.  A block pair wholly
    * in the tail has nothing to do, except in the first round of a sweep, which also refreshes the carried products. */
-  if (!FULL && col[0] >= top) { return; }
+  double* const __restrict__ dst = SPLIT ? Bout : B;   /* where the rotated rows go */
+  double* const __restrict__ carryDst = SPLIT ? carryOut : carry;   /* and the products inside the blocks: a split round reads `carry` in both partners, so it is not written either */
+  if (!FULL && col[0] >= top) {
+    if constexpr (SPLIT) {   /* not rotated, but the next round reads Bout and carryOut: this workgroup's half of the rows is copied, and by the first partner the carried products */
+      if (CARRY && half == 0 && threadIdx.x < 2 * NW) { const int64_t at = (int64_t)(threadIdx.x < NW ? P : Q) * NW + threadIdx.x % NW; carryDst[at] = carry[at]; }
+      #pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        #pragma unroll
+        for (int m = 0; m < ROWS / 2; ++m) {
+          const int mm = m + half * (ROWS / 2), k = 2 * (int)threadIdx.x + (mm & 1) + (mm >> 1) * 2 * THREADS;   /* row_of(0, mm) below */
+          if (live[c] && k < N) { dst[(int64_t)col[c] * N + k] = B[(int64_t)col[c] * N + k]; }
+        }
+      }
+    }
+    return;
+  }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   HYK_JDECL(); HYK_JSTAMP(0);
   [[maybe_unused]] double carried = 0.;
@@ -492,7 +513,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
   double x[NC][ROWS];
   /* a thread owns pairs of adjacent rows: 16-byte loads and stores where the columns are 16-byte aligned (N even) */
   static_assert(ROWS % 2 == 0, "rows are owned in adjacent pairs");
-  const bool vec2 = (N & 1) == 0 && (reinterpret_cast<uintptr_t>(B) & 15u) == 0;
+  const bool vec2 = (N & 1) == 0 && ((reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(dst)) & 15u) == 0;
   auto row_of = [&](int pass, int m) { return 2 * (int)threadIdx.x + (m & 1) + (m >> 1) * 2 * THREADS + pass * ROWS * THREADS; };
   auto load_rows = [&](int pass) {
     if (vec2) {
@@ -521,14 +542,14 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
         for (int m = 0; m < RROWS; m += 2) {
           const int k = row_of(pass, m + half * RROWS);
           /* past the caches: the next round's readers find the rows in memory either way, and the end of the launch has less to write back (a sweep at N = r = 2048: 4.70 -> 4.60 ms; the complex kernel loses with the same stores) */
-          if (live[c] && k < N) { typedef double d2 __attribute__((ext_vector_type(2))); __builtin_nontemporal_store(d2{ x[c][m], x[c][m + 1] }, reinterpret_cast<d2*>(&B[(int64_t)col[c] * N + k])); }
+          if (live[c] && k < N) { typedef double d2 __attribute__((ext_vector_type(2))); __builtin_nontemporal_store(d2{ x[c][m], x[c][m + 1] }, reinterpret_cast<d2*>(&dst[(int64_t)col[c] * N + k])); }
         }
       }
     } else {
       #pragma unroll
       for (int c = 0; c < NC; ++c) {
         #pragma unroll
-        for (int m = 0; m < RROWS; ++m) { const int k = row_of(pass, m + half * RROWS); if (live[c] && k < N) { B[(int64_t)col[c] * N + k] = x[c][m]; } }
+        for (int m = 0; m < RROWS; ++m) { const int k = row_of(pass, m + half * RROWS); if (live[c] && k < N) { dst[(int64_t)col[c] * N + k] = x[c][m]; } }
       }
     }
   };
@@ -689,7 +710,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
     if (lane == 0) { appliedAll = applied; if (half == 0) { report_cosine(rotations, worst); if (applied > 0) { atomicAdd(rotations, applied); } } }
     wave_lds_sync();
     if constexpr (CARRY) {   /* the products inside the two blocks as the steps have left them */
-      if (lane < 2 * NW && half == 0) { int ci, cj; carried_pair<BC>(lane % NW, ci, cj); const int base = lane < NW ? 0 : BC; carry[(int64_t)(lane < NW ? P : Q) * NW + lane % NW] = Gs[(base + ci) * GS + base + cj]; }
+      if (lane < 2 * NW && half == 0) { int ci, cj; carried_pair<BC>(lane % NW, ci, cj); const int base = lane < NW ? 0 : BC; carryDst[(int64_t)(lane < NW ? P : Q) * NW + lane % NW] = Gs[(base + ci) * GS + base + cj]; }
     }
     if (lane == 0) { __hip_atomic_store(&stepsReady, STEPS + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP); }
   }
@@ -725,7 +746,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
     }
   }
   if (pass == PASSES - 1) { wait_steps(STEPS + 1); }
-  if (appliedAll == 0) { return; }   /* uniform over the workgroup: nothing was rotated, the columns stay as they are */
+  if (!SPLIT && appliedAll == 0) { return; }   /* uniform over the workgroup: nothing was rotated, the columns stay as they are (a split round writes them to the other buffer all the same: scales of one) */
   #pragma unroll
   for (int c = 0; c < NC; ++c) {
     const double sc = scale[c];
@@ -1069,24 +1090,36 @@ static int compute_units() {   /* of the device current on this thread */
   return 0;
 }
 
+/* bytes of the products that travel with the blocks from round to round (enough for every round kernel: 28 doubles per block of 8 real columns) */
+static size_t carried_bytes(int32_t r) { return ((size_t)r / 4 + 2) * 28 * sizeof(double); }
+/* factors of up to this many rows can take split rounds, which write to a second copy of the factor */
+constexpr int32_t SPLIT_MAX_ROWS = 4 * 512;
+
 template <int ROWS, int BC, int THREADS = T_THREADS, int PASSES = 1>
 static int gram_sweep(hipStream_t stream, int32_t N, int32_t r, int32_t head, int32_t top, double* B, double tol, int32_t* rotations, double* carry) {
   const int blocks = (r + BC - 1) / BC, nb = (blocks + 1) & ~1;
   if constexpr (ROWS == 4 && PASSES == 1 && BC == 8) {
-    /* two workgroups per pair (one per compute unit: 512 threads with their rows in registers) while all of them still run side by side */
+    /* two workgroups per pair (one per compute unit: 512 threads with their rows in registers) while all of them still run
+     * side by side.  The split rounds go from B to the second copy behind the carried products and back: rounds 1 ..
+     * nb - 2 are an even number of them, so the sweep ends in B. */
     const int splitGrid = 16 * ((nb / 2 + 7) / 8);
     if (carry && splitGrid <= compute_units()) {
-      jacobi_gram_round_kernel<ROWS, BC, true, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, tol, rotations, carry);
-      for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, true, PASSES, true><<<splitGrid, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, tol, rotations, carry); }
-      return hipGetLastError() == hipSuccess ? 0 : -3;
+      double* carry2 = reinterpret_cast<double*>(reinterpret_cast<char*>(carry) + carried_bytes(r)); double* B2 = reinterpret_cast<double*>(reinterpret_cast<char*>(carry) + 2 * carried_bytes(r));
+      double* from = B; double* to = B2; double* cfrom = carry; double* cto = carry2;
+      jacobi_gram_round_kernel<ROWS, BC, true, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, nullptr, tol, rotations, carry, nullptr);
+      for (int round = 1; round < nb - 1; ++round) {
+        jacobi_gram_round_kernel<ROWS, BC, false, THREADS, true, PASSES, true><<<splitGrid, THREADS, 0, stream>>>(N, nb, r, head, top, round, from, to, tol, rotations, cfrom, cto);
+        double* t = from; from = to; to = t; t = cfrom; cfrom = cto; cto = t;
+      }
+      return (from == B && hipGetLastError() == hipSuccess) ? 0 : -3;
     }
   }
   if (carry) {
-    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, tol, rotations, carry);
-    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, tol, rotations, carry); }
+    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, nullptr, tol, rotations, carry, nullptr);
+    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, nullptr, tol, rotations, carry, nullptr); }
   } else {
-    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, false, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, tol, rotations, nullptr);
-    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, false, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, tol, rotations, nullptr); }
+    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, false, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, nullptr, tol, rotations, nullptr, nullptr);
+    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, false, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, nullptr, tol, rotations, nullptr, nullptr); }
   }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
@@ -1114,7 +1147,7 @@ static int blocked_sweep(hipStream_t stream, int32_t N, int32_t r, int32_t head,
 
 extern "C" int hykJacobiSetVariant(int32_t variant) { if (variant < 0 || variant > 2) { return -1; } g_jacobiVariant = variant; return 0; }
 
-extern "C" size_t hykJacobiCarryBytes(int32_t r) { return r <= 0 ? 0 : ((size_t)r / 4 + 2) * 28 * sizeof(double); }
+extern "C" size_t hykJacobiCarryBytes(int32_t N, int32_t r) { return (r <= 0 || N <= 0) ? 0 : 2 * carried_bytes(r) + (N <= SPLIT_MAX_ROWS ? (size_t)N * (size_t)r * sizeof(double) : 0); }
 
 extern "C" int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations) { return hykJacobiSweepTop(stream, Complex, N, r, r, r, B, tol, rotations, nullptr); }
 

@@ -111,9 +111,13 @@ int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t Gtype, con
  * tol is rotated.  rotations: 16 bytes of device memory, zero before the call; afterwards rotations[0] = pairs rotated and
  * the double at rotations + 2 = the largest squared cosine the sweep met (rotated or not). */
 int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations);
-/* The same sweep with hykJacobiCarryBytes(r) bytes of device memory that its rounds use to hand the products inside a
- * column block from one round to the next instead of summing them again (ignored by the kernels of variant 1).  The memory needs no initialisation and holds nothing a later sweep relies on. */
-size_t hykJacobiCarryBytes(int32_t r);
+/* The same sweep with hykJacobiCarryBytes(N, r) bytes of device memory (16-byte aligned) for its rounds: the products
+ * inside a column block travel through it from one round to the next instead of being summed again (ignored by the
+ * kernels of variant 1), and for real factors of up to 2048 rows it holds a second copy of the factor: the rounds that put
+ * two workgroups on a block pair read one copy and write the other, so that neither partner can read what the other has
+ * already rotated, whenever the device dispatches them.  The memory needs no initialisation and holds nothing a later
+ * sweep relies on; B holds the result after every sweep. */
+size_t hykJacobiCarryBytes(int32_t N, int32_t r);
 int hykJacobiSweepCarry(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations, double* carry);
 /* The same sweep with two index limits.  Pairs of two columns with index >= top are not rotated (block pairs wholly behind
  * `top` are skipped); the largest cosine is reported over the pairs with at least one column before `head` only (the pairs

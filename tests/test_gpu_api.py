@@ -478,3 +478,59 @@ def test_two_handles_on_two_threads():
         torch.cuda.synchronize()
         for j in jobs:
             ha.destroy_handle(j["h"])
+
+
+def test_two_gevd_tails_at_the_same_time():
+    """hyacinXGevd (src/gram_evd.cu:94-142) on two handles, streams and host threads at once, at sizes whose Jacobi rounds put
+    two workgroups on every block pair and fill the device (N = r = 2048 and N = r = 1024, real): while the other handle's
+    kernels hold compute units, the two partners of a pair start at different times.  The rounds read one copy of the factor
+    and write another, so the values and vectors are, bit for bit, those of each handle running alone."""
+    import threading
+    import torch
+    import hyacinth_amd as ha
+    from gpu_util import dev, zeros, ptr
+    L = ha.lib()
+    rng = np.random.default_rng(78)
+    jobs = []
+    for N in (2048, 1024):
+        W = haar(rng, N, N, False)
+        R = (2.0 ** (-np.arange(N) / (N / 24.0)))[:, None] * W.T                 # a dense factor, singular values over seven digits
+        G = R.T @ R
+        st = torch.cuda.Stream()
+        jobs.append(dict(N=N, G0=dev(np.ascontiguousarray(G.T)), G=zeros(8 * N * N), S=zeros(8 * N), X=zeros(8 * N * N), stream=st, h=ha.create_handle(stream=st.cuda_stream)))
+    torch.cuda.synchronize()
+
+    def tail(j):
+        with torch.cuda.stream(j["stream"]):                                        # the call overwrites G; no device-wide wait, the other handle keeps running
+            j["G"].copy_(j["G0"]); j["S"].zero_(); j["X"].zero_()
+        rank = L.hyacinXGevd(C.byref(j["h"]), 1e-9, j["N"], j["N"], 0, ptr(j["X"]), j["N"], ptr(j["S"]), 0, ptr(j["G"]), j["N"])
+        j["stream"].synchronize()
+        return rank, L.hykLastStatus(), j["S"].cpu().numpy().copy(), j["X"].cpu().numpy().copy()
+
+    try:
+        alone = [tail(j) for j in jobs]
+        assert all(r[0] > j["N"] // 2 and r[1] == 0 for r, j in zip(alone, jobs))
+        for (rank, _, S, X), j in zip(alone, jobs):                                  # and the vectors are an orthonormal set
+            V = X.view(np.float64).reshape(j["N"], j["N"])[:rank]
+            assert np.abs(V @ V.T - np.eye(rank)).max() <= 1e-9
+        together = [[], []]
+        start = threading.Barrier(2)
+
+        def worker(i):
+            start.wait()
+            for _ in range(3 if i == 0 else 8):
+                together[i].append(tail(jobs[i]))
+
+        threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        for i in range(2):
+            for rank, status, S, X in together[i]:
+                assert status == 0 and rank == alone[i][0]
+                assert np.array_equal(S, alone[i][2]) and np.array_equal(X, alone[i][3])
+    finally:
+        torch.cuda.synchronize()
+        for j in jobs:
+            ha.destroy_handle(j["h"])
