@@ -98,7 +98,7 @@ def lib():
         L.hykJacobiSweep.argtypes = [vp, i32, i32, i32, vp, dbl, vp]
         L.hykJacobiSweepCarry.argtypes = [vp, i32, i32, i32, vp, dbl, vp, vp]
         L.hykJacobiSweepTop.argtypes = [vp, i32, i32, i32, i32, i32, vp, dbl, vp, vp]
-        L.hykJacobiCarryBytes.argtypes = [i32, i32]; L.hykJacobiCarryBytes.restype = C.c_size_t
+        L.hykJacobiCarryBytes.argtypes = [i32]; L.hykJacobiCarryBytes.restype = C.c_size_t
         L.hykGramProfile.argtypes = [i32]
         L.hykGramProfileRead.argtypes = [C.POINTER(dbl), C.POINTER(i32)]
         L.hykMfmaCeiling.argtypes = [vp, i32, i32, i32, C.POINTER(dbl), C.POINTER(dbl)]

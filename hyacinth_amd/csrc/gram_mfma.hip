@@ -647,23 +647,33 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_ring_kernel(const GramArgs 
    * a wrap is harmless), so one unsigned reduction gives the canonical residue.  Blocks of a diagonal tile wholly below
    * the diagonal are skipped, those wholly above need no test.  CHECKED: the tile touches the matrix edge or the diagonal.
    * SIMPLE: the group adds its sums unchanged to its real plane only (every real launch, the paired complex residues). */
-  if constexpr (EPI == EPI_I64) {   /* 64-bit sums: the shared epilogue (its values and addresses leave no room for more) */
-    HYK_GRAM_EPILOGUE(EXCL)
-    return;
-  }
   const bool inner = (ta != tb) && (x0 + TILE <= args.N) && (y0 + TILE <= args.N);
   const bool simple = grp.mulRe == 1u && grp.mulIm == 0u;
   uint32_t bias = 0u;
   if constexpr (EPI == EPI_MOD) { const uint32_t over = 0x80000000u % grp.m; bias = 0x80000000u + (over ? grp.m - over : 0u); }
+  /* 64-bit sums: the two planes of the group and the signs, as wave-uniform values in scalar registers */
+  [[maybe_unused]] unsigned long long* wideRe = nullptr; [[maybe_unused]] unsigned long long* wideIm = nullptr;
+  [[maybe_unused]] bool hasRe = false, hasIm = false; [[maybe_unused]] int32_t maskRe = 0, maskIm = 0;
+  if constexpr (EPI == EPI_I64) {
+    auto uniform64 = [](uint64_t v) { return ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32)) << 32) | (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v); };
+    wideRe = reinterpret_cast<unsigned long long*>(uniform64((uint64_t)(reinterpret_cast<unsigned long long*>(args.acc) + (int64_t)grp.planeRe * args.planeStride)));
+    wideIm = reinterpret_cast<unsigned long long*>(uniform64((uint64_t)(reinterpret_cast<unsigned long long*>(args.acc) + (int64_t)grp.planeIm * args.planeStride)));
+    hasRe = __builtin_amdgcn_readfirstlane((int)grp.mulRe) != 0; hasIm = __builtin_amdgcn_readfirstlane((int)grp.mulIm) != 0;
+    maskRe = __builtin_amdgcn_readfirstlane(grp.mulRe == 2u ? -1 : 0); maskIm = __builtin_amdgcn_readfirstlane(grp.mulIm == 2u ? -1 : 0);
+  }
+  /* what the epilogue needs of the arguments, as locals: its sixteen blocks in four versions name them hundreds of times,
+   * and past some number of uses the optimiser stops reading a by-value argument structure in place and copies it to
+   * scratch memory instead (whose loads count as divergent: the load addresses of the loop above then sit in vector registers) */
+  const int32_t nCols = args.N; const int64_t planeStride = args.planeStride; uint32_t* const accBase = reinterpret_cast<uint32_t*>(args.acc);
   auto emit = [&](auto checked_, auto simple_) {
     constexpr bool CHECKED = decltype(checked_)::value != 0, SIMPLE = decltype(simple_)::value != 0;
-    #pragma unroll
-    for (int a = 0; a < 4; ++a) {
-      #pragma unroll
-      for (int b = 0; b < 4; ++b) {
+    /* one 32x32 block; a and b are compile-time values, so the accumulators are named registers whatever the optimiser
+     * makes of the loops (a loop over blocks that it declines to unroll indexes them at run time: all 256 go to scratch) */
+    auto block = [&](auto a_, auto b_) __attribute__((always_inline)) {   /* (a call that is not inlined would take the address of the kernel arguments, which then live in scratch memory) */
+        constexpr int a = decltype(a_)::value, b = decltype(b_)::value;
         __builtin_amdgcn_sched_barrier(0);   /* one 32x32 block at a time: keeps the accumulator copies out of scratch */
         bool diagBlock = false;
-        if constexpr (CHECKED) { if (ta == tb) { const int by = 4 * wy + b, bx = 4 * wx + a; if (by > bx) { continue; } diagBlock = by == bx; } }
+        if constexpr (CHECKED) { if (ta == tb) { const int by = 4 * wy + b, bx = 4 * wx + a; if (by > bx) { return; } diagBlock = by == bx; } }
         const int y = y0 + wy * WAVE_TILE + b * 32 + (lane & 31);
         int x = x0 + wx * WAVE_TILE + a * 32 + ((lane >> 5) << 2);
         int64_t e = hyk::tri_index(y, x);
@@ -671,24 +681,35 @@ __global__ __launch_bounds__(G_THREADS, 1) void gram_ring_kernel(const GramArgs 
         for (int r = 0; r < 16; ++r) {
           if (r) { if (r & 3) { e += x + 1; x += 1; } else { e += 5 * (int64_t)x + 15; x += 5; } }
           bool ok = true;
-          if constexpr (CHECKED) { ok = x < args.N && y < args.N && (!diagBlock || y <= x); }
+          if constexpr (CHECKED) { ok = x < nCols && y < nCols && (!diagBlock || y <= x); }
           if (ok) {
             const int32_t w = acc[a][b][r];
             if constexpr (EPI == EPI_MOD) {
-              uint32_t* dst = reinterpret_cast<uint32_t*>(args.acc);
+              uint32_t* dst = accBase;
               const uint32_t v = hyk::reduce_u32((uint32_t)w + bias, grp.m, grp.d);
               if constexpr (SIMPLE) {
-                uint32_t* at = &dst[(int64_t)grp.planeRe * args.planeStride + e];
+                uint32_t* at = &dst[(int64_t)grp.planeRe * planeStride + e];
                 if constexpr (EXCL) { *at = v; } else { atomicAdd(at, v); }
               } else {
-                if (grp.mulRe) { uint32_t* at = &dst[(int64_t)grp.planeRe * args.planeStride + e]; const uint32_t t = grp.mulRe == 1u ? v : hyk::reduce_u32(v * grp.mulRe, grp.m, grp.d); if constexpr (EXCL) { *at = t; } else { atomicAdd(at, t); } }
-                if (grp.mulIm) { uint32_t* at = &dst[(int64_t)grp.planeIm * args.planeStride + e]; const uint32_t t = grp.mulIm == 1u ? v : hyk::reduce_u32(v * grp.mulIm, grp.m, grp.d); if constexpr (EXCL) { *at = t; } else { atomicAdd(at, t); } }
+                if (grp.mulRe) { uint32_t* at = &dst[(int64_t)grp.planeRe * planeStride + e]; const uint32_t t = grp.mulRe == 1u ? v : hyk::reduce_u32(v * grp.mulRe, grp.m, grp.d); if constexpr (EXCL) { *at = t; } else { atomicAdd(at, t); } }
+                if (grp.mulIm) { uint32_t* at = &dst[(int64_t)grp.planeIm * planeStride + e]; const uint32_t t = grp.mulIm == 1u ? v : hyk::reduce_u32(v * grp.mulIm, grp.m, grp.d); if constexpr (EXCL) { *at = t; } else { atomicAdd(at, t); } }
+              }
+            } else {   /* 64-bit sums of the limb levels: + W or - W to the real and / or the imaginary plane of the level */
+              if constexpr (SIMPLE) {
+                unsigned long long* at = wideRe + e; const unsigned long long pos = (unsigned long long)(long long)w;
+                if constexpr (EXCL) { *at = pos; } else { atomicAdd(at, pos); }
+              } else {   /* (w ^ mask) - mask = -w for mask = -1 (a K range that the cap allows never sums to INT_MIN) */
+                if (hasRe) { const unsigned long long t = (unsigned long long)(long long)((w ^ maskRe) - maskRe); if constexpr (EXCL) { wideRe[e] = t; } else { atomicAdd(wideRe + e, t); } }
+                if (hasIm) { const unsigned long long t = (unsigned long long)(long long)((w ^ maskIm) - maskIm); if constexpr (EXCL) { wideIm[e] = t; } else { atomicAdd(wideIm + e, t); } }
               }
             }
           }
         }
-      }
-    }
+    };
+    block(IC<0>{}, IC<0>{}); block(IC<0>{}, IC<1>{}); block(IC<0>{}, IC<2>{}); block(IC<0>{}, IC<3>{});
+    block(IC<1>{}, IC<0>{}); block(IC<1>{}, IC<1>{}); block(IC<1>{}, IC<2>{}); block(IC<1>{}, IC<3>{});
+    block(IC<2>{}, IC<0>{}); block(IC<2>{}, IC<1>{}); block(IC<2>{}, IC<2>{}); block(IC<2>{}, IC<3>{});
+    block(IC<3>{}, IC<0>{}); block(IC<3>{}, IC<1>{}); block(IC<3>{}, IC<2>{}); block(IC<3>{}, IC<3>{});
   };
   if (mode == 2) { /* every block of this wavefront lies below the diagonal */ }
   else if (inner) { if (simple) { emit(IC<0>{}, IC<1>{}); } else { emit(IC<0>{}, IC<0>{}); } }

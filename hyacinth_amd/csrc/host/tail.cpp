@@ -76,7 +76,7 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
     rank = run_potrfp(handle, f, lrqr ? eps : 0., N, N, jpiv.as<int32_t>());
     if (rank <= 0 || !hyh::ok()) { return 0; }
     /* B = (R P^T)^H, N x rank, FP64 */
-    hyh::Scratch B(handle, (size_t)N * rank * 8 * (1 + Complex)), sigma(handle, sizeof(double) * (size_t)rank), counter(handle, 64), carry(handle, hykJacobiCarryBytes(N, rank));
+    hyh::Scratch B(handle, (size_t)N * rank * 8 * (1 + Complex)), sigma(handle, sizeof(double) * (size_t)rank), counter(handle, 64), carry(handle, hykJacobiCarryBytes(rank));
     if (!hyh::ok()) { return 0; }
     HYH_KERNEL(hykFactorToB(s, N, rank, f.type, f.Rt.p, f.ldr, B.as<double>()));
     const int32_t maxSweeps = sweeps > 0 ? 5 * sweeps : 30; int32_t used = 0;
@@ -138,6 +138,7 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
         struct { int32_t rotations, pad; double cosine2; } seen = { 0, 0, 0. };
         HYH_CHECK(hipMemcpyAsync(&seen, counter.p, sizeof(seen), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
         if (!hyh::ok()) { return 0; }
+        if (seen.pad != 0) { hyh::fail(-5, "Jacobi sweep", "a workgroup gave up waiting for the partner it shares a block pair with; no basis was produced", __FILE__, __LINE__); return 0; }
         if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: %d rotations, largest cosine %.2le among pairs with a column before %d%s\n", used, seen.rotations, std::sqrt(seen.cosine2), headCols, top < cols ? " (floor of small columns left alone)" : ""); }
         if (hyh::jacobi_sweeps_done(seen.rotations, seen.cosine2, lastCosine2, rotateAbove)) { break; }
         if (watchOutput) {

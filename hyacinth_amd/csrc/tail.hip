@@ -442,19 +442,29 @@ template <int BC> __device__ __forceinline__ void carried_pair(int t, int& i, in
  * loaded again: three loads and two stores of half the rows instead of one each of all, for blocks twice as wide. */
 /* SPLIT: two workgroups per block pair, partners on one XCD.  Both load all rows, form the same sums in the same order and
  * therefore work out the same rotations, bit for bit; each replays them on one half of the rows only (the first or the last
- * two of a thread's four) and stores that half: no word passes between the two, the second read of the pair's rows comes
- * out of the L2 the partner filled, and the replay of the first wavefront and the stores, which end a round, are half as
- * long.  For the launches that leave half of the compute units idle otherwise.
- * A split round is OUT OF PLACE: every workgroup reads the columns from B and writes its half of the rows to Bout, another
- * buffer, so that no load of the launch can meet a store of the same launch, whenever the two partners are dispatched
- * (in place, a partner that starts after the other has stored would read half-rotated columns and form other rotations).
- * Every block is in exactly one pair of a round, and a split round writes every pair it is given: the pairs that it does
- * not rotate (wholly in the tail that is left alone, or nothing above the threshold) are copied, so Bout holds all live
- * columns after the launch and the host swaps the two buffers from round to round. */
+ * two of a thread's four) and stores that half: the second read of the pair's rows comes out of the L2 the partner filled,
+ * and the replay of the first wavefront and the stores, which end a round, are half as long.  For the launches that leave
+ * half of the compute units idle otherwise.
+ * The round works in place, so a partner must never load rows that the other has already rotated and stored, however far
+ * apart the device dispatches the two.  One 32-bit word per pair and round (zero before the launch) orders them:
+ *   bits 0-1  workgroups that have arrived (fetch-add on arrival);
+ *   bit 2, 3  this half's workgroup has all its loads (rows and carried products) in registers;
+ *   bit 4     one workgroup has taken the whole pair.
+ * Before it stores, a workgroup looks at the word.  The partner has loaded: it stores its half.  The partner has arrived
+ * but not finished loading: it waits (the partner is running and sets its bit without waiting for anything; the wait is
+ * bounded all the same and, given up, raises rotations[1], which the host reports as a failure).  The partner has not
+ * arrived: a compare-and-swap from exactly "one arrival, my loads done" sets bit 4, and this workgroup then rotates and
+ * stores both halves (it loads the other half's rows again and replays the round's rotations from LDS); a partner that
+ * arrives afterwards finds bit 4 in what its fetch-add returns and leaves without storing anything (whatever it has
+ * loaded meanwhile is discarded).  If the swap fails, the partner has arrived in between: wait as above.  So no load
+ * whose values are used can observe a store of the same launch.  The cosine, the rotation count and the carried
+ * products are written by the workgroup that is sure to finish: the first half's, or the one that took the pair. */
 template <int ROWS, int BC, bool FULL, int THREADS, bool CARRY, int PASSES, bool SPLIT = false>
-__global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, int32_t nb, int32_t r, int32_t head, int32_t top, int32_t round, double* __restrict__ B, double* __restrict__ Bout, double tol, int32_t* __restrict__ rotations, double* __restrict__ carry, double* __restrict__ carryOut) {
+__global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, int32_t nb, int32_t r, int32_t head, int32_t top, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations, double* __restrict__ carry, uint32_t* __restrict__ pairWords) {
   constexpr int NC = 2 * BC, NG = NC * (NC + 1) / 2, WAVES = THREADS / 64, STEPS = FULL ? NC - 1 : BC, GS = NC + 1;
   constexpr bool SLIM = CARRY && !FULL;                    /* norms and cross products only */
+  constexpr uint32_t PW_COUNT = 3u, PW_LOADED = 4u, PW_TAKEN = 16u;   /* the pair's word: arrivals, loaded bits (<< half), pair taken by one workgroup */
+  constexpr int PWAVE = WAVES - 1;                          /* the wavefront that handles the word (not the first: nothing may sit on the chain of steps) */
   constexpr int NW = BC * (BC - 1) / 2, NP = SLIM ? NC + BC * BC : NG;
   constexpr int CH = NP >= 32 ? 32 : 16, TAIL = NP % CH;
   static_assert((TAIL & (TAIL - 1)) == 0 && (TAIL == 0 || TAIL >= 4) && BC * BC <= 64 && 2 * NW <= 64, "tail chunk a power of two; one lane of the first wavefront per pair of pairs and per carried product");
@@ -473,6 +483,9 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
   __shared__ int32_t pairCol[BC][2];
   __shared__ int32_t appliedAll;
   __shared__ int32_t stepsReady;
+  __shared__ double worstAll;
+  __shared__ int32_t pairTaken;     /* split rounds: the partner has taken the whole pair, nothing to do here */
+  __shared__ int32_t storeMode;     /* split rounds: 0 undecided, 1 this half only, 2 both halves, 3 gave up */
   /* Workgroups go to the 8 XCDs in turn.  Pair i of a round takes its blocks over from the pairs i - 1 and i + 1 of the round
    * before: with the pairs numbered so that neighbours run on the same XCD, most of what a workgroup loads was written
    * through the L2 it sits behind. */
@@ -489,31 +502,19 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
   if (!live[0]) { return; }
   /* Columns from `top` on are the tail that is left alone: pairs of two tail columns are not rotated.  A block pair wholly
    * in the tail has nothing to do, except in the first round of a sweep, which also refreshes the carried products. */
-  double* const __restrict__ dst = SPLIT ? Bout : B;   /* where the rotated rows go */
-  double* const __restrict__ carryDst = SPLIT ? carryOut : carry;   /* and the products inside the blocks: a split round reads `carry` in both partners, so it is not written either */
-  if (!FULL && col[0] >= top) {
-    if constexpr (SPLIT) {   /* not rotated, but the next round reads Bout and carryOut: this workgroup's half of the rows is copied, and by the first partner the carried products */
-      if (CARRY && half == 0 && threadIdx.x < 2 * NW) { const int64_t at = (int64_t)(threadIdx.x < NW ? P : Q) * NW + threadIdx.x % NW; carryDst[at] = carry[at]; }
-      #pragma unroll
-      for (int c = 0; c < NC; ++c) {
-        #pragma unroll
-        for (int m = 0; m < ROWS / 2; ++m) {
-          const int mm = m + half * (ROWS / 2), k = 2 * (int)threadIdx.x + (mm & 1) + (mm >> 1) * 2 * THREADS;   /* row_of(0, mm) below */
-          if (live[c] && k < N) { dst[(int64_t)col[c] * N + k] = B[(int64_t)col[c] * N + k]; }
-        }
-      }
-    }
-    return;
-  }
+  if (!FULL && col[0] >= top) { return; }
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   HYK_JDECL(); HYK_JSTAMP(0);
   [[maybe_unused]] double carried = 0.;
   if constexpr (SLIM) { if (wave == 0 && lane < 2 * NW) { carried = carry[(int64_t)(lane < NW ? P : Q) * NW + lane % NW]; } }
+  [[maybe_unused]] uint32_t* const word = SPLIT ? &pairWords[(int64_t)(round - 1) * pairs + i] : nullptr;
+  [[maybe_unused]] uint32_t arrival = 0u;
+
   static_assert(PASSES == 1 || PASSES == 2, "all rows at once or in two halves");
   double x[NC][ROWS];
   /* a thread owns pairs of adjacent rows: 16-byte loads and stores where the columns are 16-byte aligned (N even) */
   static_assert(ROWS % 2 == 0, "rows are owned in adjacent pairs");
-  const bool vec2 = (N & 1) == 0 && ((reinterpret_cast<uintptr_t>(B) | reinterpret_cast<uintptr_t>(dst)) & 15u) == 0;
+  const bool vec2 = (N & 1) == 0 && (reinterpret_cast<uintptr_t>(B) & 15u) == 0;
   auto row_of = [&](int pass, int m) { return 2 * (int)threadIdx.x + (m & 1) + (m >> 1) * 2 * THREADS + pass * ROWS * THREADS; };
   auto load_rows = [&](int pass) {
     if (vec2) {
@@ -534,7 +535,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
       }
     }
   };
-  auto store_rows = [&](int pass) {
+  auto store_rows = [&](int pass, int half) {
     if (vec2) {
       #pragma unroll
       for (int c = 0; c < NC; ++c) {
@@ -542,20 +543,22 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
         for (int m = 0; m < RROWS; m += 2) {
           const int k = row_of(pass, m + half * RROWS);
           /* past the caches: the next round's readers find the rows in memory either way, and the end of the launch has less to write back (a sweep at N = r = 2048: 4.70 -> 4.60 ms; the complex kernel loses with the same stores) */
-          if (live[c] && k < N) { typedef double d2 __attribute__((ext_vector_type(2))); __builtin_nontemporal_store(d2{ x[c][m], x[c][m + 1] }, reinterpret_cast<d2*>(&dst[(int64_t)col[c] * N + k])); }
+          if (live[c] && k < N) { typedef double d2 __attribute__((ext_vector_type(2))); __builtin_nontemporal_store(d2{ x[c][m], x[c][m + 1] }, reinterpret_cast<d2*>(&B[(int64_t)col[c] * N + k])); }
         }
       }
     } else {
       #pragma unroll
       for (int c = 0; c < NC; ++c) {
         #pragma unroll
-        for (int m = 0; m < RROWS; ++m) { const int k = row_of(pass, m + half * RROWS); if (live[c] && k < N) { dst[(int64_t)col[c] * N + k] = x[c][m]; } }
+        for (int m = 0; m < RROWS; ++m) { const int k = row_of(pass, m + half * RROWS); if (live[c] && k < N) { B[(int64_t)col[c] * N + k] = x[c][m]; } }
       }
     }
   };
   #pragma unroll
   for (int pass = 0; pass < PASSES; ++pass) {
   load_rows(pass);
+  /* arrival at the pair's word, asked behind the row loads (memory answers a wavefront in order, and an atomic takes longer than a load: asked first, it would hold this wavefront's rows back); the answer is needed after the sums */
+  if constexpr (SPLIT) { if (wave == PWAVE && lane == 0) { arrival = __hip_atomic_fetch_add(word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); } }
   HYK_JWAIT(); HYK_JSTAMP(1);
   /* products numbered by diagonal: p = d NC + c stands for (c, (c + d) % NC), d = 0 .. NC / 2 (the last diagonal only for
    * c < NC / 2): every unordered pair once, and p splits back into the pair by shifts.  Summed over the wavefront 32 at a time. */
@@ -600,7 +603,19 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
     }
   }
   if (threadIdx.x == 0) { stepsReady = 0; }
+  if constexpr (SPLIT) {
+    if (wave == 0) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }   /* the carried products are in registers too (the rows are: the sums have used them) */
+    if (wave == PWAVE && lane == 0) { pairTaken = (arrival & PW_TAKEN) ? 1 : 0; storeMode = 0; }
+  }
   __syncthreads();
+  if constexpr (SPLIT) {
+    if (pairTaken) { return; }   /* uniform: the partner rotates and stores both halves; what was loaded here may be half rotated and is dropped */
+    /* Every load of this workgroup has returned: each thread has used its rows in the sums, and the barrier has passed.  Say
+     * so.  The atomic is issued after that point in program order and orders nothing else: what the partner stores once it
+     * has seen the bit cannot reach loads that have already delivered their values (a release here would also write the
+     * XCD's L2 back, which holds the last round's rows: a microsecond per round for nothing). */
+    if (wave == PWAVE && lane == 0) { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); __hip_atomic_fetch_or(word, PW_LOADED << half, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+  }
   HYK_JSTAMP(3);
   /* From here on the wavefronts meet through `stepsReady` only: the first wavefront publishes the number of steps whose
    * rotations are in `fast` (and STEPS + 1 once the scales and the rotation count are there as well), the others replay
@@ -707,10 +722,10 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
     }
     #pragma unroll
     for (int off = 32; off > 0; off >>= 1) { worst = fmax(worst, __shfl_xor(worst, off, 64)); applied += __shfl_xor(applied, off, 64); }
-    if (lane == 0) { appliedAll = applied; if (half == 0) { report_cosine(rotations, worst); if (applied > 0) { atomicAdd(rotations, applied); } } }
+    if (lane == 0) { appliedAll = applied; worstAll = worst; if constexpr (!SPLIT) { report_cosine(rotations, worst); if (applied > 0) { atomicAdd(rotations, applied); } } }
     wave_lds_sync();
-    if constexpr (CARRY) {   /* the products inside the two blocks as the steps have left them */
-      if (lane < 2 * NW && half == 0) { int ci, cj; carried_pair<BC>(lane % NW, ci, cj); const int base = lane < NW ? 0 : BC; carryDst[(int64_t)(lane < NW ? P : Q) * NW + lane % NW] = Gs[(base + ci) * GS + base + cj]; }
+    if constexpr (CARRY && !SPLIT) {   /* the products inside the two blocks as the steps have left them */
+      if (lane < 2 * NW) { int ci, cj; carried_pair<BC>(lane % NW, ci, cj); const int base = lane < NW ? 0 : BC; carry[(int64_t)(lane < NW ? P : Q) * NW + lane % NW] = Gs[(base + ci) * GS + base + cj]; }
     }
     if (lane == 0) { __hip_atomic_store(&stepsReady, STEPS + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP); }
   }
@@ -722,9 +737,17 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
   #pragma unroll
   for (int pass = PASSES - 1; pass >= 0; --pass) {
   if (pass != PASSES - 1) { load_rows(pass); }
+  [[maybe_unused]] uint32_t early = 0u;   /* split rounds: the pair's word as it was at the second step (asked for then, looked at when the stores are due) */
   #pragma unroll
   for (int step = 0; step < STEPS; ++step) {
     if (pass == PASSES - 1) { wait_steps(FULL ? STEPS + 1 : step + 1); }
+    if constexpr (SPLIT) {
+      if (wave == PWAVE && lane == 0) {
+        if (step == 1) { early = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }   /* asked for early: the answer takes longer than a step, and this wavefront must not wait for it */
+        /* the usual case: the partner had loaded long before, and the others learn it before they are through with the last step */
+        if (step == STEPS - 1 && (early & (PW_LOADED << (half ^ 1)))) { __hip_atomic_store(&storeMode, 1 | 4, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP); }
+      }
+    }
     /* Nothing of the compiler's moves across this point: not the records of later steps (fetched ahead they would wait in
      * scratch memory), and not the arithmetic of this thread's rows either (it is needed only when the rows are stored, and
      * would otherwise sink behind the waits for all later steps, which takes the overlap away). */
@@ -746,7 +769,37 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
     }
   }
   if (pass == PASSES - 1) { wait_steps(STEPS + 1); }
-  if (!SPLIT && appliedAll == 0) { return; }   /* uniform over the workgroup: nothing was rotated, the columns stay as they are (a split round writes them to the other buffer all the same: scales of one) */
+  if constexpr (SPLIT) {
+    /* Who stores what (see the comment above the kernel).  One lane settles it and says so in storeMode (bit 2: settled). */
+    if (wave == PWAVE && lane == 0 && !(early & (PW_LOADED << (half ^ 1)))) {
+      const uint32_t mine = PW_LOADED << half, theirs = PW_LOADED << (half ^ 1);
+      int decided = 0;
+      for (int spin = 0; decided == 0 && spin < (1 << 22); ++spin) {
+        const uint32_t seen = __hip_atomic_load(word, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+        if (seen & theirs) { decided = 1; }
+        else if ((seen & PW_COUNT) == 1u) {   /* alone so far */
+          uint32_t expected = 1u | mine;
+          if (seen == expected && __hip_atomic_compare_exchange_strong(word, &expected, expected | PW_TAKEN, __ATOMIC_ACQ_REL, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) { decided = 2; }
+        } else { __builtin_amdgcn_s_sleep(2); }   /* the partner is here and loading */
+      }
+      if (decided == 0) { decided = 3; atomicExch(&rotations[1], 1); }   /* never seen with a running partner: no stores rather than wrong ones */
+      __hip_atomic_store(&storeMode, decided | 4, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    while (!(__hip_atomic_load(&storeMode, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) & 4)) { __builtin_amdgcn_s_sleep(1); }
+    /* cosine, rotation count and carried products from the workgroup that is sure to finish; nothing waits for them */
+    if (wave == PWAVE) {
+      const int m = storeMode & 3;
+      if (m == 2 || (m == 1 && half == 0)) {
+        if (lane == 0) { report_cosine(rotations, worstAll); if (appliedAll > 0) { atomicAdd(rotations, appliedAll); } }
+        if constexpr (CARRY) {   /* the products inside the two blocks as the steps have left them: the partner, if there is one, has read its own already */
+          if (lane < 2 * NW) { int ci, cj; carried_pair<BC>(lane % NW, ci, cj); const int base = lane < NW ? 0 : BC; carry[(int64_t)(lane < NW ? P : Q) * NW + lane % NW] = Gs[(base + ci) * GS + base + cj]; }
+        }
+      }
+    }
+  }
+  [[maybe_unused]] const int mode = SPLIT ? (storeMode & 3) : 1;
+  if (SPLIT && mode == 3) { return; }
+  if (appliedAll == 0) { return; }   /* uniform over the workgroup: nothing was rotated, the columns stay as they are */
   #pragma unroll
   for (int c = 0; c < NC; ++c) {
     const double sc = scale[c];
@@ -754,8 +807,34 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
     for (int m = 0; m < RROWS; ++m) { x[c][m] *= sc; }
   }
   HYK_JSTAMP(5);
-  store_rows(pass);
+  store_rows(pass, half);
   HYK_JWAIT(); HYK_JSTAMP(6);
+  if constexpr (SPLIT) {
+    if (mode == 2) {   /* the partner was not there: its half as well, from memory (nobody else writes these rows in this launch) */
+      const int other = half ^ 1;
+      #pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        #pragma unroll
+        for (int m = 0; m < RROWS; ++m) { const int k = row_of(pass, m + other * RROWS); x[c][m] = (live[c] && k < N) ? B[(int64_t)col[c] * N + k] : 0.; }
+      }
+      #pragma unroll
+      for (int step = 0; step < STEPS; ++step) {
+        #pragma unroll
+        for (int j = 0; j < BC; ++j) {
+          const FastRot fr = fast[step][j]; const int c0 = j, c1 = BC + (j + step) % BC;   /* a split round is never the first of a sweep: cross pairs only */
+          #pragma unroll
+          for (int m = 0; m < RROWS; ++m) { x[c0][m] = fma(-fr.t1, x[c1][m], x[c0][m]); x[c1][m] = fma(fr.t2, x[c0][m], x[c1][m]); }
+        }
+      }
+      #pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const double sc = scale[c];
+        #pragma unroll
+        for (int m = 0; m < RROWS; ++m) { x[c][m] *= sc; }
+      }
+      store_rows(pass, other);
+    }
+  }
   }   /* passes */
   HYK_JREPORT();
 }
@@ -1092,34 +1171,29 @@ static int compute_units() {   /* of the device current on this thread */
 
 /* bytes of the products that travel with the blocks from round to round (enough for every round kernel: 28 doubles per block of 8 real columns) */
 static size_t carried_bytes(int32_t r) { return ((size_t)r / 4 + 2) * 28 * sizeof(double); }
-/* factors of up to this many rows can take split rounds, which write to a second copy of the factor */
-constexpr int32_t SPLIT_MAX_ROWS = 4 * 512;
+/* and of the words that order the two workgroups of a pair in the split rounds: one per pair and round of 8-column blocks */
+static size_t pair_word_bytes(int32_t r) { const size_t nb = (((size_t)r + 7) / 8 + 1) & ~(size_t)1; return (nb * nb / 2 * sizeof(uint32_t) + 255) / 256 * 256; }
 
 template <int ROWS, int BC, int THREADS = T_THREADS, int PASSES = 1>
 static int gram_sweep(hipStream_t stream, int32_t N, int32_t r, int32_t head, int32_t top, double* B, double tol, int32_t* rotations, double* carry) {
   const int blocks = (r + BC - 1) / BC, nb = (blocks + 1) & ~1;
   if constexpr (ROWS == 4 && PASSES == 1 && BC == 8) {
-    /* two workgroups per pair (one per compute unit: 512 threads with their rows in registers) while all of them still run
-     * side by side.  The split rounds go from B to the second copy behind the carried products and back: rounds 1 ..
-     * nb - 2 are an even number of them, so the sweep ends in B. */
+    /* two workgroups per pair (one per compute unit: 512 threads with their rows in registers) while all of them still run side by side */
     const int splitGrid = 16 * ((nb / 2 + 7) / 8);
     if (carry && splitGrid <= compute_units()) {
-      double* carry2 = reinterpret_cast<double*>(reinterpret_cast<char*>(carry) + carried_bytes(r)); double* B2 = reinterpret_cast<double*>(reinterpret_cast<char*>(carry) + 2 * carried_bytes(r));
-      double* from = B; double* to = B2; double* cfrom = carry; double* cto = carry2;
-      jacobi_gram_round_kernel<ROWS, BC, true, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, nullptr, tol, rotations, carry, nullptr);
-      for (int round = 1; round < nb - 1; ++round) {
-        jacobi_gram_round_kernel<ROWS, BC, false, THREADS, true, PASSES, true><<<splitGrid, THREADS, 0, stream>>>(N, nb, r, head, top, round, from, to, tol, rotations, cfrom, cto);
-        double* t = from; from = to; to = t; t = cfrom; cfrom = cto; cto = t;
-      }
-      return (from == B && hipGetLastError() == hipSuccess) ? 0 : -3;
+      uint32_t* words = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(carry) + carried_bytes(r));
+      if (hykGramWorkspaceClear(stream, words, pair_word_bytes(r)) != 0) { return -3; }
+      jacobi_gram_round_kernel<ROWS, BC, true, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, tol, rotations, carry, nullptr);
+      for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, true, PASSES, true><<<splitGrid, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, tol, rotations, carry, words); }
+      return hipGetLastError() == hipSuccess ? 0 : -3;
     }
   }
   if (carry) {
-    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, nullptr, tol, rotations, carry, nullptr);
-    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, nullptr, tol, rotations, carry, nullptr); }
+    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, tol, rotations, carry, nullptr);
+    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, tol, rotations, carry, nullptr); }
   } else {
-    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, false, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, nullptr, tol, rotations, nullptr, nullptr);
-    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, false, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, nullptr, tol, rotations, nullptr, nullptr); }
+    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, false, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, tol, rotations, nullptr, nullptr);
+    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, false, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, tol, rotations, nullptr, nullptr); }
   }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
@@ -1147,7 +1221,7 @@ static int blocked_sweep(hipStream_t stream, int32_t N, int32_t r, int32_t head,
 
 extern "C" int hykJacobiSetVariant(int32_t variant) { if (variant < 0 || variant > 2) { return -1; } g_jacobiVariant = variant; return 0; }
 
-extern "C" size_t hykJacobiCarryBytes(int32_t N, int32_t r) { return (r <= 0 || N <= 0) ? 0 : 2 * carried_bytes(r) + (N <= SPLIT_MAX_ROWS ? (size_t)N * (size_t)r * sizeof(double) : 0); }
+extern "C" size_t hykJacobiCarryBytes(int32_t r) { return r <= 0 ? 0 : carried_bytes(r) + pair_word_bytes(r); }
 
 extern "C" int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations) { return hykJacobiSweepTop(stream, Complex, N, r, r, r, B, tol, rotations, nullptr); }
 
@@ -1304,6 +1378,7 @@ extern "C" int hykOrthonormalize(hipStream_t stream, int32_t Complex, int32_t N,
     if (hykJacobiSweep(stream, Complex, N, r, V, 2.220446049250313e-16 * sqrt((double)N), counter) != 0) { return -3; }
     struct { int32_t rotations, pad; double cosine2; } seen = { 0, 0, 0. }; const double level = 8. * 2.220446049250313e-16 * sqrt((double)N);
     if (hipMemcpyAsync(&seen, counter, sizeof(seen), hipMemcpyDeviceToHost, stream) != hipSuccess || hipStreamSynchronize(stream) != hipSuccess) { return -3; }
+    if (seen.pad != 0) { return -5; }   /* a split round gave up (hykJacobiSweep passes no carry memory, so this cannot be set here; kept with the layout) */
     if (seen.rotations == 0 || seen.cosine2 <= level * level) { break; }
   }
   if (hykColumnNorms(stream, Complex, N, r, V, sigma) != 0) { return -3; }

@@ -108,16 +108,16 @@ int hykPotrfpStatic(hipStream_t stream, int32_t computeUnits, double eps, int32_
 /* SVD tail.  Replaces the cuSOLVER gesvdj call and the copies around it, src/gram_evd.cu:110-137. */
 int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t Gtype, const void* Rt, int32_t ldr, double* B);
 /* One sweep of one-sided Jacobi over the r columns of B (N x r, FP64, complex interleaved): every pair whose cosine exceeds
- * tol is rotated.  rotations: 16 bytes of device memory, zero before the call; afterwards rotations[0] = pairs rotated and
- * the double at rotations + 2 = the largest squared cosine the sweep met (rotated or not). */
+ * tol is rotated.  rotations: 16 bytes of device memory, zero before the call; afterwards rotations[0] = pairs rotated,
+ * rotations[1] != 0 if a workgroup gave up waiting for its partner (split rounds of hykJacobiSweepCarry: B is then not to be
+ * used) and the double at rotations + 2 = the largest squared cosine the sweep met (rotated or not). */
 int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations);
-/* The same sweep with hykJacobiCarryBytes(N, r) bytes of device memory (16-byte aligned) for its rounds: the products
- * inside a column block travel through it from one round to the next instead of being summed again (ignored by the
- * kernels of variant 1), and for real factors of up to 2048 rows it holds a second copy of the factor: the rounds that put
- * two workgroups on a block pair read one copy and write the other, so that neither partner can read what the other has
- * already rotated, whenever the device dispatches them.  The memory needs no initialisation and holds nothing a later
- * sweep relies on; B holds the result after every sweep. */
-size_t hykJacobiCarryBytes(int32_t N, int32_t r);
+/* The same sweep with hykJacobiCarryBytes(r) bytes of device memory (16-byte aligned) for its rounds: the products inside a
+ * column block travel through it from one round to the next instead of being summed again (ignored by the kernels of
+ * variant 1), and it holds the words through which the two workgroups that share a block pair (real factors of up to 2048
+ * rows, while the device holds them all at once) keep either from reading rows the other has already rotated.  The
+ * memory needs no initialisation and holds nothing a later sweep relies on. */
+size_t hykJacobiCarryBytes(int32_t r);
 int hykJacobiSweepCarry(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations, double* carry);
 /* The same sweep with two index limits.  Pairs of two columns with index >= top are not rotated (block pairs wholly behind
  * `top` are skipped); the largest cosine is reported over the pairs with at least one column before `head` only (the pairs

@@ -525,7 +525,7 @@ def test_jacobi_sweep_kernels(gl, variant, carry, cplx, N, r):
     B = (B @ mix) * 10.0 ** (-6.0 * np.arange(r) / r)                       # graded like a pivoted Cholesky factor
     want = np.linalg.svd(B, compute_uv=False)
     dB = dev(np.ascontiguousarray(B.T)); counter = zeros(64)
-    carried = zeros(gl.L.hykJacobiCarryBytes(N, r)); carried.fill_(255)       # all-ones bytes: NaN, must never be read before written
+    carried = zeros(gl.L.hykJacobiCarryBytes(r)); carried.fill_(255)       # all-ones bytes: NaN, must never be read before written
     tol = float(2.220446049250313e-16 * np.sqrt(N))
     assert gl.L.hykJacobiSetVariant(variant) == 0
     try:
@@ -572,7 +572,7 @@ def test_jacobi_sweeps_with_limits(gl, variant, carry, cplx, N, r, head, top):
     assert gl.L.hykJacobiSetVariant(variant) == 0
     try:
         dB = dev(np.ascontiguousarray(B.T)); counter = zeros(64)
-        carried = zeros(gl.L.hykJacobiCarryBytes(N, r)); carried.fill_(255)
+        carried = zeros(gl.L.hykJacobiCarryBytes(r)); carried.fill_(255)
         for sweeps in range(30):
             counter.zero_()
             print("jacobi limits", variant, carry, cplx, N, r, head, top, "sweep", sweeps, flush=True)
