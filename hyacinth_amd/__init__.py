@@ -31,7 +31,7 @@ API_SYMBOLS = [
 KERNEL_SYMBOLS = [
     "hykColumnExponents", "hykSliceRange", "hykQuantizeLimbs", "hykQuantizeCrt", "hykZeroRows",
     "hykGramWorkspaceBytes", "hykGramWorkspaceClear", "hykGramCrt", "hykGramLimbs", "hykGramSetSlab",
-    "hykGramProfile", "hykGramProfileRead", "hykMfmaCeiling", "hykGramRange", "hykDequantize", "hykPotrfpWorkspaceBytes", "hykPotrfp", "hykPotrfpLeftLooking", "hykPotrfpStaticMaxN", "hykPotrfpStatic", "hykFactorToB", "hykJacobiSweep", "hykJacobiSweepCarry", "hykJacobiSweepTop", "hykJacobiCarryBytes", "hykJacobiSetVariant",
+    "hykGramProfile", "hykGramProfileRead", "hykMfmaCeiling", "hykGramRange", "hykDequantize", "hykPotrfpWorkspaceBytes", "hykPotrfp", "hykPotrfpLeftLooking", "hykPotrfpStaticMaxN", "hykPotrfpStatic", "hykFactorToB", "hykJacobiSweep", "hykJacobiSweepCarry", "hykJacobiSweepTop", "hykJacobiCarryBytes", "hykJacobiSetVariant", "hykJacobiSetSplitTest",
     "hykColumnNorms", "hykBasisOut", "hykValuesOut", "hykInterpSolve", "hykInterpOut", "hykMatcopy",
     "hykSumSquares", "hykMatmulCf16", "hykGemm", "hykOrthonormalize", "hykLastStatus", "hykTestFailAllocation", "hykColumnExponentsOp", "hykQuantizeLimbsOp", "hykQuantizeCrtOp",
     "hykQuantizeScaleBatchOp", "hykHerkBatchOp", "hykLastHerkPlan", "hykMaxCosine",
@@ -95,6 +95,7 @@ def lib():
         L.hykGramLimbs.argtypes = [vp, i32, i32, i32, vp, i64, i32, i32, i32, vp, vp]
         L.hykGramSetSlab.argtypes = [i32]
         L.hykJacobiSetVariant.argtypes = [i32]
+        L.hykJacobiSetSplitTest.argtypes = [i32]
         L.hykJacobiSweep.argtypes = [vp, i32, i32, i32, vp, dbl, vp]
         L.hykJacobiSweepCarry.argtypes = [vp, i32, i32, i32, vp, dbl, vp, vp]
         L.hykJacobiSweepTop.argtypes = [vp, i32, i32, i32, i32, i32, vp, dbl, vp, vp]

@@ -34,8 +34,9 @@ inline int elem_bytes(int t) { static const int b[12] = { 8, 16, 4, 8, 2, 4, 16,
 
 /* Stream-ordered scratch from the handle's pool (reference: cudaMallocFromPoolAsync / cudaFreeAsync throughout).
  * When the handle owns its pool, blocks are kept and reused instead of being returned after every call: the runtime's
- * pool calls cost up to a millisecond each for multi-gigabyte blocks, more than the kernels between them.  All work of a
- * handle is ordered on its one stream, so a reused block is never touched by two calls at once.  hyacinDestroy frees them. */
+ * pool calls cost up to a millisecond each for multi-gigabyte blocks, more than the kernels between them.  The work of a
+ * handle is ordered on its stream, so a reused block is never touched by two calls at once; a block that was last used on
+ * another stream (the caller has changed handle->hipStream) is handed out after a device-wide wait.  hyacinDestroy frees them. */
 void* scratch_acquire(const hyacinHandle_t* h, size_t bytes, bool* kept);
 void scratch_release(const hyacinHandle_t* h, void* p, bool kept);
 void scratch_drop_all(const hyacinHandle_t* h);

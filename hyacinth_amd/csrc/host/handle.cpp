@@ -19,11 +19,11 @@ constexpr uint32_t OWNS_MEMPOOL = 0x4, OWNS_PINNED = 0x8, OWNS_TIMER = 0x10;   /
 
 struct EventTimer { std::vector<std::pair<hyh::Segment, hipEvent_t>> events; hyh::Segment last = hyh::Segment::untimed; };
 
-/* blocks kept per handle-owned pool */
-struct Block { void* p; size_t bytes; bool busy; };
+/* blocks kept per handle-owned pool; `stream`: the stream whose work used the block last */
+struct Block { void* p; size_t bytes; bool busy; hipStream_t stream; };
 std::mutex g_keptMutex; std::map<hipMemPool_t, std::vector<Block>> g_kept;
 
-std::atomic<int> g_failAllocation{ 0 };   /* test hook: the n-th scratch acquisition from now on fails */
+thread_local int g_failAllocation = 0;   /* test hook: the n-th scratch acquisition of this host thread from now on fails */
 
 bool env_get(const char* key, std::string& out) { const char* v = std::getenv(key); if (!v) { return false; } out = v; return true; }
 bool env_true(const std::string& s) { return s == "1" || s == "true" || s == "True"; }
@@ -71,22 +71,30 @@ void hyh::fail(int code, const char* what, const char* detail, const char* file,
 }
 
 extern "C" int hykLastStatus(void) { return hyh::call_status().code; }
-extern "C" int hykTestFailAllocation(int32_t nth) { g_failAllocation.store(nth > 0 ? nth : 0); return 0; }
+extern "C" int hykTestFailAllocation(int32_t nth) { g_failAllocation = nth > 0 ? nth : 0; return 0; }
 
 void* hyh::scratch_acquire(const hyacinHandle_t* h, size_t bytes, bool* kept) {
   void* p = nullptr; *kept = false;
-  if (g_failAllocation.load(std::memory_order_relaxed) > 0 && g_failAllocation.fetch_sub(1) == 1) { return nullptr; }
+  if (g_failAllocation > 0 && g_failAllocation-- == 1) { return nullptr; }
   if ((h->HandleOwnedResource & OWNS_MEMPOOL) && h->mempool) {
     std::lock_guard<std::mutex> lock(g_keptMutex);
     std::vector<Block>& blocks = g_kept[h->mempool]; Block* best = nullptr;
     for (Block& b : blocks) { if (!b.busy && b.bytes >= bytes && b.bytes / 4 <= bytes && (!best || b.bytes < best->bytes)) { best = &b; } }
-    if (best) { best->busy = true; *kept = true; return best->p; }
+    if (best) {
+      /* The caller may have put another stream into the handle since the block was last used (the fields may be edited
+       * between calls).  Work queued on the old stream may still touch the block, and that stream may no longer exist, so
+       * it cannot be waited on by name: the device is. */
+      if (best->stream != h->hipStream) { HYH_CHECK(hipDeviceSynchronize()); best->stream = h->hipStream; }
+      best->busy = true; *kept = true; return best->p;
+    }
     if (blocks.size() >= 64) {   /* many different sizes have come by: return the idle ones to the pool */
+      bool foreign = false; for (Block& b : blocks) { foreign = foreign || (!b.busy && b.stream != h->hipStream); }
+      if (foreign) { HYH_CHECK(hipDeviceSynchronize()); }   /* a block last used on another stream is freed on this one */
       std::vector<Block> live; for (Block& b : blocks) { if (b.busy) { live.push_back(b); } else { HYH_CHECK(hipFreeAsync(b.p, h->hipStream)); } } blocks.swap(live);
     }
     const size_t rounded = (bytes + 255) / 256 * 256;
     HYH_CHECK(hipMallocFromPoolAsync(&p, rounded, h->mempool, h->hipStream));
-    if (p) { blocks.push_back(Block{ p, rounded, true }); *kept = true; }
+    if (p) { blocks.push_back(Block{ p, rounded, true, h->hipStream }); *kept = true; }
     return p;
   }
   HYH_CHECK(hipMallocFromPoolAsync(&p, bytes, h->mempool, h->hipStream));
@@ -97,12 +105,14 @@ void hyh::scratch_release(const hyacinHandle_t* h, void* p, bool kept) {
   if (!kept) { HYH_CHECK(hipFreeAsync(p, h->hipStream)); return; }
   std::lock_guard<std::mutex> lock(g_keptMutex);
   auto it = g_kept.find(h->mempool); if (it == g_kept.end()) { return; }
-  for (Block& b : it->second) { if (b.p == p) { b.busy = false; return; } }
+  for (Block& b : it->second) { if (b.p == p) { b.busy = false; b.stream = h->hipStream; return; } }
 }
 
 void hyh::scratch_drop_all(const hyacinHandle_t* h) {
   std::lock_guard<std::mutex> lock(g_keptMutex);
   auto it = g_kept.find(h->mempool); if (it == g_kept.end()) { return; }
+  bool foreign = false; for (Block& b : it->second) { foreign = foreign || b.stream != h->hipStream; }
+  if (foreign) { HYH_CHECK(hipDeviceSynchronize()); }
   for (Block& b : it->second) { HYH_CHECK(hipFreeAsync(b.p, h->hipStream)); }
   g_kept.erase(it);
 }

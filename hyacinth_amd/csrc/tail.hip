@@ -460,7 +460,7 @@ template <int BC> __device__ __forceinline__ void carried_pair(int t, int& i, in
  * whose values are used can observe a store of the same launch.  The cosine, the rotation count and the carried
  * products are written by the workgroup that is sure to finish: the first half's, or the one that took the pair. */
 template <int ROWS, int BC, bool FULL, int THREADS, bool CARRY, int PASSES, bool SPLIT = false>
-__global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, int32_t nb, int32_t r, int32_t head, int32_t top, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations, double* __restrict__ carry, uint32_t* __restrict__ pairWords) {
+__global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, int32_t nb, int32_t r, int32_t head, int32_t top, int32_t round, double* __restrict__ B, double tol, int32_t* __restrict__ rotations, double* __restrict__ carry, uint32_t* __restrict__ pairWords, int32_t splitTest) {
   constexpr int NC = 2 * BC, NG = NC * (NC + 1) / 2, WAVES = THREADS / 64, STEPS = FULL ? NC - 1 : BC, GS = NC + 1;
   constexpr bool SLIM = CARRY && !FULL;                    /* norms and cross products only */
   constexpr uint32_t PW_COUNT = 3u, PW_LOADED = 4u, PW_TAKEN = 16u;   /* the pair's word: arrivals, loaded bits (<< half), pair taken by one workgroup */
@@ -558,7 +558,13 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
   for (int pass = 0; pass < PASSES; ++pass) {
   load_rows(pass);
   /* arrival at the pair's word, asked behind the row loads (memory answers a wavefront in order, and an atomic takes longer than a load: asked first, it would hold this wavefront's rows back); the answer is needed after the sums */
-  if constexpr (SPLIT) { if (wave == PWAVE && lane == 0) { arrival = __hip_atomic_fetch_add(word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); } }
+  if constexpr (SPLIT) {
+    if (wave == PWAVE && lane == 0) {
+      /* tests (hykJacobiSetSplitTest 1 / 2): this half's workgroup arrives only after the partner has taken the pair, as a workgroup does that the device dispatches late */
+      if ((splitTest == 1 && half == 1) || (splitTest == 2 && half == 0)) { for (int spin = 0; spin < (1 << 22) && !(__hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) & PW_TAKEN); ++spin) { __builtin_amdgcn_s_sleep(8); } }
+      arrival = __hip_atomic_fetch_add(word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
   HYK_JWAIT(); HYK_JSTAMP(1);
   /* products numbered by diagonal: p = d NC + c stands for (c, (c + d) % NC), d = 0 .. NC / 2 (the last diagonal only for
    * c < NC / 2): every unordered pair once, and p splits back into the pair by shifts.  Summed over the wavefront 32 at a time. */
@@ -610,6 +616,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
   __syncthreads();
   if constexpr (SPLIT) {
     if (pairTaken) { return; }   /* uniform: the partner rotates and stores both halves; what was loaded here may be half rotated and is dropped */
+    if (splitTest == 3 && half == 1) { return; }   /* tests: a partner that arrives and is never heard of again */
     /* Every load of this workgroup has returned: each thread has used its rows in the sums, and the barrier has passed.  Say
      * so.  The atomic is issued after that point in program order and orders nothing else: what the partner stores once it
      * has seen the bit cannot reach loads that have already delivered their values (a release here would also write the
@@ -774,7 +781,7 @@ __global__ __launch_bounds__(THREADS) void jacobi_gram_round_kernel(int32_t N, i
     if (wave == PWAVE && lane == 0 && !(early & (PW_LOADED << (half ^ 1)))) {
       const uint32_t mine = PW_LOADED << half, theirs = PW_LOADED << (half ^ 1);
       int decided = 0;
-      for (int spin = 0; decided == 0 && spin < (1 << 22); ++spin) {
+      for (int spin = 0; decided == 0 && spin < (splitTest == 3 ? 256 : (1 << 22)); ++spin) {
         const uint32_t seen = __hip_atomic_load(word, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
         if (seen & theirs) { decided = 1; }
         else if ((seen & PW_COUNT) == 1u) {   /* alone so far */
@@ -1161,6 +1168,7 @@ extern "C" int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t
 }
 
 /* one sweep = every pair of the r columns of B (N x r, FP64, complex interleaved) once; rotations counts the rotations applied */
+static thread_local int g_splitTest = 0;   /* hykJacobiSetSplitTest */
 static thread_local int g_jacobiVariant = 0;   /* 0: Gram-space rounds, 8-column blocks for real factors where they fit (default); 1: the step kernel everywhere; 2: Gram-space rounds, 4-column blocks */
 
 static int compute_units() {   /* of the device current on this thread */
@@ -1183,17 +1191,17 @@ static int gram_sweep(hipStream_t stream, int32_t N, int32_t r, int32_t head, in
     if (carry && splitGrid <= compute_units()) {
       uint32_t* words = reinterpret_cast<uint32_t*>(reinterpret_cast<char*>(carry) + carried_bytes(r));
       if (hykGramWorkspaceClear(stream, words, pair_word_bytes(r)) != 0) { return -3; }
-      jacobi_gram_round_kernel<ROWS, BC, true, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, tol, rotations, carry, nullptr);
-      for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, true, PASSES, true><<<splitGrid, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, tol, rotations, carry, words); }
+      jacobi_gram_round_kernel<ROWS, BC, true, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, tol, rotations, carry, nullptr, 0);
+      for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, true, PASSES, true><<<splitGrid, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, tol, rotations, carry, words, g_splitTest); }
       return hipGetLastError() == hipSuccess ? 0 : -3;
     }
   }
   if (carry) {
-    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, tol, rotations, carry, nullptr);
-    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, tol, rotations, carry, nullptr); }
+    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, tol, rotations, carry, nullptr, 0);
+    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, true, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, tol, rotations, carry, nullptr, 0); }
   } else {
-    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, false, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, tol, rotations, nullptr, nullptr);
-    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, false, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, tol, rotations, nullptr, nullptr); }
+    jacobi_gram_round_kernel<ROWS, BC, true, THREADS, false, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, 0, B, tol, rotations, nullptr, nullptr, 0);
+    for (int round = 1; round < nb - 1; ++round) { jacobi_gram_round_kernel<ROWS, BC, false, THREADS, false, PASSES><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, tol, rotations, nullptr, nullptr, 0); }
   }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
@@ -1218,6 +1226,8 @@ static int blocked_sweep(hipStream_t stream, int32_t N, int32_t r, int32_t head,
   for (int round = 1; round < nb - 1; ++round) { jacobi_block_round_kernel<CPLX, ROWS, BC, false, THREADS><<<nb / 2, THREADS, 0, stream>>>(N, nb, r, head, top, round, B, tol, rotations); }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
+
+extern "C" int hykJacobiSetSplitTest(int32_t mode) { if (mode < 0 || mode > 3) { return -1; } g_splitTest = mode; return 0; }
 
 extern "C" int hykJacobiSetVariant(int32_t variant) { if (variant < 0 || variant > 2) { return -1; } g_jacobiVariant = variant; return 0; }
 

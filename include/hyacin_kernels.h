@@ -130,6 +130,13 @@ int hykJacobiSweepTop(hipStream_t stream, int32_t Complex, int32_t N, int32_t r,
  * factors, 2 for complex ones above 2048 rows).  All rotate by the same rule, and for equal block sizes they visit the
  * pairs in the same order; kept selectable so that tests cover every kernel.  The setting is per host thread. */
 int hykJacobiSetVariant(int32_t variant);
+/* Test hook (no counterpart in the reference) for the rounds that put two workgroups on a block pair: what they do when the
+ * device does not start the partners together, forced from the host so that every kernel still ends normally.  0 (default)
+ * nothing forced; 1 / 2 the workgroup of the second / first half of the rows arrives only when its partner has taken the
+ * whole pair (and then leaves: the partner's result stands); 3 the second half's workgroup arrives and leaves without
+ * reporting its loads, and the first gives up after 256 polls: nothing of the pair is stored, rotations[1] is set and
+ * hyacinXGevd ends with status -5.  Per host thread. */
+int hykJacobiSetSplitTest(int32_t mode);
 int hykColumnNorms(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, const double* B, double* sigma);
 
 /* How far a set of columns is from orthogonal, from their Gram matrix (no counterpart in the reference, which takes what
@@ -186,12 +193,12 @@ int hykLastHerkPlan(hykHerkPlan* out);
 
 /* Status of the last outermost hyacin.h call made on the calling thread: 0, or the code of the first failure inside it
  * (a HIP error number, a negative kernel-layer return value, -4 a scratch allocation that failed, -5 a pivoted Cholesky
- * whose workgroups lost each other).  A failed call has launched nothing after the failure, returned 0 and written
+ * or a Jacobi round whose workgroups lost each other).  A failed call has launched nothing after the failure, returned 0 and written
  * neither S nor V (the pivot vector of an interpolation may already hold the pivots).  No counterpart in the reference, which drops every status in release builds (include/internal.hpp:232-236). */
 int hykLastStatus(void);
 
-/* Test hook (no counterpart in the reference): the nth scratch acquisition from now on, in any thread, fails as if the
- * memory pool were exhausted; 0 switches the hook off. */
+/* Test hook (no counterpart in the reference): the nth scratch acquisition that the calling host thread makes from now on
+ * fails as if the memory pool were exhausted; 0 switches the hook off.  Other threads' calls are not affected. */
 int hykTestFailAllocation(int32_t nth);
 
 #ifdef __cplusplus

@@ -554,6 +554,39 @@ def test_jacobi_sweep_kernels(gl, variant, carry, cplx, N, r):
     assert np.linalg.norm(Un - Qb @ (Qb.conj().T @ Un)) <= 1e-9 * np.sqrt(r)
 
 
+@pytest.mark.parametrize("N,r", [(2048, 96), (1000, 130), (2047, 33), (2048, 256)])
+def test_jacobi_split_rounds_with_a_late_partner(gl, N, r):
+    """The rounds that put two workgroups on a block pair, with the dispatch order forced from the host: the workgroup of
+    one half arrives only when its partner has taken the whole pair, finds that in the pair's word and leaves; the partner has
+    rotated and stored both halves.  Either way round the sweep leaves exactly the bits of the sweep in which the partners
+    start together (same sums, same rotations, same arithmetic on every row).  With a partner that arrives and then never
+    reports its loads, the waiting workgroup gives up: rotations[1] is set."""
+    from gpu_util import dev, host, ptr, stream, sync, zeros
+    rng = np.random.default_rng(7 * N + r)
+    B = rng.standard_normal((N, r)) @ (np.triu(rng.standard_normal((r, r))) * 0.1 + np.eye(r)) * 10.0 ** (-6.0 * np.arange(r) / r)
+    tol = float(2.220446049250313e-16 * np.sqrt(N))
+    out = {}
+    try:
+        for mode in (0, 1, 2, 3):
+            assert gl.L.hykJacobiSetSplitTest(mode) == 0
+            dB = dev(np.ascontiguousarray(B.T)); counter = zeros(64); carried = zeros(gl.L.hykJacobiCarryBytes(r)); carried.fill_(255)
+            flags = []
+            for sweep in range(1 if mode == 3 else 3):
+                counter.zero_()
+                print("split rounds", N, r, "mode", mode, "sweep", sweep, flush=True)
+                assert gl.L.hykJacobiSweepCarry(stream(), 0, N, r, ptr(dB), tol, ptr(counter), ptr(carried)) == 0
+                sync()
+                flags.append(int(host(counter, np.int32)[1]))
+            out[mode] = (host(dB, np.float64, (r, N)).copy(), int(host(counter, np.int32)[0]), flags)
+    finally:
+        gl.L.hykJacobiSetSplitTest(0)
+    assert out[0][2] == [0, 0, 0] and out[1][2] == [0, 0, 0] and out[2][2] == [0, 0, 0]
+    assert out[0][1] > 0
+    for mode in (1, 2):
+        assert out[mode][1] == out[0][1] and np.array_equal(out[mode][0], out[0][0])
+    assert out[3][2] == [1]
+
+
 @pytest.mark.parametrize("variant,carry", [(0, 1), (0, 0), (1, 0), (2, 1)])
 @pytest.mark.parametrize("cplx,N,r,head,top", [(0, 1000, 130, 37, 37), (0, 2048, 96, 40, 64), (1, 600, 50, 9, 9), (1, 2048, 40, 12, 20), (0, 700, 20, 5, 20), (0, 300, 40, 0, 0)])
 def test_jacobi_sweeps_with_limits(gl, variant, carry, cplx, N, r, head, top):
