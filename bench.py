@@ -143,6 +143,76 @@ def make_workload(torch, name):
     return St, N
 
 
+def recipe_expectation(name, rank):
+    """What the recipe of a workload fixes in closed form: the rank hyacinTsvdFit must return and the relative projection
+    residual |A - A V V^H| / |A| of a basis of `rank` vectors.  A = U diag(s) V^H + noise has, for M >> N, singular values
+    sigma_i^2 = s_i^2 + nu^2 M (nu^2: variance of a noise entry); the rank is the energy rule of the reference
+    (src/gram_evd.cu:58-60: keep i < K while sum_{j >= i} sigma_j^2 > eps^2 sum_j sigma_j^2) and the residual of the best
+    rank-r basis is sqrt(sum_{j >= r} sigma_j^2) / |A|.  The interpolation stops its pivoted Cholesky when the trace left
+    is eps^2 of the whole (src/hyacin_potrfp.cu:224-269), which is the squared residual of A = A[:, piv] X^H: expected eps."""
+    import numpy as np
+    num, at, opA, M, N, K, eps, alg, fit, desc = WORKLOADS[name]
+    cplx = at & 1
+    i = np.arange(N, dtype=np.float64)
+    if fit == "hyacinInterpolateFit":
+        return {"expected_rank": None, "expected_rel_residual": eps, "rule": "trace left after the pivoted Cholesky <= eps^2 trace(G)"}
+    if name == "gauss":
+        return {"expected_rank": None, "expected_rel_residual": None, "rule": "no closed form (Gaussian matrix)"}
+    if name == "cfg4":
+        # rank-256 product with entries CN(0, 1/256) on both sides: |L R|_F^2 = M N / 256 spread over 256 values; noise
+        # 1e-4 complex Gaussian plus the rounding of the cast to half (ulp 2^-15 at |a| ~ 1/16: variance 2^-30 / 12 per part)
+        nu2 = (1e-8 + 2 * 2.0 ** -30 / 12) * M
+        sig2 = np.full(N, nu2)
+        sig2[:256] += M * N / 256.0 / 256.0
+    else:
+        s = {"cfg1": 10.0 ** (-i / 16.0), "cfg2": 2.0 ** (-i / 32.0), "cfg3": 10.0 ** (-i / 128.0), "target": 10.0 ** (-i / 128.0)}[name]
+        noise = {"cfg2": 1e-7, "cfg3": 1e-14, "target": 1e-14}.get(name, 0.0)
+        sig2 = s * s + noise * noise * M * (2 if cplx else 1)
+    tail = np.concatenate([np.cumsum(sig2[::-1])[::-1], [0.0]])            # tail[r] = sum_{j >= r} sigma_j^2
+    cut = int(np.count_nonzero(tail[:N] > eps * eps * tail[0]))
+    return {"expected_rank": min(K, cut), "expected_rel_residual": float(np.sqrt(tail[min(rank, N)] / tail[0])) if rank is not None else None,
+            "rule": "energy rule on sigma_i^2 = s_i^2 + noise^2 M; residual = sqrt(sum_{j >= rank} sigma_j^2) / |A|"}
+
+
+def recipe_values(name):
+    """(s, bound): the singular values the recipe builds its matrix from and a bound on what its noise moves them by
+    (Weyl: the spectral norm of an M x N Gaussian matrix, nu (sqrt M + sqrt N), times sqrt 2 for complex entries); None for
+    the workloads whose values are not given in closed form."""
+    import numpy as np
+    num, at, opA, M, N, K, eps, alg, fit, desc = WORKLOADS[name]
+    i = np.arange(N, dtype=np.float64)
+    s = {"cfg1": 10.0 ** (-i / 16.0), "cfg2": 2.0 ** (-i / 32.0), "cfg3": 10.0 ** (-i / 128.0), "target": 10.0 ** (-i / 128.0)}.get(name)
+    if s is None:
+        return None
+    noise = {"cfg2": 1e-7, "cfg3": 1e-14, "target": 1e-14}.get(name, 0.0)
+    return s, noise * (math.sqrt(M) + math.sqrt(N)) * (math.sqrt(2.0) if at & 1 else 1.0)
+
+
+def fit_quality(torch, L, h, name, A, lda, rank, S, V):
+    """Measured counterpart of recipe_expectation (outside every timed region): the relative residual of what the fit
+    returned.  Truncated SVD: sqrt(hyacinCheckNorm(rank) / hyacinCheckNorm(0)).  Interpolation: |A - A[:, piv] X^H| / |A|
+    on a sample of 8192 rows (the rows of the recipes are statistically alike), in FP64 on the device."""
+    num, at, opA, M, N, K, eps, alg, fit, desc = WORKLOADS[name]
+    op, pA = opA.encode(), C.c_void_p(A.data_ptr())
+    if fit == "hyacinInterpolateFit":
+        rows = torch.arange(0, M, max(1, M // 8192), device="cuda")[:8192]
+        As = (A[:, rows].T if opA == "N" else A[rows]).double()                                   # sample x N
+        piv = S.view(torch.int32)[:N].long() - 1
+        X = V.view(torch.float64).reshape(K, N).T[:, :rank]                                       # N x rank
+        return float((As - As[:, piv[:rank]] @ X.T).norm() / As.norm())
+    err = L.hyacinCheckNorm(C.byref(h), op, M, N, pA, lda, rank, C.c_void_p(V.data_ptr()), N, at)
+    nrm = L.hyacinCheckNorm(C.byref(h), op, M, N, pA, lda, 0, None, N, at)
+    assert L.hykLastStatus() == 0 and nrm > 0
+    return math.sqrt(max(err, 0.0) / nrm)
+
+
+def fit_record(torch, L, h, name, A, lda, rank, S, V, ms):
+    num, at, opA, M, N, K, eps, alg, fit, desc = WORKLOADS[name]
+    rec = {"call": fit, "K": K, "rank": rank, "ms": ms, "timing": "median of 5 after 2 warm-ups", "rel_residual": fit_quality(torch, L, h, name, A, lda, rank, S, V)}
+    rec.update(recipe_expectation(name, rank))
+    return rec
+
+
 def cpu_baseline(Ahost, at, alg, order, u):
     """The oracle's quantize + int8 Gram + reconstruction on a row sample of the workload, all host cores."""
     import numpy as np
@@ -272,7 +342,7 @@ def brief(torch, ha, L, name, steps, warmup):
         assert L.hykLastStatus() == 0
         return {"workload": "%s: %s" % (name, desc), "ms_per_step": dt * 1e3, "value": M * N * (N + 1) * (4 if cplx else 1) / dt / 1e12, "unit": "TFLOP/s",
                 "pct_int8_mfma_peak": 100.0 * (plan.int8Ops / t_kernel / 1e12 if t_kernel > 0 else 0.0) / INT8_PEAK_TOPS, "contraction_calls": plan.gramCalls,
-                "fit": {"call": fit_name, "K": K, "rank": rank, "ms": sorted(times[2:])[len(times[2:]) // 2]}}
+                "fit": fit_record(torch, L, h, name, A, lda, rank, S, V, sorted(times[2:])[len(times[2:]) // 2])}
     finally:
         ha.destroy_handle(h)
 
@@ -458,7 +528,7 @@ def main():
         stages["quantize"]["frac_of_copy_stream"] = stages["quantize"]["GB/s"] / copy_gbs
         del src, dst
 
-    fit_ms, fit_rank, fit_gauss = None, None, None
+    fit_ms, fit_rank, fit_gauss, fit_rec = None, None, None, None
     if not a.no_fit:
         real = torch.float64 if at in (0, 1) else (torch.float32 if at in (2, 3) else torch.float16)
         S = torch.zeros(max(K, N), dtype=torch.float64, device="cuda")      # singular values, or the pivot vector of the interpolation
@@ -473,6 +543,7 @@ def main():
             times.append((time.perf_counter() - t1) * 1e3)
         assert L.hykLastStatus() == 0, "the fit reported a failure"
         fit_ms = sorted(times[2:])[len(times[2:]) // 2]
+        fit_rec = fit_record(torch, L, h, a.workload, A, lda, fit_rank, S, V, fit_ms)   # rank and residual against the recipe's closed form
         # The default workload also times the same fit on the Gaussian matrix of the same shape and accuracy (workload
         # "gauss"), on which the fit times quoted before the seeded recipes were measured: its Cholesky factor is close to
         # diagonal, so the Jacobi sweeps start in their quadratic phase (4 sweeps instead of the recipe's 10).
@@ -486,7 +557,8 @@ def main():
                 torch.cuda.synchronize()
                 gt.append((time.perf_counter() - t1) * 1e3)
             assert L.hykLastStatus() == 0, "the fit reported a failure"
-            fit_gauss = {"call": fit_name, "workload": "gauss: " + WORKLOADS["gauss"][9], "K": K, "rank": grank, "ms": sorted(gt[2:])[len(gt[2:]) // 2], "timing": "median of 5 after 2 warm-ups"}
+            fit_gauss = fit_record(torch, L, h, "gauss", Ag, ldag, grank, S, V, sorted(gt[2:])[len(gt[2:]) // 2])
+            fit_gauss["workload"] = "gauss: " + WORKLOADS["gauss"][9]
             del Ag
 
     roofline = {"bound": "mfma", "achieved": achieved, "peak": INT8_PEAK_TOPS, "unit": "TFLOP/s", "frac": achieved / INT8_PEAK_TOPS,
@@ -511,7 +583,7 @@ def main():
         "config": {"workload": "%s: %s" % (a.workload, desc), "M": M, "N": N, "opA": opA, "eps": eps, "algorithm": plan_alg, "order": order,
                    "quant_bits": u, "gram_limbs": lP, "row_slices": batches, "rows_per_contraction": plan_rows, "contraction_calls": plan.gramCalls},
         "pct_int8_mfma_peak": 100.0 * achieved / INT8_PEAK_TOPS,
-        "tsvd_fit_ms": fit_ms, "fit": {"call": fit_name, "K": K, "rank": fit_rank, "ms": fit_ms, "timing": "median of 5 after 2 warm-ups"},
+        "tsvd_fit_ms": fit_ms, "fit": fit_rec,
         "hbm_stages": stages,
         "roofline": roofline,
     }
