@@ -57,6 +57,7 @@ extern "C" void hyacinCreate(hyacinHandle_t* handle) {
   }
   if (handle->pinnedWorkspace == nullptr) { HYH_CHECK(hipHostMalloc(&handle->pinnedWorkspace, 64, hipHostMallocDefault)); handle->HandleOwnedResource |= OWNS_PINNED; }
 
+  if (env_get("HYACIN_PLAIN_LAUNCH", s)) { (void)hykPotrfpSetPlainLaunch(env_true(s) ? 1 : 0); }   /* for runs under a kernel-tracing profiler */
   const bool timer = env_get("HYACIN_CREATE_TIMER", s) ? env_true(s) : false;
   if (timer && handle->timer == nullptr) { handle->timer = new EventTimer(); handle->HandleOwnedResource |= OWNS_TIMER; }
   const bool verbose = env_get("HYACIN_VERBOSE", s) ? env_true(s) : false;

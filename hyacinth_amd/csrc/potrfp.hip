@@ -49,6 +49,12 @@ struct Record { uint64_t w[8]; };
 constexpr int RECORD_WORDS = 7;
 constexpr int STAGE_BYTES = 48 * 1024;
 constexpr int MAX_WORKGROUPS = 256;
+/* hykPotrfpSetPlainLaunch: the kernels here are launched cooperatively (the runtime then guarantees that all workgroups are
+ * resident, which their waits for each other rely on).  With this set, a grid that the occupancy query says fits the device
+ * is started with a plain launch instead: on an otherwise idle device that comes to the same, and a grid that does not
+ * become resident after all fails safe (every wait is bounded and gives the run up with rank -1). */
+std::atomic<int> g_plainLaunch{ 0 };
+
 constexpr int SPIN_LIMIT = 1 << 22;   /* polls of one record before the run is given up (seconds; a healthy wait is microseconds) */
 
 struct PotrfArgs {
@@ -276,6 +282,11 @@ template <bool DD, bool CPLX> int launch(hipStream_t stream, PotrfArgs& args, in
   int perCu = 0; if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, potrfp_kernel<DD, CPLX>, P_THREADS, 0) != hipSuccess || perCu < 1) { return -3; }
   int grid = cus < MAX_WORKGROUPS ? cus : MAX_WORKGROUPS; const int want = (args.N + P_WAVES - 1) / P_WAVES; if (grid > want) { grid = want; } if (grid < 1) { grid = 1; }
   if ((int64_t)grid * P_WAVES * 64 < args.N) { return -1; }   /* a wavefront tracks at most 64 columns */
+  if (g_plainLaunch.load(std::memory_order_relaxed)) {
+    int dev = 0, units = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) { return -3; }
+    if ((int64_t)grid <= (int64_t)units * perCu) { potrfp_kernel<DD, CPLX><<<grid, P_THREADS, 0, stream>>>(args); return hipGetLastError() == hipSuccess ? 0 : -3; }
+  }
   void* params[] = { &args };
   hipError_t e = hipLaunchCooperativeKernel(reinterpret_cast<const void*>(&potrfp_kernel<DD, CPLX>), dim3(grid), dim3(P_THREADS), params, 0, stream);
   return e == hipSuccess ? 0 : -3;
@@ -545,6 +556,7 @@ __global__ __launch_bounds__(THREADS) void potrfp_blocked_kernel(const Args a) {
         if (panel > 0) {   /* every workgroup has applied the previous panel to G' */
           const uint32_t want = (uint32_t)nwg * (uint32_t)panel; int spins = 0;
           while (__hip_atomic_load(reinterpret_cast<uint32_t*>(&a.ctl[CTL_COUNTER]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < want) { if (++spins > SPIN) { failed = true; break; } }
+          __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");   /* pairs with the release of the bump below: what the other workgroups wrote to G' and Rt before they bumped the counter is what the loads from here on see */
         }
         specCol = -1;
         HYK_STAMP(0);
@@ -753,9 +765,9 @@ __global__ __launch_bounds__(THREADS) void potrfp_blocked_kernel(const Args a) {
       }
       __syncthreads();
     }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   /* every thread's stores of this panel's update have left (the release below names the order; this wait is what makes it cheap for the one thread that bumps) */
     __syncthreads();
-    if (tid == 0) { __hip_atomic_fetch_add(reinterpret_cast<uint32_t*>(&a.ctl[CTL_COUNTER]), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+    if (tid == 0) { __hip_atomic_fetch_add(reinterpret_cast<uint32_t*>(&a.ctl[CTL_COUNTER]), 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT); }
     HYK_STAMP(6);
   }
 #ifdef HYK_POTRFP_TIMING
@@ -783,6 +795,11 @@ template <bool DD, bool CPLX> int launch(hipStream_t stream, Args& args, int cus
   if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes) != hipSuccess) { return -3; }
   int perCu = 0; if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, potrfp_blocked_kernel<DD, CPLX>, THREADS, ldsBytes) != hipSuccess || perCu < 1) { return -3; }
   int grid = cus < 256 ? cus : 256; if (grid < args.agents) { return -1; }
+  if (g_plainLaunch.load(std::memory_order_relaxed)) {   /* hykPotrfpSetPlainLaunch: see there */
+    int dev = 0, units = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) { return -3; }
+    if ((int64_t)grid <= (int64_t)units * perCu) { potrfp_blocked_kernel<DD, CPLX><<<grid, THREADS, ldsBytes, stream>>>(args); return hipGetLastError() == hipSuccess ? 0 : -3; }
+  }
   void* params[] = { &args };
   return hipLaunchCooperativeKernel(fn, dim3(grid), dim3(THREADS), params, (unsigned)ldsBytes, stream) == hipSuccess ? 0 : -3;
 }
@@ -821,6 +838,8 @@ int run_potrfp(hipStream_t stream, bool blocked, int32_t computeUnits, double ep
   return cplx ? launch<false, true>(stream, a, computeUnits) : launch<false, false>(stream, a, computeUnits);
 }
 }  // namespace
+
+extern "C" int hykPotrfpSetPlainLaunch(int32_t enable) { g_plainLaunch.store(enable ? 1 : 0, std::memory_order_relaxed); return 0; }
 
 extern "C" size_t hykPotrfpWorkspaceBytes(int32_t N, int32_t Gtype) {
   if (N <= 0) { return 0; }

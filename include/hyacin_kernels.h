@@ -96,6 +96,13 @@ int hykDequantize(hipStream_t stream, int32_t N, int32_t orderC, const uint64_t*
 size_t hykPotrfpWorkspaceBytes(int32_t N, int32_t Gtype);
 int hykPotrfp(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, int32_t N, int32_t Gtype, void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, void* workspace, int32_t* rankOut);
 int hykPotrfpLeftLooking(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, int32_t N, int32_t Gtype, void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, void* workspace, int32_t* rankOut);
+/* Process-wide launch mode of the two kernels above (no counterpart in the reference).  They are launched cooperatively by
+ * default.  enable != 0: a grid that fits the device by the occupancy query is started with a plain launch.  For runs under
+ * profilers whose kernel tracing does not get along with cooperative launches (rocprofv3 --kernel-trace: the process then
+ * ends with a segmentation fault in the runtime's exit handler, after the trace has been written); hyacinCreate switches
+ * it on when the environment variable HYACIN_PLAIN_LAUNCH is 1 / true.  The bounded waits inside the kernels make a grid
+ * that is not resident after all end with rank -1 (status -5) instead of hanging. */
+int hykPotrfpSetPlainLaunch(int32_t enable);
 
 /* hykPotrfp for callers that cannot allocate device memory (code under HIP graph capture, serving loops, harnesses that
  * forbid hipMalloc).  No counterpart in the reference.  The workspace of hykPotrfp (diagonal, position table, exchange

@@ -371,6 +371,30 @@ def test_potrfp_kernel(gl, oracle, entry, gbase, cplx, N, r, K, eps64, epsdd, fl
         assert not got[p[:t], t, :].any()
 
 
+@pytest.mark.parametrize("entry", ["hykPotrfp", "hykPotrfpLeftLooking"])
+@pytest.mark.parametrize("gbase,cplx,N", [(0, 0, 600), (6, 1, 300), (6, 0, 2048)])
+def test_potrfp_plain_launch(gl, entry, gbase, cplx, N):
+    """hykPotrfpSetPlainLaunch: the same kernels started with a plain launch (for runs under a kernel-tracing profiler) give
+    the rank, pivots and factor bits of the cooperative launch."""
+    from gpu_util import dev, zeros, ptr, stream, sync, host
+    rng = np.random.default_rng(43 + cplx + gbase)
+    gtype = gbase + cplx
+    raw = spd_raw(rng, N, min(N, 120), cplx, gbase, 1e-9)
+    width = raw.shape[2]
+    outs = []
+    try:
+        for plain in (0, 1):
+            assert gl.L.hykPotrfpSetPlainLaunch(plain) == 0
+            Rt, jp, rk, ws, dG = zeros(N * N * width * 8), zeros(N * 4), zeros(4), zeros(gl.L.hykPotrfpWorkspaceBytes(N, gtype)), dev(raw)
+            print(entry, "plain launch", plain, "N", N, "gtype", gtype, flush=True)
+            assert getattr(gl.L, entry)(stream(), 256, 1e-7, N, N, gtype, ptr(dG), N, ptr(Rt), N, ptr(jp), ptr(ws), ptr(rk)) == 0
+            sync()
+            outs.append((int(host(rk, np.int32)[0]), host(jp, np.int32).copy(), host(Rt, np.float64).copy()))
+    finally:
+        gl.L.hykPotrfpSetPlainLaunch(0)
+    assert outs[0][0] > 0 and outs[0][0] == outs[1][0] and np.array_equal(outs[0][1], outs[1][1]) and np.array_equal(outs[0][2], outs[1][2])
+
+
 @pytest.mark.parametrize("cplx", [0, 1])
 @pytest.mark.parametrize("opA", ["N", "T", "C"])
 @pytest.mark.parametrize("M,N,K,pad", [(300, 70, 45, 0), (128, 128, 64, 0), (1000, 260, 333, 8), (257, 129, 1, 0), (96, 40, 200, 3)])
