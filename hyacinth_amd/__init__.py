@@ -125,9 +125,9 @@ def lib():
         L.hykLastHerkPlan.argtypes = [C.POINTER(HerkPlan)]
         L.hykLastStatus.argtypes = []
         L.hykTestFailAllocation.argtypes = [i32]
-        L.hykFactorToB.argtypes = [vp, i32, i32, i32, vp, i32, vp]
+        L.hykFactorToB.argtypes = [vp, i32, i32, i32, vp, i32, i32, vp]
         L.hykColumnNorms.argtypes = [vp, i32, i32, i32, vp, vp]
-        L.hykBasisOut.argtypes = [vp, i32, i32, i32, vp, vp, vp, vp, i64]
+        L.hykBasisOut.argtypes = [vp, i32, i32, i32, i32, vp, vp, vp, vp, i64]
         L.hykValuesOut.argtypes = [vp, i32, i32, vp, vp]
         L.hykInterpSolve.argtypes = [vp, i32, i32, i32, vp, i32, vp, vp, vp]
         L.hykInterpOut.argtypes = [vp, i32, i32, i32, vp, vp, vp, i64]

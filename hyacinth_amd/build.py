@@ -15,7 +15,7 @@ ROOT = os.path.dirname(HERE)
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libhyacin.so")
 
-KERNELS = ["exponent.hip", "quantize.hip", "gram_mfma.hip", "dequantize.hip", "potrfp.hip", "tail.hip", "matcopy.hip", "gemm.hip"]
+KERNELS = ["exponent.hip", "quantize.hip", "gram_mfma.hip", "dequantize.hip", "potrfp.hip", "tail.hip", "tail_f32.hip", "matcopy.hip", "gemm.hip"]
 HOST = ["host/handle.cpp", "host/herk.cpp", "host/tail.cpp", "host/lra.cpp"]
 
 # -ffp-contract=off: the double-double code relies on error-free transforms.

@@ -6,7 +6,8 @@
  * src/gram_id.cpp:28-101 (interp, hyacinXGinterp).  The factorization itself runs in the HIP kernels of
  * potrfp.hip and tail.hip; no vendor solver is involved.  Differences that are visible to a caller:
  *  - an FP32 Gram is widened to FP64 before the Cholesky (the reference factors it in FP32);
- *  - the SVD always runs in FP64, also for FP32 / FP16 storage (the reference uses FP32 there);
+ *  - the SVD runs on a factor in doubles for FP64 storage and in floats for FP32 / FP16 storage, as the reference's does;
+ *    every rotation is worked out in FP64 either way;
  *  - the Jacobi iteration stops as soon as a sweep applies no rotation, or leaves only cosines that the quadratic
  *    contraction measured over the last two sweeps puts within 8 thresholds, or once the values that are handed out have
  *    stopped moving and their columns are orthogonal to sqrt(eps); a sweep here is one plain round-robin pass over all
@@ -75,10 +76,12 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
   { Factor f(handle, N, N, (int)Gtype, G, ldg);
     rank = run_potrfp(handle, f, lrqr ? eps : 0., N, N, jpiv.as<int32_t>());
     if (rank <= 0 || !hyh::ok()) { return 0; }
-    /* B = (R P^T)^H, N x rank, FP64 */
-    hyh::Scratch B(handle, (size_t)N * rank * 8 * (1 + Complex)), sigma(handle, sizeof(double) * (size_t)rank), counter(handle, 64), carry(handle, hykJacobiCarryBytes(rank));
+    /* B = (R P^T)^H, N x rank, in the precision of the output storage type: doubles for FP64, floats for FP32 and FP16
+     * (reference: src/gram_evd.cu:96-98) */
+    const bool wideB = (int)Atype == HYACIN_F64 || (int)Atype == HYACIN_F64_COMPLEX; const int Btype = (wideB ? HYACIN_F64 : HYACIN_F32) + Complex;
+    hyh::Scratch B(handle, (size_t)N * rank * (wideB ? 8 : 4) * (1 + Complex)), sigma(handle, sizeof(double) * (size_t)rank), counter(handle, 64), carry(handle, hykJacobiCarryBytes(rank));
     if (!hyh::ok()) { return 0; }
-    HYH_KERNEL(hykFactorToB(s, N, rank, f.type, f.Rt.p, f.ldr, B.as<double>()));
+    HYH_KERNEL(hykFactorToB(s, N, rank, f.type, f.Rt.p, f.ldr, Btype, B.p));
     const int32_t maxSweeps = sweeps > 0 ? 5 * sweeps : 30; int32_t used = 0;
     /* A pair is rotated while its cosine exceeds the storage precision, but never below sqrt(N) FP64 roundings: that is
      * what the dot product of two columns of length N carries as noise (the threshold of LAPACK's xGESVJ); rotating
@@ -88,7 +91,7 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
     std::vector<double> before((size_t)rank), after, sig;
     auto fetch_norms = [&](std::vector<double>& v, int32_t cols) {
       v.resize((size_t)cols);
-      HYH_KERNEL(hykColumnNorms(s, Complex, N, cols, B.as<double>(), sigma.as<double>()));
+      HYH_KERNEL(hykColumnNorms(s, Btype, N, cols, B.p, sigma.as<double>()));
       HYH_CHECK(hipMemcpyAsync(v.data(), sigma.p, sizeof(double) * (size_t)cols, hipMemcpyDeviceToHost, s));
     };
     /* How far the columns that can be handed out (the K largest norms) are from orthogonal: the largest cosine among them,
@@ -101,13 +104,13 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
       const int32_t kept = std::min(K, ncols);
       std::nth_element(order.begin(), order.begin() + (kept - 1), order.end(), [&](int32_t a, int32_t b) { return norm[(size_t)a] > norm[(size_t)b]; });
       for (int32_t i = 0; i < kept; ++i) { mark[(size_t)order[(size_t)i]] = 1; }
-      hyh::Scratch gram(handle, (size_t)ncols * ncols * 8 * (1 + Complex)), dMark(handle, sizeof(int32_t) * (size_t)ncols), dOut(handle, 64);
+      hyh::Scratch gram(handle, (size_t)ncols * ncols * (wideB ? 8 : 4) * (1 + Complex)), dMark(handle, sizeof(int32_t) * (size_t)ncols), dOut(handle, 64);
       if (!hyh::ok()) { return 0.; }
       double cos2 = 0.;
       HYH_CHECK(hipMemcpyAsync(dMark.p, mark.data(), sizeof(int32_t) * (size_t)ncols, hipMemcpyHostToDevice, s));
       HYH_KERNEL(hykGramWorkspaceClear(s, dOut.p, 64));
-      HYH_KERNEL(hykGemm(s, 'C', 'N', ncols, ncols, N, 1., HYACIN_F64 + Complex, B.p, N, B.p, N, 0., gram.p, ncols));
-      HYH_KERNEL(hykMaxCosine(s, Complex, ncols, gram.as<double>(), ncols, dMark.as<int32_t>(), dOut.as<double>()));
+      HYH_KERNEL(hykGemm(s, 'C', 'N', ncols, ncols, N, 1., Btype, B.p, N, B.p, N, 0., gram.p, ncols));
+      HYH_KERNEL(hykMaxCosine(s, Btype, ncols, gram.p, ncols, dMark.as<int32_t>(), dOut.as<double>()));
       HYH_CHECK(hipMemcpyAsync(&cos2, dOut.p, sizeof(double), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
       return std::sqrt(cos2);
     };
@@ -133,7 +136,7 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
         const int32_t top = watchOutput ? hyh::jacobi_tail_start(before, K, eps) : cols;   /* a broad floor of small columns is left alone */
         HYH_KERNEL(hykGramWorkspaceClear(s, counter.p, 64));
         const int32_t headCols = watchOutput ? std::min(top, hyh::jacobi_head(before, K)) : cols;   /* cosines are watched on the pairs that involve a column that can be handed out */
-        HYH_KERNEL(hykJacobiSweepTop(s, Complex, N, cols, headCols, top, B.as<double>(), rotateAbove, counter.as<int32_t>(), carry.as<double>())); ++used;
+        HYH_KERNEL(hykJacobiSweepTop(s, Btype, N, cols, headCols, top, B.p, rotateAbove, counter.as<int32_t>(), carry.as<double>())); ++used;
         if (watchOutput) { fetch_norms(after, cols); }
         struct { int32_t rotations, pad; double cosine2; } seen = { 0, 0, 0. };
         HYH_CHECK(hipMemcpyAsync(&seen, counter.p, sizeof(seen), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
@@ -174,10 +177,10 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
     HYH_CHECK(hipMemcpyAsync(dS.p, Sout.data(), sizeof(double) * (size_t)K, hipMemcpyHostToDevice, s));
     if (rank > 0) { HYH_CHECK(hipMemcpyAsync(dOrder.p, order.data(), sizeof(int32_t) * (size_t)rank, hipMemcpyHostToDevice, s)); }
     HYH_KERNEL(hykValuesOut(s, K, (int32_t)Atype, dS.as<double>(), S));
-    if (rank > 0) { HYH_KERNEL(hykBasisOut(s, N, rank, (int32_t)Atype, B.as<double>(), sigma.as<double>(), dOrder.as<int32_t>(), X, ldx)); }
+    if (rank > 0) { HYH_KERNEL(hykBasisOut(s, N, rank, (int32_t)Atype, Btype, B.p, sigma.as<double>(), dOrder.as<int32_t>(), X, ldx)); }
     HYH_CHECK(hipStreamSynchronize(s));   /* Sout / order are host temporaries */
     if (!hyh::ok()) { return 0; }
-    if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ-%s [eps=%.1le] [M=%d] [N=%d] [K=%d] [sweeps=%d] [SVD-rank=%d]\n", Complex ? "FP64-COMPLEX" : "FP64", eps, N, rank, K, used, svdRank); }
+    if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ-%s [eps=%.1le] [M=%d] [N=%d] [K=%d] [sweeps=%d] [SVD-rank=%d]\n", wideB ? (Complex ? "FP64-COMPLEX" : "FP64") : (Complex ? "FP32-COMPLEX" : "FP32"), eps, N, rank, K, used, svdRank); }
   }
   return hyh::ok() ? rank : 0;
 }

@@ -112,27 +112,32 @@ int hykPotrfpSetPlainLaunch(int32_t enable);
 int32_t hykPotrfpStaticMaxN(void);
 int hykPotrfpStatic(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, int32_t N, int32_t Gtype, void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, int32_t* rankOut);
 
-/* SVD tail.  Replaces the cuSOLVER gesvdj call and the copies around it, src/gram_evd.cu:110-137. */
-int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t Gtype, const void* Rt, int32_t ldr, double* B);
-/* One sweep of one-sided Jacobi over the r columns of B (N x r, FP64, complex interleaved): every pair whose cosine exceeds
+/* SVD tail.  Replaces the cuSOLVER gesvdj call and the copies around it, src/gram_evd.cu:110-137.
+ * The factor B = (R P^T)^H is N x rank, column-major, complex interleaved, in the precision the reference runs its SVD in
+ * (src/gram_evd.cu:96-98): Btype = HYK_F64 / HYK_F64C (0 / 1, doubles) for FP64 storage, HYK_F32 / HYK_F32C (2 / 3, floats)
+ * for FP32 and FP16 storage.  With floats a thread keeps its rows and does the arithmetic on them in single precision;
+ * the column products of a round are summed across threads in FP64 and every rotation is worked out in FP64. */
+int hykFactorToB(hipStream_t stream, int32_t N, int32_t rank, int32_t Gtype, const void* Rt, int32_t ldr, int32_t Btype, void* B);
+/* One sweep of one-sided Jacobi over the r columns of B (N x r of type Btype): every pair whose cosine exceeds
  * tol is rotated.  rotations: 16 bytes of device memory, zero before the call; afterwards rotations[0] = pairs rotated,
  * rotations[1] != 0 if a workgroup gave up waiting for its partner (split rounds of hykJacobiSweepCarry: B is then not to be
  * used) and the double at rotations + 2 = the largest squared cosine the sweep met (rotated or not). */
-int hykJacobiSweep(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations);
+int hykJacobiSweep(hipStream_t stream, int32_t Btype, int32_t N, int32_t r, void* B, double tol, int32_t* rotations);
 /* The same sweep with hykJacobiCarryBytes(r) bytes of device memory (16-byte aligned) for its rounds: the products inside a
  * column block travel through it from one round to the next instead of being summed again (ignored by the kernels of
  * variant 1), and it holds the words through which the two workgroups that share a block pair (real factors of up to 2048
  * rows, while the device holds them all at once) keep either from reading rows the other has already rotated.  The
  * memory needs no initialisation and holds nothing a later sweep relies on. */
 size_t hykJacobiCarryBytes(int32_t r);
-int hykJacobiSweepCarry(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, double* B, double tol, int32_t* rotations, double* carry);
+int hykJacobiSweepCarry(hipStream_t stream, int32_t Btype, int32_t N, int32_t r, void* B, double tol, int32_t* rotations, double* carry);
 /* The same sweep with two index limits.  Pairs of two columns with index >= top are not rotated (block pairs wholly behind
  * `top` are skipped); the largest cosine is reported over the pairs with at least one column before `head` only (the pairs
  * whose convergence the caller waits for), while rotations[0] still counts every rotation.  head = top = r is the plain
  * sweep.  carry may be null. */
-int hykJacobiSweepTop(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, int32_t head, int32_t top, double* B, double tol, int32_t* rotations, double* carry);
+int hykJacobiSweepTop(hipStream_t stream, int32_t Btype, int32_t N, int32_t r, int32_t head, int32_t top, void* B, double tol, int32_t* rotations, double* carry);
 /* Which kernel a sweep runs: 0 (default) one Gram matrix per round and workgroup, the steps of the round taken on it by
- * one wavefront; real factors in blocks of 8 columns, complex ones in blocks of 4, the rows in two halves where N > 2048;
+ * one wavefront; real factors in blocks of 8 columns, complex ones in blocks of 4, the rows of a factor in doubles in two
+ * halves where N > 2048;
  * 1 one reduction and barrier per step; 2 as 0 with the narrower blocks that hold all rows at once (4 columns for real
  * factors, 2 for complex ones above 2048 rows).  All rotate by the same rule, and for equal block sizes they visit the
  * pairs in the same order; kept selectable so that tests cover every kernel.  The setting is per host thread. */
@@ -144,14 +149,14 @@ int hykJacobiSetVariant(int32_t variant);
  * reporting its loads, and the first gives up after 256 polls: nothing of the pair is stored, rotations[1] is set and
  * hyacinXGevd ends with status -5.  Per host thread. */
 int hykJacobiSetSplitTest(int32_t mode);
-int hykColumnNorms(hipStream_t stream, int32_t Complex, int32_t N, int32_t r, const double* B, double* sigma);
+int hykColumnNorms(hipStream_t stream, int32_t Btype, int32_t N, int32_t r, const void* B, double* sigma);
 
 /* How far a set of columns is from orthogonal, from their Gram matrix (no counterpart in the reference, which takes what
- * gesvdj returns after its sweep budget, src/gram_evd.cu:9-42): G is n x n column-major FP64 (complex interleaved when
- * Complex), mark[p] != 0 selects the columns that count; *out (device, zero before the call) receives the largest
+ * gesvdj returns after its sweep budget, src/gram_evd.cu:9-42): G is n x n column-major of type Gtype (HYK_F64 / HYK_F64C /
+ * HYK_F32 / HYK_F32C, complex interleaved), mark[p] != 0 selects the columns that count; *out (device, zero before the call) receives the largest
  * |G[p, q]|^2 / (G[p, p] G[q, q]) over the marked pairs p < q. */
-int hykMaxCosine(hipStream_t stream, int32_t Complex, int32_t n, const double* G, int64_t ldg, const int32_t* mark, double* out);
-int hykBasisOut(hipStream_t stream, int32_t N, int32_t rank, int32_t Atype, const double* B, const double* sigma, const int32_t* order, void* X, int64_t ldx);
+int hykMaxCosine(hipStream_t stream, int32_t Gtype, int32_t n, const void* G, int64_t ldg, const int32_t* mark, double* out);
+int hykBasisOut(hipStream_t stream, int32_t N, int32_t rank, int32_t Atype, int32_t Btype, const void* B, const double* sigma, const int32_t* order, void* X, int64_t ldx);
 int hykValuesOut(hipStream_t stream, int32_t K, int32_t Atype, const double* S, void* out);
 
 /* Interpolation tail.  Replaces cuBLAS trsm + scatter modes 'U' / 'I', src/gram_id.cpp:40-46, src/matcopy.cu:48-52.

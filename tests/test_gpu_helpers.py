@@ -99,42 +99,47 @@ def test_zero_rows(L):
         assert np.array_equal(host(dB, np.int8, B.shape), want)
 
 
+@pytest.mark.parametrize("wide", [1, 0])
 @pytest.mark.parametrize("cplx", [0, 1])
 @pytest.mark.parametrize("dd", [0, 1])
-def test_factor_to_b(L, cplx, dd):
-    """B[c, k] = conj(R[k, c]) (high words of a double-double factor), src/gram_evd.cu:110-117."""
+def test_factor_to_b(L, cplx, dd, wide):
+    """B[c, k] = conj(R[k, c]) (high words of a double-double factor), src/gram_evd.cu:110-117, in doubles or rounded to floats
+    (the precision the SVD of that storage type runs in, src/gram_evd.cu:96-98)."""
     from gpu_util import dev, zeros, ptr, stream, sync, host
     rng = np.random.default_rng(61)
     N, rank, ldr = 70, 33, 40
     WR = 2 if dd else 1
     WE = WR * (2 if cplx else 1)
     Rt = rng.standard_normal((N, ldr, WE))
-    dR, B = dev(Rt), zeros(N * rank * 8 * (1 + cplx))
-    assert L.hykFactorToB(stream(), N, rank, (6 if dd else 0) + cplx, ptr(dR), ldr, ptr(B)) == 0
+    real = np.float64 if wide else np.float32
+    dR, B = dev(Rt), zeros(N * rank * (8 if wide else 4) * (1 + cplx))
+    assert L.hykFactorToB(stream(), N, rank, (6 if dd else 0) + cplx, ptr(dR), ldr, (0 if wide else 2) + cplx, ptr(B)) == 0
     sync()
-    got = host(B, np.float64, (rank, N, 1 + cplx))
-    assert np.array_equal(got[..., 0], Rt[:, :rank, 0].T)
+    got = host(B, real, (rank, N, 1 + cplx))
+    assert np.array_equal(got[..., 0], Rt[:, :rank, 0].T.astype(real))
     if cplx:
-        assert np.array_equal(got[..., 1], -Rt[:, :rank, WR].T)
+        assert np.array_equal(got[..., 1], (-Rt[:, :rank, WR].T).astype(real))
+    assert L.hykFactorToB(stream(), N, rank, (6 if dd else 0) + cplx, ptr(dR), ldr, 1 - cplx, ptr(B)) == -1     # real factor, complex B
 
 
+@pytest.mark.parametrize("wide", [1, 0])
 @pytest.mark.parametrize("atype", [ha.F64, ha.F32, ha.F16, ha.F64C, ha.F32C, ha.F16C])
-def test_basis_and_values_out(L, atype):
+def test_basis_and_values_out(L, atype, wide):
     """X[:, j] = B[:, order[j]] / sigma[order[j]] in the storage type (a zero column stays zero); S in the real storage type."""
     from gpu_util import dev, ptr, stream, sync, host
     rng = np.random.default_rng(62)
     cplx, real = atype & 1, NP_REAL[atype & ~1]
     N, r, ldx = 50, 9, 57
-    B = rng.standard_normal((r, N, 1 + cplx))
+    B = rng.standard_normal((r, N, 1 + cplx)).astype(np.float64 if wide else np.float32)
     sigma = rng.uniform(0.5, 2.0, r); sigma[4] = 0.0
     order = rng.permutation(r).astype(np.int32)[:7]
     X0 = np.full((7, ldx, 1 + cplx), 3.0, real)
     dB, dS, dO, dX = dev(B), dev(sigma), dev(order), dev(X0)
-    assert L.hykBasisOut(stream(), N, 7, atype, ptr(dB), ptr(dS), ptr(dO), ptr(dX), ldx) == 0
+    assert L.hykBasisOut(stream(), N, 7, atype, (0 if wide else 2) + cplx, ptr(dB), ptr(dS), ptr(dO), ptr(dX), ldx) == 0
     sync()
     got = host(dX, real, X0.shape)
     inv = np.where(sigma > 0, 1.0 / np.where(sigma > 0, sigma, 1.0), 0.0)
-    want = (B[order] * inv[order][:, None, None]).astype(real)
+    want = (B[order].astype(np.float64) * inv[order][:, None, None]).astype(real)
     assert np.array_equal(got[:, :N], want) and (got[:, N:] == 3.0).all()
     S = rng.uniform(0, 3, 11)
     dSi, dSo = dev(S), dev(np.zeros(11, real))
@@ -192,8 +197,9 @@ def test_orthonormalize(L, cplx, N, r):
 
 
 @pytest.mark.parametrize("cplx", [0, 1])
+@pytest.mark.parametrize("wide", [1, 0])
 @pytest.mark.parametrize("n,pad", [(2, 0), (37, 3), (300, 0)])
-def test_max_cosine(L, cplx, n, pad):
+def test_max_cosine(L, cplx, n, pad, wide):
     """hykMaxCosine: the largest |G[p, q]|^2 / (G[p, p] G[q, q]) over the marked pairs of a Gram matrix, against numpy;
     unmarked columns do not count, a zero diagonal entry under a non-zero product counts as 1."""
     from gpu_util import dev, zeros, ptr, stream, sync, host
@@ -202,7 +208,7 @@ def test_max_cosine(L, cplx, n, pad):
     X[:, 0] *= 1e-9
     G = X.conj().T @ X
     ld = n + pad
-    buf = np.full((n, ld, 2) if cplx else (n, ld), np.nan)          # [column][row]: column-major with padding rows
+    buf = np.full((n, ld, 2) if cplx else (n, ld), np.nan, np.float64 if wide else np.float32)   # [column][row]: column-major with padding rows
     if cplx:
         buf[:, :n, 0] = G.real.T
         buf[:, :n, 1] = G.imag.T
@@ -211,12 +217,14 @@ def test_max_cosine(L, cplx, n, pad):
     mark = (rng.random(n) < 0.7).astype(np.int32)
     mark[:2] = 1
     dG, dM, out = dev(buf), dev(mark), zeros(8)
-    assert L.hykMaxCosine(stream(), cplx, n, ptr(dG), ld, ptr(dM), ptr(out)) == 0
+    assert L.hykMaxCosine(stream(), (0 if wide else 2) + cplx, n, ptr(dG), ld, ptr(dM), ptr(out)) == 0
     sync()
+    if not wide:                                                    # what the kernel saw
+        G = (buf[:, :n, 0] + 1j * buf[:, :n, 1]).T.astype(np.complex128) if cplx else buf[:, :n].T.astype(np.float64)
     d = np.real(np.diag(G))
     c2 = np.abs(G) ** 2 / np.outer(d, d)
     keep = np.outer(mark, mark).astype(bool) & ~np.eye(n, dtype=bool)
     want = c2[keep].max()
     got = host(out, np.float64)[0]
     assert abs(got - want) <= 1e-12 * want
-    assert L.hykMaxCosine(stream(), cplx, n, ptr(dG), n - 1, ptr(dM), ptr(out)) == -1
+    assert L.hykMaxCosine(stream(), (0 if wide else 2) + cplx, n, ptr(dG), n - 1, ptr(dM), ptr(out)) == -1

@@ -533,49 +533,59 @@ def test_gemm_fp64(gl, cplx, opA, opB, M, N, K):
     assert np.abs(got - want).max() <= 1e-13 * np.abs(want).max() * max(1, K) ** 0.5
 
 
+@pytest.mark.parametrize("wide", [1, 0])
 @pytest.mark.parametrize("variant,carry", [(0, 0), (0, 1), (1, 0), (2, 0), (2, 1)])
 @pytest.mark.parametrize("cplx,N,r", [(0, 300, 40), (0, 1000, 130), (0, 2048, 96), (0, 2500, 70), (0, 4096, 40), (1, 600, 50), (1, 2048, 40), (1, 3000, 24), (1, 4096, 36), (0, 64, 64), (0, 700, 20), (0, 701, 40), (0, 1023, 64), (0, 2047, 33), (0, 2048, 256)])
-def test_jacobi_sweep_kernels(gl, variant, carry, cplx, N, r):
+def test_jacobi_sweep_kernels(gl, variant, carry, cplx, N, r, wide):
     """One-sided Jacobi sweeps on a graded N x r factor: every kernel behind hykJacobiSweep / hykJacobiSweepCarry (Gram-space
     rounds with blocks of 8 and of 4 columns, with and without the products inside a block carried from round to round in
     memory that starts as NaN, the step kernel, the pair kernel for few columns) must leave orthogonal columns whose norms are
     the singular values numpy finds, to 32 sqrt(r) eps of the largest (a column takes part in a few hundred rotations), and
-    whose span is unchanged.  Odd N takes the kernels' element-wise loads (columns not 16-byte aligned); r = 256 gives the 16
-    block pairs of a round that are numbered by XCD."""
+    whose span is unchanged.  Odd N takes the kernels' element-wise loads (columns not aligned to a pair of rows); r = 256
+    gives the 16 block pairs of a round that are numbered by XCD.  wide = 0: the factor in floats (the SVD of FP32 / FP16
+    storage, src/gram_evd.cu:96-98), eps that of single precision; above 2048 rows a workgroup then takes all rows at once."""
     from gpu_util import dev, host, ptr, stream, sync, zeros
     rng = np.random.default_rng(1000 * N + r + cplx)
+    real, eps = (np.float64, 2.220446049250313e-16) if wide else (np.float32, 1.1920929e-07)
+    cpx = np.complex128 if wide else np.complex64
+    btype = (0 if wide else 2) + cplx
     B = rng.standard_normal((N, r)) + (1j * rng.standard_normal((N, r)) if cplx else 0)
     mix = np.triu(rng.standard_normal((r, r))) * 0.1 + np.eye(r)          # columns correlated
-    B = (B @ mix) * 10.0 ** (-6.0 * np.arange(r) / r)                       # graded like a pivoted Cholesky factor
-    want = np.linalg.svd(B, compute_uv=False)
+    B = ((B @ mix) * 10.0 ** ((-6.0 if wide else -3.0) * np.arange(r) / r)).astype(cpx if cplx else real)   # graded like a pivoted Cholesky factor
+    want = np.linalg.svd(B.astype(np.complex128 if cplx else np.float64), compute_uv=False)
     dB = dev(np.ascontiguousarray(B.T)); counter = zeros(64)
     carried = zeros(gl.L.hykJacobiCarryBytes(r)); carried.fill_(255)       # all-ones bytes: NaN, must never be read before written
-    tol = float(2.220446049250313e-16 * np.sqrt(N))
+    tol = float(eps * np.sqrt(N))
     assert gl.L.hykJacobiSetVariant(variant) == 0
     try:
         sweeps = 0
         while True:
             counter.zero_()
-            print("jacobi", variant, cplx, N, r, "sweep", sweeps, flush=True)
+            print("jacobi", variant, cplx, N, r, "wide", wide, "sweep", sweeps, flush=True)
             if carry:
-                assert gl.L.hykJacobiSweepCarry(stream(), cplx, N, r, ptr(dB), tol, ptr(counter), ptr(carried)) == 0
+                assert gl.L.hykJacobiSweepCarry(stream(), btype, N, r, ptr(dB), tol, ptr(counter), ptr(carried)) == 0
             else:
-                assert gl.L.hykJacobiSweep(stream(), cplx, N, r, ptr(dB), tol, ptr(counter)) == 0
+                assert gl.L.hykJacobiSweep(stream(), btype, N, r, ptr(dB), tol, ptr(counter)) == 0
             sync(); sweeps += 1
             rotations = int(host(counter, np.int32)[0]); cos2 = float(host(counter, np.float64)[1])
+            assert int(host(counter, np.int32)[1]) == 0
             if rotations == 0:
                 break
             assert sweeps < 30, "no convergence"
         assert cos2 <= (8 * tol) ** 2
     finally:
         gl.L.hykJacobiSetVariant(0)
-    U = host(dB, np.complex128 if cplx else np.float64, (r, N)).T
+    U = host(dB, cpx if cplx else real, (r, N)).T.astype(np.complex128 if cplx else np.float64)
     got = np.sort(np.linalg.norm(U, axis=0))[::-1]
-    assert np.max(np.abs(got - want)) <= 32 * 2.220446049250313e-16 * want[0] * np.sqrt(r)
+    assert np.max(np.abs(got - want)) <= 32 * eps * want[0] * np.sqrt(r)
+    sig = zeros(8 * r)                                                     # hykColumnNorms on the same memory
+    assert gl.L.hykColumnNorms(stream(), btype, N, r, ptr(dB), ptr(sig)) == 0
+    sync()
+    assert np.max(np.abs(host(sig, np.float64) - np.linalg.norm(U, axis=0))) <= 1e-12 * want[0]
     Un = U / np.linalg.norm(U, axis=0)
     assert np.max(np.abs(Un.conj().T @ Un - np.eye(r))) <= 16 * tol
-    Qb, _ = np.linalg.qr(B)                                               # same column space
-    assert np.linalg.norm(Un - Qb @ (Qb.conj().T @ Un)) <= 1e-9 * np.sqrt(r)
+    Qb, _ = np.linalg.qr(B.astype(np.complex128 if cplx else np.float64))                                               # same column space
+    assert np.linalg.norm(Un - Qb @ (Qb.conj().T @ Un)) <= (1e-9 if wide else 1e-3) * np.sqrt(r)
 
 
 @pytest.mark.parametrize("N,r", [(2048, 96), (1000, 130), (2047, 33), (2048, 256)])
