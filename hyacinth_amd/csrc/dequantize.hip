@@ -11,6 +11,7 @@
  * to the 106-bit mantissa via error-free transforms (compile without FP
  * contraction).
  */
+#include <type_traits>
 #include <hip/hip_runtime.h>
 #include "hyk_common.h"
 #include "hyk_dd.h"
@@ -36,27 +37,63 @@ __device__ __forceinline__ dd_t conv_dd(int L, const uint64_t* a, int32_t e) {
   return dd_t{ ldexp(res.x, e), ldexp(res.y, e) };
 }
 
-/* KIND: 0 FP32, 1 FP64, 2 double-double */
+/* One element of G: W scalars of type T ({re}, {re, im}, {hi, lo} or {re hi, re lo, im hi, im lo}), stored in one piece. */
+template <typename T, int W> struct alignas(sizeof(T) * W > 16 ? 16 : sizeof(T) * W) Elem { T v[W]; };
+
+/* KIND: 0 FP32, 1 FP64, 2 double-double.  A workgroup takes one 32 x 32 tile (tile row <= tile column) of the upper
+ * triangle: thread (y, x) reads the limbs of C[y, x] (entries of a column are adjacent in the packed triangle, so 32
+ * threads read 256 adjacent bytes per limb), converts, stores G[y, x] (adjacent in y) and parks the value in LDS; after the
+ * barrier the tile is read across and its conjugate stored to the lower triangle as G[x, y], adjacent in x: both triangles
+ * leave in full lines (a thread per entry writing its own mirror image puts every element of the lower triangle into a
+ * line of its own).  Entries on the diagonal are written by the second pass (conjugated: the imaginary part of a
+ * diagonal entry is -0 where the integer is 0, as with the reference's order of its two stores,
+ * src/fp_i63tp_dequantize.cu:121-129). */
+constexpr int DQ_TILE = 32;
 template <int KIND, int CPLX>
 __global__ __launch_bounds__(256) void dequantize_kernel(int32_t N, int32_t L, const uint64_t* __restrict__ C, int64_t strideC, const int32_t* __restrict__ vexp, void* __restrict__ Gv, int64_t ldg) {
-  const int64_t y = (int64_t)blockIdx.x * 256 + threadIdx.x, x = blockIdx.y;
-  if (y > x) { return; }
-  const int32_t ex = vexp[x], ey = vexp[y]; const bool zero = (ex == HYK_INT_MAX || ey == HYK_INT_MAX); const int32_t e = zero ? 0 : -(ex + ey);
-  uint64_t re[3] = { 0, 0, 0 }, im[3] = { 0, 0, 0 }; const uint64_t* src = &C[hyk::tri_index(y, x)];
-  for (int l = 0; l < L; ++l) { re[l] = src[l * strideC]; if (CPLX) { im[l] = src[(L + l) * strideC]; } }
-  const int64_t up = y + x * ldg, lo = x + y * ldg;
-  if constexpr (KIND == 2) {
-    dd_t z{ 0., 0. }, vr = zero ? z : conv_dd(L, re, e), vi = (zero || !CPLX) ? z : conv_dd(L, im, e); double* g = reinterpret_cast<double*>(Gv);
-    if constexpr (CPLX) { double4* g4 = reinterpret_cast<double4*>(Gv); g4[up] = make_double4(vr.x, vr.y, vi.x, vi.y); g4[lo] = make_double4(vr.x, vr.y, -vi.x, -vi.y); }
-    else { double2* g2 = reinterpret_cast<double2*>(g); g2[up] = make_double2(vr.x, vr.y); g2[lo] = make_double2(vr.x, vr.y); }
-  } else if constexpr (KIND == 1) {
-    const double vr = zero ? 0. : conv_f64(L, re, e), vi = (zero || !CPLX) ? 0. : conv_f64(L, im, e);
-    if constexpr (CPLX) { double2* g2 = reinterpret_cast<double2*>(Gv); g2[up] = make_double2(vr, vi); g2[lo] = make_double2(vr, -vi); }
-    else { double* g = reinterpret_cast<double*>(Gv); g[up] = vr; g[lo] = vr; }
-  } else {
-    const float vr = zero ? 0.f : (float)conv_f64(L, re, e), vi = (zero || !CPLX) ? 0.f : (float)conv_f64(L, im, e);
-    if constexpr (CPLX) { float2* g2 = reinterpret_cast<float2*>(Gv); g2[up] = make_float2(vr, vi); g2[lo] = make_float2(vr, -vi); }
-    else { float* g = reinterpret_cast<float*>(Gv); g[up] = vr; g[lo] = vr; }
+  using T = std::conditional_t<KIND == 0, float, double>;
+  constexpr int W = (KIND == 2 ? 2 : 1) * (CPLX ? 2 : 1);
+  using E = Elem<T, W>;
+  if (blockIdx.x > blockIdx.y) { return; }   /* tile row > tile column: below the diagonal */
+  __shared__ E tile[DQ_TILE][DQ_TILE + 1];   /* [x][y], one element of padding per row */
+  const int y0 = (int)blockIdx.x * DQ_TILE, x0 = (int)blockIdx.y * DQ_TILE, ti = threadIdx.x % DQ_TILE, tj = threadIdx.x / DQ_TILE;
+  E* G = reinterpret_cast<E*>(Gv);
+  {
+    const int y = y0 + ti; const int32_t ey = y < N ? vexp[y] : 0;
+    #pragma unroll
+    for (int p = 0; p < DQ_TILE / 8; ++p) {
+      const int xl = tj + 8 * p, x = x0 + xl;
+      if (x >= N || y > x) { continue; }
+      const int32_t ex = vexp[x]; const bool zero = (ex == HYK_INT_MAX || ey == HYK_INT_MAX); const int32_t e = zero ? 0 : -(ex + ey);
+      uint64_t re[3] = { 0, 0, 0 }, im[3] = { 0, 0, 0 }; const uint64_t* src = &C[hyk::tri_index(y, x)];
+      for (int l = 0; l < L; ++l) { re[l] = src[l * strideC]; if (CPLX) { im[l] = src[(L + l) * strideC]; } }
+      E out;
+      if constexpr (KIND == 2) {
+        const dd_t z{ 0., 0. }, vr = zero ? z : conv_dd(L, re, e), vi = (zero || !CPLX) ? z : conv_dd(L, im, e);
+        out.v[0] = vr.x; out.v[1] = vr.y; if constexpr (CPLX) { out.v[2] = vi.x; out.v[3] = vi.y; }
+      } else if constexpr (KIND == 1) {
+        out.v[0] = zero ? 0. : conv_f64(L, re, e); if constexpr (CPLX) { out.v[1] = zero ? 0. : conv_f64(L, im, e); }
+      } else {
+        out.v[0] = zero ? 0.f : (float)conv_f64(L, re, e); if constexpr (CPLX) { out.v[1] = zero ? 0.f : (float)conv_f64(L, im, e); }
+      }
+      tile[xl][ti] = out;
+      if (y < x) { G[(int64_t)y + (int64_t)x * ldg] = out; }
+    }
+  }
+  __syncthreads();
+  {
+    const int x = x0 + ti;
+    #pragma unroll
+    for (int p = 0; p < DQ_TILE / 8; ++p) {
+      const int yl = tj + 8 * p, y = y0 + yl;
+      if (x >= N || y > x) { continue; }
+      E out = tile[ti][yl];
+      if constexpr (CPLX) {
+        #pragma unroll
+        for (int w = W / 2; w < W; ++w) { out.v[w] = -out.v[w]; }
+      }
+      G[(int64_t)x + (int64_t)y * ldg] = out;
+    }
   }
 }
 
@@ -65,7 +102,7 @@ __global__ __launch_bounds__(256) void dequantize_kernel(int32_t N, int32_t L, c
 extern "C" int hykDequantize(hipStream_t stream, int32_t N, int32_t orderC, const uint64_t* C, const int32_t* vexp, int32_t Gtype, void* G, int64_t ldg) {
   if (N <= 0) { return 0; }
   if (orderC < 1 || orderC > 3 || N > 65535 || ldg < N) { return -1; }
-  const int64_t strideC = ((int64_t)N * N + N) / 2; dim3 grid((uint32_t)((N + 255) / 256), (uint32_t)N);
+  const int64_t strideC = ((int64_t)N * N + N) / 2; const uint32_t tiles = (uint32_t)((N + DQ_TILE - 1) / DQ_TILE); dim3 grid(tiles, tiles);
   switch (Gtype) {
     case HYK_F32: dequantize_kernel<0, 0><<<grid, 256, 0, stream>>>(N, orderC, C, strideC, vexp, G, ldg); break;
     case HYK_F32C: dequantize_kernel<0, 1><<<grid, 256, 0, stream>>>(N, orderC, C, strideC, vexp, G, ldg); break;
@@ -75,5 +112,5 @@ extern "C" int hykDequantize(hipStream_t stream, int32_t N, int32_t orderC, cons
     case HYK_DDC: dequantize_kernel<2, 1><<<grid, 256, 0, stream>>>(N, orderC, C, strideC, vexp, G, ldg); break;
     default: return -1;  /* triple-float / quad-float Grams are only chosen on GPUs without fast FP64 */
   }
-  return 0;
+  return hipGetLastError() == hipSuccess ? 0 : -3;
 }
