@@ -12,6 +12,7 @@
  * products C = op(A) B, the shape of matmul_cf16_{cn,tn,nn} and of the stage products of the segmented fit, run on the
  * matrix cores (the two kernels below).
  */
+#include <type_traits>
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 #include "hyk_common.h"
@@ -48,6 +49,13 @@ __global__ __launch_bounds__(256) void gemm_kernel(char opA, char opB, int32_t M
     #pragma unroll
     for (int j = 0; j < 4; ++j) { cr[i][j] = 0; ci[i][j] = 0; }
   }
+  typedef double d4_t __attribute__((ext_vector_type(4)));
+  [[maybe_unused]] d4_t mr[2][2], mi[2][2];   /* FP64: accumulators of the matrix-core blocks, [block of n][block of m] */
+  #pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    #pragma unroll
+    for (int j = 0; j < 2; ++j) { mr[i][j] = d4_t{ 0., 0., 0., 0. }; mi[i][j] = d4_t{ 0., 0., 0., 0. }; }
+  }
   for (int k0 = 0; k0 < K; k0 += GK) {
     #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -56,6 +64,34 @@ __global__ __launch_bounds__(256) void gemm_kernel(char opA, char opB, int32_t M
       { const int j = (opB == 'N') ? (p >> 4) : (p & 63), kk = (opB == 'N') ? (p & 15) : (p >> 6); Acc re, im; fetch<S, CPLX>(B, ldb, opB, k0 + kk, n0 + j, (n0 + j) < N && (k0 + kk) < K, re, im); sb[kk][j][0] = re; if constexpr (CPLX) { sb[kk][j][1] = im; } }
     }
     __syncthreads();
+    if constexpr (std::is_same<S, double>::value) {
+      /* FP64 on the matrix cores: v_mfma_f64_16x16x4_f64, a wavefront takes a 32 x 32 quarter of the tile as 2 x 2 blocks.
+       * The instruction's row operand is B (lane: column n = lane % 16 of the block, k = lane / 16) and its column operand
+       * op(A) (row m = lane % 16, k = lane / 16), so that a lane ends up with entries C[m, lane / 16 + 4 r] (the FP64 blocks interleave their rows over the four register pairs): lanes 0-15
+       * store 16 adjacent rows m.  Complex products as four real ones (the negated imaginary part makes -Ai Bi). */
+      const int lane = tid & 63, wave = tid >> 6, l16 = lane & 15, lk = lane >> 4, mb = (wave & 1) * 32, nb = (wave >> 1) * 32;
+      #pragma unroll
+      for (int k4 = 0; k4 < GK / 4; ++k4) {
+        const int kk = 4 * k4 + lk;
+        double ar[2], ai[2], br[2], bi[2];
+        #pragma unroll
+        for (int b = 0; b < 2; ++b) { ar[b] = sa[kk][mb + 16 * b + l16][0]; br[b] = sb[kk][nb + 16 * b + l16][0]; if constexpr (CPLX) { ai[b] = sa[kk][mb + 16 * b + l16][1]; bi[b] = sb[kk][nb + 16 * b + l16][1]; } }
+        #pragma unroll
+        for (int bn = 0; bn < 2; ++bn) {
+          #pragma unroll
+          for (int bm = 0; bm < 2; ++bm) {
+            mr[bn][bm] = __builtin_amdgcn_mfma_f64_16x16x4f64(br[bn], ar[bm], mr[bn][bm], 0, 0, 0);
+            if constexpr (CPLX) {
+              mr[bn][bm] = __builtin_amdgcn_mfma_f64_16x16x4f64(-bi[bn], ai[bm], mr[bn][bm], 0, 0, 0);
+              mi[bn][bm] = __builtin_amdgcn_mfma_f64_16x16x4f64(bi[bn], ar[bm], mi[bn][bm], 0, 0, 0);
+              mi[bn][bm] = __builtin_amdgcn_mfma_f64_16x16x4f64(br[bn], ai[bm], mi[bn][bm], 0, 0, 0);
+            }
+          }
+        }
+      }
+      __syncthreads();
+      continue;
+    }
     #pragma unroll
     for (int kk = 0; kk < GK; ++kk) {
       Acc ar[4], ai[4], br[4], bi[4];
@@ -70,6 +106,23 @@ __global__ __launch_bounds__(256) void gemm_kernel(char opA, char opB, int32_t M
       }
     }
     __syncthreads();
+  }
+  if constexpr (std::is_same<S, double>::value) {
+    const int lane = tid & 63, wave = tid >> 6, l16 = lane & 15, lk = lane >> 4, mb = (wave & 1) * 32, nb = (wave >> 1) * 32;
+    #pragma unroll
+    for (int bn = 0; bn < 2; ++bn) {
+      #pragma unroll
+      for (int bm = 0; bm < 2; ++bm) {
+        #pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int64_t m = m0 + mb + 16 * bm + l16, n = n0 + nb + 16 * bn + lk + 4 * r; if (m >= M || n >= N) { continue; }
+          double* c = reinterpret_cast<double*>(&C[(m + n * ldc) * W]);
+          if constexpr (CPLX) { double orr = 0., oi = 0.; if (beta != 0.) { orr = c[0]; oi = c[1]; } c[0] = alpha * mr[bn][bm][r] + beta * orr; c[1] = alpha * mi[bn][bm][r] + beta * oi; }
+          else { double o = 0.; if (beta != 0.) { o = c[0]; } c[0] = alpha * mr[bn][bm][r] + beta * o; }
+        }
+      }
+    }
+    return;
   }
   #pragma unroll
   for (int i = 0; i < 4; ++i) {
