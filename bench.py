@@ -38,12 +38,17 @@ INT8_PEAK_TOPS = 5000.0   # MI355X dense INT8 MFMA peak, 5.0 POP/s
 HBM_PEAK_GBS = 8000.0     # MI355X HBM3E peak, 8 TB/s
 SEED0 = 0x48594143494E0000
 
+RECIPE = {"cfg4seg": "cfg4"}   # workloads that share another one's matrix
+
 WORKLOADS = {
     # name: (number, type, opA, M, N, K, eps, algorithm, fit entry point, description)
     "cfg1": (1, 0, "N", 4096, 256, 256, 1e-10, b"L", "hyacinTsvdFit", "real FP64 M=4096 N=256 eps=1e-10: U diag(10^(-i/16)) V^T (limbs, 6 digits)"),
     "cfg2": (2, 2, "T", 65536, 1024, 512, 1e-5, b"A", "hyacinTsvdFit", "real FP32 opA=T (stored N x M) M=65536 N=1024 eps=1e-5: U diag(2^(-i/32)) V^T + 1e-7 G (CRT real, 8 moduli)"),
     "cfg3": (3, 1, "N", 131072, 2048, 1024, 1e-12, b"A", "hyacinTsvdFitSegmentN", "complex FP64 M=131072 N=2048 eps=1e-12: U diag(10^(-i/128)) V^H + 1e-14 (Gr + i Gi) (CRT complex, 15 moduli)"),
     "cfg4": (4, 5, "C", 262144, 4096, 256, 1e-3, b"L", "hyacinTsvdFit", "complex FP16 opA=C (stored N x M) M=262144 N=4096 eps=1e-3: rank-256 L R + 1e-4 noise (limbs, 3 digits x 3 groups)"),
+    # configuration 4's matrix through the column-segmented fit: N = 4096, K = 256 gives four segments of 1024 columns, whose
+    # bases are combined with the complex FP16 products on the matrix cores (matmul_cf16_cn, then _nn; src/lra.cpp:106-115)
+    "cfg4seg": (4, 5, "C", 262144, 4096, 256, 1e-3, b"L", "hyacinTsvdFitSegmentN", "complex FP16 opA=C M=262144 N=4096 eps=1e-3, configuration 4's matrix: column-segmented fit, 4 segments"),
     "cfg5": (5, 0, "N", 1048576, 4096, 2048, 1e-8, b"A", "hyacinInterpolateFit", "real FP64 M=1048576 N=4096 eps=1e-8: (U diag(10^(-i/256)) V^T) D, D log-uniform in [1e-6, 1e6] (CRT real, 11 moduli)"),
     "target": (6, 0, "N", 131072, 2048, 1024, 1e-12, b"A", "hyacinTsvdFit", "real FP64 M=131072 N=2048 eps=1e-12: U diag(10^(-i/128)) V^T + 1e-14 G (CRT real, 14 moduli)"),
     # the target's shape on a plain Gaussian matrix with column scales 10^(-8 j / N): full numerical rank, well separated
@@ -111,6 +116,7 @@ def make_workload(torch, name):
     """Returns (tensor as the configuration stores it, lda).  opA = 'N': column-major M x N, tensor [N][M](, 2);
     opA = 'T' / 'C': the stored N x M matrix, tensor [M][N](, 2) (conjugated for 'C', so that op(stored) = A)."""
     num, at, opA, M, N, K, eps, alg, fit, desc = WORKLOADS[name]
+    name = RECIPE.get(name, name)
     g = torch.Generator(device="cuda")
     g.manual_seed(SEED0 + num)
     cplx = at & 1
@@ -152,6 +158,7 @@ def recipe_expectation(name, rank):
     is eps^2 of the whole (src/hyacin_potrfp.cu:224-269), which is the squared residual of A = A[:, piv] X^H: expected eps."""
     import numpy as np
     num, at, opA, M, N, K, eps, alg, fit, desc = WORKLOADS[name]
+    name = RECIPE.get(name, name)
     cplx = at & 1
     i = np.arange(N, dtype=np.float64)
     if fit == "hyacinInterpolateFit":
@@ -180,6 +187,7 @@ def recipe_values(name):
     the workloads whose values are not given in closed form."""
     import numpy as np
     num, at, opA, M, N, K, eps, alg, fit, desc = WORKLOADS[name]
+    name = RECIPE.get(name, name)
     i = np.arange(N, dtype=np.float64)
     s = {"cfg1": 10.0 ** (-i / 16.0), "cfg2": 2.0 ** (-i / 32.0), "cfg3": 10.0 ** (-i / 128.0), "target": 10.0 ** (-i / 128.0)}.get(name)
     if s is None:
@@ -610,7 +618,7 @@ def main():
         ha.destroy_handle(h)
         h = None
         others = []
-        for name in ("cfg1", "cfg2", "cfg3", "cfg4", "cfg5"):
+        for name in ("cfg1", "cfg2", "cfg3", "cfg4", "cfg4seg", "cfg5"):
             torch.cuda.empty_cache()
             try:
                 others.append(brief(torch, ha, L, name, a.steps, a.warmup))

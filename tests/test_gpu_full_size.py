@@ -159,6 +159,7 @@ def test_fit_at_full_width(env, at, M, N, K, eps):
 API_CASES = [
     ("config 2: hyacinTsvdFit opA=T real FP32 65536 x 1024", "hyacinTsvdFit", F32, "T", 65536, 1024, 512, 1e-5, b"A", 1 << 10, 64),
     ("config 4: hyacinTsvdFit opA=C complex FP16 262144 x 4096, limbs", "hyacinTsvdFit", F16C, "C", 262144, 4096, 256, 1e-3, b"L", 30, 32),
+    ("config 4 segmented: hyacinTsvdFitSegmentN on the same matrix (four column segments, complex FP16 stage products)", "hyacinTsvdFitSegmentN", F16C, "C", 262144, 4096, 256, 1e-3, b"L", 30, 32),
     ("config 5: hyacinInterpolateFit real FP64 1048576 x 4096", "hyacinInterpolateFit", F64, "N", 1048576, 4096, 2048, 1e-8, b"A", 1 << 16, 32),
     ("config 3: hyacinTsvdFitSegmentN complex FP64 131072 x 2048", "hyacinTsvdFitSegmentN", F64C, "N", 131072, 2048, 1024, 1e-12, b"A", 1 << 20, 64),
 ]
