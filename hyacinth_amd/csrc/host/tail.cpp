@@ -99,13 +99,18 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
      * of what the vectors still lack: singular values 2 % apart leave their vectors several per cent away from orthogonal
      * when the values have long stopped moving.  What is handed out as singular vectors is held to sqrt(eps): the
      * projector V V^H is then right to eps. */
+    /* (its scratch -- the Gram matrix of the columns, the marks, the result word -- is taken once, before the sweeps: whether a
+     * sweep ends "settled" depends on the data, and an allocation in the middle of the loop would make the calls that can
+     * fail depend on it too; needed only when fewer values are handed out than the factor has columns) */
+    const bool mayCheck = K < rank && rank > 1;
+    hyh::Scratch gram(handle, mayCheck ? (size_t)rank * rank * (wideB ? 8 : 4) * (1 + Complex) : 0), dMark(handle, mayCheck ? sizeof(int32_t) * (size_t)rank : 0), dOut(handle, mayCheck ? 64 : 0);
+    if (!hyh::ok()) { return 0; }
     auto handed_out_defect = [&](const std::vector<double>& norm, int32_t ncols) -> double {
       std::vector<int32_t> order((size_t)ncols), mark((size_t)ncols, 0); std::iota(order.begin(), order.end(), 0);
       const int32_t kept = std::min(K, ncols);
       std::nth_element(order.begin(), order.begin() + (kept - 1), order.end(), [&](int32_t a, int32_t b) { return norm[(size_t)a] > norm[(size_t)b]; });
       for (int32_t i = 0; i < kept; ++i) { mark[(size_t)order[(size_t)i]] = 1; }
-      hyh::Scratch gram(handle, (size_t)ncols * ncols * (wideB ? 8 : 4) * (1 + Complex)), dMark(handle, sizeof(int32_t) * (size_t)ncols), dOut(handle, 64);
-      if (!hyh::ok()) { return 0.; }
+      if (!gram.p || !hyh::ok()) { return 0.; }
       double cos2 = 0.;
       HYH_CHECK(hipMemcpyAsync(dMark.p, mark.data(), sizeof(int32_t) * (size_t)ncols, hipMemcpyHostToDevice, s));
       HYH_KERNEL(hykGramWorkspaceClear(s, dOut.p, 64));

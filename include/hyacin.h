@@ -77,7 +77,23 @@ int32_t hyacinInterpolateFit(
 
 /* reference: include/hyacin.h:83-97, src/lra.cpp:52-84,222-232.
  * Truncated SVD right basis V (N x rank) and singular values S (K reals of the
- * storage precision; entries >= rank are zero).  Returns rank. */
+ * storage precision; entries >= rank are zero).  Returns rank.
+ *
+ * How the SVD of the Cholesky factor ends here (the reference hands the factor to the
+ * vendor's gesvdj with handle->JacobiSVDSweeps as its sweep limit, src/gram_evd.cu:148-150):
+ *  - the sweeps are plain round-robin Jacobi sweeps, each of which does less than a sweep of
+ *    the vendor's blocked solver, so the limit is 5 * |JacobiSVDSweeps| of them: 15 with the
+ *    default of 3; JacobiSVDSweeps == 0 (the reference's bidiagonalization backend) means a
+ *    limit of 30.  They end earlier when a sweep finds no pair above the rotation threshold,
+ *    or, with K below the rank of the factor, when the K values handed out have stopped
+ *    moving and their vectors are orthogonal to sqrt(eps);
+ *  - what is guaranteed for the result: S agrees with the singular values of op(A) to
+ *    10 eps S[0] (eps clamped to the machine precision of the storage type), and the columns
+ *    of V are orthonormal to max(sqrt(eps), rounding of the storage type) in every entry of
+ *    V^H V - I, to max(eps, 1e-12) when all of the factor's columns are handed out (K >= rank
+ *    of the factor), so that the projector V V^H is right to eps;
+ *  - a failure (allocation, launch, workgroups that lost each other) returns rank 0 with S
+ *    and V untouched; hykLastStatus() in hyacin_kernels.h tells which. */
 int32_t hyacinTsvdFit(
   const hyacinHandle_t* handle, double eps, char opA,
   int32_t M, int32_t N, int32_t K,

@@ -104,11 +104,13 @@ int hykPotrfpLeftLooking(hipStream_t stream, int32_t computeUnits, double eps, i
  * that is not resident after all end with rank -1 (status -5) instead of hanging. */
 int hykPotrfpSetPlainLaunch(int32_t enable);
 
-/* hykPotrfp for callers that cannot allocate device memory (code under HIP graph capture, serving loops, harnesses that
- * forbid hipMalloc).  No counterpart in the reference.  The workspace of hykPotrfp (diagonal, position table, exchange
- * records; 197 120 bytes) is a device array built into the library, one copy per device, so the call allocates nothing; inputs
- * and outputs are the caller's as in hykPotrfp.  N <= hykPotrfpStaticMaxN() (8192), larger N returns -2 with a message on
- * stderr.  All calls on one device share the array: calls that overlap on one device (two streams, two threads) race. */
+/* hykPotrfp for callers that may not call hipMalloc (serving loops, harnesses that forbid it).  No counterpart in the
+ * reference.  The workspace of hykPotrfp (diagonal, position table, exchange records; 197 120 bytes) is a device array
+ * built into the library, one copy per device, so the call allocates no device memory; inputs and outputs are the caller's
+ * as in hykPotrfp.  N <= hykPotrfpStaticMaxN() (8192), larger N returns -2 with a message on stderr.  The first call on a
+ * device looks the array's address up and sets a kernel attribute (which may load the code object): make one warm-up call
+ * outside any region that must not block.  The launch is cooperative and therefore not meant for stream capture.  All calls
+ * on one device share the array: calls that overlap on one device (two streams, two threads) race, and nothing detects it. */
 int32_t hykPotrfpStaticMaxN(void);
 int hykPotrfpStatic(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, int32_t N, int32_t Gtype, void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, int32_t* rankOut);
 

@@ -308,3 +308,61 @@ def test_jacobi_tail_rule(hm):
     assert top(nrm, K, 0.0) == K
     sv = np.linalg.svd(B, compute_uv=False)
     assert np.allclose(np.sort(sv[:K]), np.sort(nrm[:K]), rtol=1e-12) and sv[K] <= nrm[:K].min() / 32
+
+
+def test_stop_rules_on_a_cluster_straddling_k(hm):
+    """The loop of hyacinXGevd (host/tail.cpp) on the host, with a plain cyclic one-sided Jacobi in numpy in place of the
+    kernels and the stop rules of host/jacobi_stop.hpp as compiled: a factor whose values 10 .. 14 are within 1e-3 of
+    each other while K = 12 values are handed out, so that kept and discarded columns stay coupled long after the kept
+    values have stopped moving.  Whatever sweep the rules end on, what is handed out must keep the library's promise: values
+    within 10 eps of the largest, vectors orthonormal to sqrt(eps), residual of the basis within (10 eps)^2 |R|^2 of the
+    optimal one.  (The orthogonality gate is the numpy twin of hykMaxCosine on the K largest columns.)"""
+    rng = np.random.default_rng(17)
+    n, r, K, eps = 48, 32, 12, 1e-8
+    sv = np.concatenate([2.0 ** -np.arange(10.0), 1e-3 * (1 + 1e-3 * np.array([2.0, 1.0, 0.0, -1.0, -2.0])), 1e-5 * 2.0 ** -np.arange(17.0)])
+    U, _ = np.linalg.qr(rng.standard_normal((n, r))); W, _ = np.linalg.qr(rng.standard_normal((r, r)))
+    R = (U * sv) @ W.T                                          # n x r, singular values sv
+    # columns graded as after a pivoted Cholesky: B = Q-less factor of R^T R with column pivoting stands in for the factor
+    _, T, piv = __import__("scipy.linalg", fromlist=["qr"]).qr(R, mode="economic", pivoting=True)
+    B = T.T.copy()                                              # r x r: column j = row j of the triangular factor; B^T B ~ P^T R^T R P
+    tol = max(2.220446049250313e-16 * np.sqrt(r), eps / 16)
+
+    def arr(v):
+        return np.ascontiguousarray(v, dtype=np.float64)
+
+    before = np.linalg.norm(B, axis=0)
+    last = 0.0
+    for sweep in range(60):
+        head = hm.hm_jacobi_head(_p(arr(before)), r, K)
+        rotations, worst = 0, 0.0
+        for p in range(r - 1):
+            for q in range(p + 1, r):
+                a, b, g = B[:, p] @ B[:, p], B[:, q] @ B[:, q], B[:, p] @ B[:, q]
+                if a * b > 0 and (p < head or q < head):
+                    worst = max(worst, g * g / (a * b))
+                if g * g > tol * tol * a * b and g != 0.0:
+                    zeta = (b - a) / (2 * g); t = np.sign(zeta) / (abs(zeta) + np.hypot(1.0, zeta)) if zeta != 0 else 1.0
+                    c = 1 / np.hypot(1.0, t); s = c * t
+                    B[:, p], B[:, q] = c * B[:, p] - s * B[:, q], s * B[:, p] + c * B[:, q]
+                    rotations += 1
+        after = np.linalg.norm(B, axis=0)
+        if hm.hm_jacobi_done(rotations, worst, last, tol):
+            break
+        if hm.hm_jacobi_settled(_p(arr(before)), _p(arr(after)), r, K, eps):
+            top = np.argsort(-after)[:K]
+            Vn = B[:, top] / after[top]
+            defect = np.abs(Vn.T @ Vn - np.eye(K)).max()
+            if defect <= np.sqrt(eps):
+                break
+        last, before = worst, after
+    else:
+        raise AssertionError("the rules never ended the sweeps")
+    order = np.argsort(-after)[:K]
+    S, V = after[order], B[:, order] / after[order]
+    assert np.abs(S - sv[:K]).max() <= 10 * eps * sv[0]
+    assert np.abs(V.T @ V - np.eye(K)).max() <= np.sqrt(eps)
+    F = T.T                                                     # the factor the sweeps started from; the rotations act on its columns from the right
+    resid2 = (F ** 2).sum() - ((V.T @ F) ** 2).sum()            # |F^T - F^T V V^T|_F^2 for orthonormal V: what the projection leaves
+    excess = resid2 - (sv[K:] ** 2).sum()
+    print("sweeps", sweep + 1, "excess residual", excess, "of", (sv ** 2).sum())
+    assert excess <= (10 * eps) ** 2 * (sv ** 2).sum()

@@ -52,6 +52,27 @@ def test_potrfp_static_matches_workspace_version(gtype):
         assert np.array_equal(got[2], want[2])
 
 
+def test_potrfp_static_allocates_no_device_memory():
+    """After a warm-up call (symbol lookup, kernel attribute), a hykPotrfpStatic call leaves the amount of free device memory
+    exactly where it was, while the workspace version's caller had to allocate."""
+    import torch
+    import hyacinth_amd as ha
+    from gpu_util import dev, zeros, ptr, stream, sync
+    L = ha.lib()
+    rng = np.random.default_rng(905)
+    N, K, gtype = 600, 600, 6
+    raw = spd(rng, N, 60, 0, True)
+    Rt, jp, rk = zeros(N * N * raw.shape[2] * 8), zeros(N * 4), zeros(4)
+    dG = [dev(raw) for _ in range(3)]                          # every buffer exists before the measurement starts
+    assert L.hykPotrfpStatic(stream(), 256, 1e-9, K, N, gtype, ptr(dG[0]), N, ptr(Rt), N, ptr(jp), ptr(rk)) == 0
+    sync()
+    before = torch.cuda.mem_get_info()[0]
+    for g in dG[1:]:
+        assert L.hykPotrfpStatic(stream(), 256, 1e-9, K, N, gtype, ptr(g), N, ptr(Rt), N, ptr(jp), ptr(rk)) == 0
+    sync()
+    assert torch.cuda.mem_get_info()[0] == before
+
+
 def test_potrfp_static_rejects_oversize():
     import hyacinth_amd as ha
     from gpu_util import zeros, ptr, stream
