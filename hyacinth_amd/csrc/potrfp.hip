@@ -52,8 +52,15 @@ constexpr int MAX_WORKGROUPS = 256;
 /* hykPotrfpSetPlainLaunch: the kernels here are launched cooperatively (the runtime then guarantees that all workgroups are
  * resident, which their waits for each other rely on).  With this set, a grid that the occupancy query says fits the device
  * is started with a plain launch instead: on an otherwise idle device that comes to the same, and a grid that does not
- * become resident after all fails safe (every wait is bounded and gives the run up with rank -1). */
+ * become resident after all fails safe (every wait is bounded and gives the run up with rank -1).  The same plain launch
+ * is what a call falls back to when the runtime refuses the cooperative one (seen when a second process on the device has
+ * made cooperative launches of its own): the refusal is cleared from the runtime's error state and not reported. */
 std::atomic<int> g_plainLaunch{ 0 };
+
+bool fits_device(int grid, int perCu) {
+  int dev = 0, units = 0;
+  return hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && (int64_t)grid <= (int64_t)units * perCu;
+}
 
 constexpr int SPIN_LIMIT = 1 << 22;   /* polls of one record before the run is given up (seconds; a healthy wait is microseconds) */
 
@@ -282,14 +289,14 @@ template <bool DD, bool CPLX> int launch(hipStream_t stream, PotrfArgs& args, in
   int perCu = 0; if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, potrfp_kernel<DD, CPLX>, P_THREADS, 0) != hipSuccess || perCu < 1) { return -3; }
   int grid = cus < MAX_WORKGROUPS ? cus : MAX_WORKGROUPS; const int want = (args.N + P_WAVES - 1) / P_WAVES; if (grid > want) { grid = want; } if (grid < 1) { grid = 1; }
   if ((int64_t)grid * P_WAVES * 64 < args.N) { return -1; }   /* a wavefront tracks at most 64 columns */
-  if (g_plainLaunch.load(std::memory_order_relaxed)) {
-    int dev = 0, units = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) { return -3; }
-    if ((int64_t)grid <= (int64_t)units * perCu) { potrfp_kernel<DD, CPLX><<<grid, P_THREADS, 0, stream>>>(args); return hipGetLastError() == hipSuccess ? 0 : -3; }
+  const bool fits = fits_device(grid, perCu);
+  if (!(g_plainLaunch.load(std::memory_order_relaxed) && fits)) {
+    void* params[] = { &args };
+    if (hipLaunchCooperativeKernel(reinterpret_cast<const void*>(&potrfp_kernel<DD, CPLX>), dim3(grid), dim3(P_THREADS), params, 0, stream) == hipSuccess) { return 0; }
+    (void)hipGetLastError();   /* refused: not to be found by the next call that asks for the last error */
+    if (!fits) { return -3; }
   }
-  void* params[] = { &args };
-  hipError_t e = hipLaunchCooperativeKernel(reinterpret_cast<const void*>(&potrfp_kernel<DD, CPLX>), dim3(grid), dim3(P_THREADS), params, 0, stream);
-  return e == hipSuccess ? 0 : -3;
+  potrfp_kernel<DD, CPLX><<<grid, P_THREADS, 0, stream>>>(args); return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
 
@@ -795,13 +802,14 @@ template <bool DD, bool CPLX> int launch(hipStream_t stream, Args& args, int cus
   if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes) != hipSuccess) { return -3; }
   int perCu = 0; if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&perCu, potrfp_blocked_kernel<DD, CPLX>, THREADS, ldsBytes) != hipSuccess || perCu < 1) { return -3; }
   int grid = cus < 256 ? cus : 256; if (grid < args.agents) { return -1; }
-  if (g_plainLaunch.load(std::memory_order_relaxed)) {   /* hykPotrfpSetPlainLaunch: see there */
-    int dev = 0, units = 0;
-    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&units, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) { return -3; }
-    if ((int64_t)grid <= (int64_t)units * perCu) { potrfp_blocked_kernel<DD, CPLX><<<grid, THREADS, ldsBytes, stream>>>(args); return hipGetLastError() == hipSuccess ? 0 : -3; }
+  const bool fits = fits_device(grid, perCu);
+  if (!(g_plainLaunch.load(std::memory_order_relaxed) && fits)) {   /* hykPotrfpSetPlainLaunch: see there */
+    void* params[] = { &args };
+    if (hipLaunchCooperativeKernel(fn, dim3(grid), dim3(THREADS), params, (unsigned)ldsBytes, stream) == hipSuccess) { return 0; }
+    (void)hipGetLastError();
+    if (!fits) { return -3; }
   }
-  void* params[] = { &args };
-  return hipLaunchCooperativeKernel(fn, dim3(grid), dim3(THREADS), params, (unsigned)ldsBytes, stream) == hipSuccess ? 0 : -3;
+  potrfp_blocked_kernel<DD, CPLX><<<grid, THREADS, ldsBytes, stream>>>(args); return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
 __global__ void clear_kernel(uint64_t* p, int words) { for (int i = threadIdx.x; i < words; i += blockDim.x) { p[i] = 0ull; } }

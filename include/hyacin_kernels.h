@@ -101,7 +101,9 @@ int hykPotrfpLeftLooking(hipStream_t stream, int32_t computeUnits, double eps, i
  * profilers whose kernel tracing does not get along with cooperative launches (rocprofv3 --kernel-trace: the process then
  * ends with a segmentation fault in the runtime's exit handler, after the trace has been written); hyacinCreate switches
  * it on when the environment variable HYACIN_PLAIN_LAUNCH is 1 / true.  The bounded waits inside the kernels make a grid
- * that is not resident after all end with rank -1 (status -5) instead of hanging. */
+ * that is not resident after all end with rank -1 (status -5) instead of hanging.  A call whose cooperative launch the
+ * runtime refuses (a second process on the device that has made cooperative launches of its own) takes the same plain
+ * launch, whatever this setting. */
 int hykPotrfpSetPlainLaunch(int32_t enable);
 
 /* hykPotrfp for callers that may not call hipMalloc (serving loops, harnesses that forbid it).  No counterpart in the

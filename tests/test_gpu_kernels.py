@@ -185,6 +185,21 @@ def test_gram_limbs_bit_exact(gl, oracle, N, K, rows, cplx, order):
     assert np.array_equal(got2, want2)
 
 
+@pytest.mark.parametrize("kind,cplx,order", [("crt", 0, 3), ("crt", 1, 4), ("crt", 1, 22), ("limbs", 0, 2), ("limbs", 1, 3), ("limbs", 1, 9)])
+def test_gram_split_along_k(gl, oracle, kind, cplx, order):
+    """A K long enough for the few tiles of a small N to be cut along K: the parts of a tile add into the same sums.  Complex
+    CRT order 22 has moduli whose three products share planes, complex limb order 9 does not fit one launch's tables."""
+    rng = np.random.default_rng(37)
+    N, K, rows, orderC = 70, 16384, 16300, 3
+    panels = random_panels(rng, oracle.n_panels(kind, order, cplx), N, K, rows, -125, 126)
+    want = oracle.i8herk(kind, cplx, N, order, panels, 0, orderC)
+    print("gram split along K", kind, cplx, order, flush=True)
+    got = gl.gram(kind, cplx, N, order, panels, orderC)
+    assert np.array_equal(got, want)
+    want2 = oracle.i8herk(kind, cplx, N, order, panels[:, :, :4096], 1, orderC, Cin=want)
+    assert np.array_equal(gl.gram(kind, cplx, N, order, panels[:, :, :4096], orderC, beta=1, Cin=got), want2)
+
+
 def test_gram_extreme_values_and_long_k(gl, oracle):
     """All -128 digits over a K that needs several int32-safe splits; all-(-125) residues over K = 131072 rows are covered by the bound."""
     N, K = 20, 16384 * 3

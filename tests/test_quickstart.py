@@ -55,9 +55,15 @@ def test_quickstart_runs(tmp_path):
     """rank 2 (the matrix is a sum of two rank-one terms), relative projection error at the level of eps, an orthonormal
     basis, and the two singular values numpy finds for the same matrix."""
     exe = build_quickstart(tmp_path)
+    # this process first makes a cooperative launch of its own (a pivoted Cholesky): the quick start then runs as a second
+    # process on the device, where the runtime refuses cooperative launches and the library has to start its kernel plainly
+    import hyacinth_amd as ha
+    from test_zz_no_alloc import spd, run
+    assert run(ha.lib(), False, spd(np.random.default_rng(5), 200, 30, 0, False), 200, 200, 0, 1e-9)[0] > 0
     r = subprocess.run([exe], capture_output=True, text=True, timeout=120)
     assert r.returncode == 0, r.stdout + r.stderr
-    print(r.stdout, flush=True)
+    print(r.stdout, r.stderr, flush=True)
+    assert "failed" not in r.stderr
     m = re.search(r"rank = (\d+), relative projection error = (\S+), orthonormality defect = (\S+), S0 = (\S+), S1 = (\S+), S2 = (\S+)", r.stdout)
     assert m, r.stdout
     i, j = np.arange(512)[:, None], np.arange(128)[None, :]
