@@ -68,21 +68,60 @@ inline int jacobi_head(const std::vector<double>& norm, int kept) {
  * and their vectors are handed out.  G = R^H R is the sum over the rows of R of their outer products, so leaving the rows
  * from t on out of the SVD takes a positive semidefinite matrix of trace tau_t = sum_{j >= t} |row j|^2 off G: no eigenvalue
  * moves up and none moves down by more than tau_t, hence 0 <= sigma_i - sigma'_i <= tau_t / (sigma_i + sigma'_i) <=
- * tau_t / (2 sigma'_i) for the values sigma' of the truncated factor.  With tau_t <= eps sigma'_1 sigma'_K every value that is
- * handed out is within eps sigma_1 / 2 of the true one, and the residual |A - A V V^H|^2 grows by at most tau_t.
+ * tau_t / (2 sigma'_i) for the values sigma' of the truncated factor.  With tau_t <= 4 eps sigma'_1 sigma'_K every value that
+ * is handed out is within 2 eps sigma_1 of the true one (a fifth of the 10 eps sigma_1 the values are held to; the bound is
+ * attained only when all the weight left out lies along the K-th vector), and the residual |A - A V V^H|^2, which depends on
+ * the span of V alone, grows by at most tau_t (V spans the leading subspace of G - E with E positive semidefinite of trace
+ * tau_t: tr((I - P) G) = tr((I - P)(G - E)) + tr((I - P) E) <= the optimum for G + tau_t).
  * jacobi_columns_needed guesses t from the column norms (largest norm for sigma_1, K-th largest norm for sigma_K, a quarter of
  * the bound for the guess: the norms of the columns are not the singular values); jacobi_truncation_holds is the test with
  * the values the sweeps have found, and the caller goes on with all columns when it fails.  A noise floor under the wanted
- * values, which costs a cyclic Jacobi method the most sweeps, is what this leaves out. */
+ * values, which costs a cyclic Jacobi method the most sweeps, and the graded columns beneath it are what this leaves out:
+ * the work of a sweep goes with the square of the columns it takes. */
+constexpr double kTruncationBudget = 4.;   /* tau_t <= kTruncationBudget eps sigma'_1 sigma'_K */
 inline int jacobi_columns_needed(const std::vector<double>& norm, int K, double eps) {
   const int r = (int)norm.size(); if (K < 1 || K >= r) { return r; }
   std::vector<double> v(norm); std::nth_element(v.begin(), v.begin() + (K - 1), v.end(), std::greater<double>());
-  const double nuK = v[(size_t)(K - 1)], nu1 = *std::max_element(norm.begin(), norm.end()), bound = 0.25 * eps * nu1 * nuK;
+  const double nuK = v[(size_t)(K - 1)], nu1 = *std::max_element(norm.begin(), norm.end()), bound = 0.25 * kTruncationBudget * eps * nu1 * nuK;
   double sum = 0.; int t = r;
   while (t > K && sum + norm[(size_t)(t - 1)] * norm[(size_t)(t - 1)] <= bound) { sum += norm[(size_t)(t - 1)] * norm[(size_t)(t - 1)]; --t; }
   return t;
 }
-inline bool jacobi_truncation_holds(double dropped2, double sigma1, double sigmaK, double eps) { return dropped2 <= eps * sigma1 * sigmaK; }
+inline bool jacobi_truncation_holds(double dropped2, double sigma1, double sigmaK, double eps) { return dropped2 <= kTruncationBudget * eps * sigma1 * sigmaK; }
+
+/* The same cut with the sharper of the two bounds.  What moves a singular value is the largest eigenvalue of what is taken off
+ * G, not its trace (Weyl): 0 <= sigma_i^2 - sigma'_i^2 <= |E|_2, and |E|_2 = |R_d|_2^2 is the largest eigenvalue of the Gram
+ * matrix M = B_d^H B_d of the columns left out.  For the rows of a noise floor (hundreds of rows of about equal norm pointing
+ * in unrelated directions) that is a small fraction of the trace: d rows of squared norm w weigh d w, their largest
+ * eigenvalue is about w (1 + sqrt(d / N))^2.  M is small (d x d) and cheap to form; its largest eigenvalue is bounded from
+ * above by min(largest absolute row sum, Frobenius norm, trace), all three taken on the trailing block [t, r) for every t
+ * in one pass from the back.  The residual |A - A V V^H|^2 still grows by up to the trace, so the trace must stay either
+ * within the same budget as |E|_2 (the rule above, which needs nothing else) or within 1 / 64 of the squared residual itself
+ * (the squared values that are not handed out): a residual 0.8 % larger.
+ *
+ * absGram: |M[i][j]| for the columns c0 .. r - 1 of B, d x d with d = r - c0, column-major; valueBudget bounds |E|_2,
+ * residualBudget the trace where it exceeds valueBudget.  Returns the smallest t >= max(c0, K) whose trailing block passes
+ * (r when none does); trace / spectral: the two figures of that block, for the test after the sweeps. */
+struct JacobiCut { int cols; double trace, spectral; };
+inline JacobiCut jacobi_columns_needed_spectral(const std::vector<double>& absGram, int r, int c0, int K, double valueBudget, double residualBudget) {
+  JacobiCut cut{ r, 0., 0. }; const int d = r - c0; if (d <= 0 || absGram.size() < (size_t)d * (size_t)d) { return cut; }
+  std::vector<double> rowSum((size_t)d, 0.); double frob2 = 0., trace = 0.;
+  for (int t = r - 1; t >= std::max(c0, K); --t) {
+    const int i = t - c0; double own = 0.;
+    for (int j = i; j < d; ++j) { const double a = absGram[(size_t)i + (size_t)j * (size_t)d]; own += a; if (j > i) { rowSum[(size_t)j] += a; frob2 += 2. * a * a; } else { frob2 += a * a; trace += a; } }
+    rowSum[(size_t)i] = own;
+    double gersh = 0.; for (int j = i; j < d; ++j) { gersh = std::max(gersh, rowSum[(size_t)j]); }
+    const double spectral = std::min(std::min(gersh, std::sqrt(frob2)), trace);
+    if (!(spectral <= valueBudget && (trace <= valueBudget || trace <= residualBudget))) { break; }
+    cut.cols = t; cut.trace = trace; cut.spectral = spectral;
+  }
+  return cut;
+}
+/* the test with the values found: sigma1, sigmaK as above, outside2 = the sum of the squared values found that are not handed out */
+inline bool jacobi_truncation_holds_spectral(double trace, double spectral, double sigma1, double sigmaK, double outside2, double eps) {
+  const double budget = kTruncationBudget * eps * sigma1 * sigmaK;
+  return spectral <= budget && (trace <= budget || trace <= outside2 / 64.);
+}
 
 /* Columns a sweep may leave alone.  Let nu be the K-th largest column norm and b = max(nu^2, eps^2 sum of all squared norms).
  * The tail is the longest index range [top, r) whose squared norms sum to at most b / 1024; it is used only when it holds

@@ -99,6 +99,11 @@ int hm_jacobi_tail_start(const double* norm, int r, int K, double eps) { return 
 int hm_jacobi_settled(const double* before, const double* after, int r, int kept, double eps) { return hyh::jacobi_output_settled(std::vector<double>(before, before + r), std::vector<double>(after, after + r), kept, eps) ? 1 : 0; }
 int hm_jacobi_columns_needed(const double* norm, int r, int K, double eps) { return hyh::jacobi_columns_needed(std::vector<double>(norm, norm + r), K, eps); }
 int hm_jacobi_truncation_holds(double dropped2, double sigma1, double sigmaK, double eps) { return hyh::jacobi_truncation_holds(dropped2, sigma1, sigmaK, eps) ? 1 : 0; }
+int hm_jacobi_columns_needed_spectral(const double* absGram, int r, int c0, int K, double valueBudget, double residualBudget, double* traceOut, double* spectralOut) {
+  const size_t d = (size_t)(r - c0); const hyh::JacobiCut c = hyh::jacobi_columns_needed_spectral(std::vector<double>(absGram, absGram + d * d), r, c0, K, valueBudget, residualBudget);
+  *traceOut = c.trace; *spectralOut = c.spectral; return c.cols;
+}
+int hm_jacobi_truncation_holds_spectral(double trace, double spectral, double sigma1, double sigmaK, double outside2, double eps) { return hyh::jacobi_truncation_holds_spectral(trace, spectral, sigma1, sigmaK, outside2, eps) ? 1 : 0; }
 int hm_jacobi_head(const double* norm, int r, int kept) { return hyh::jacobi_head(std::vector<double>(norm, norm + r), kept); }
 
 }

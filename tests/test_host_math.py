@@ -255,7 +255,8 @@ def test_jacobi_head(hm):
 
 def test_jacobi_columns_needed(hm):
     """Which prefix of the factor's columns the SVD works on (host/jacobi_stop.hpp): the trailing columns whose squared norms
-    sum to at most eps nu_1 nu_K / 4 are left out, never fewer than K columns kept.  The bound behind it, checked on an
+    sum to at most eps nu_1 nu_K (a quarter of the 4 eps sigma_1 sigma_K the values found must confirm) are left out, never fewer
+    than K columns kept.  The bound behind it, checked on an
     explicit matrix: dropping rows of R of squared Frobenius norm tau moves every singular value down, by at most
     tau / (2 sigma') (sigma' the value without them)."""
     rng = np.random.default_rng(11)
@@ -263,19 +264,61 @@ def test_jacobi_columns_needed(hm):
         a = np.ascontiguousarray(norm, dtype=np.float64)
         return hm.hm_jacobi_columns_needed(_p(a), len(a), K, eps)
     floor = np.concatenate([10.0 ** -np.arange(8.0), np.full(100, 1e-9)])        # 8 graded columns over a floor of 100
-    # K = 4: nu_1 = 1, nu_4 = 1e-3; eps = 1e-6 allows 2.5e-10: all of the floor (1e-16) and the columns below it
+    # K = 4: nu_1 = 1, nu_4 = 1e-3; eps = 1e-6 allows 1e-9: all of the floor (1e-16) and the columns below it
     t = need(floor, 4, 1e-6)
-    assert 4 <= t <= 8 and (floor[t:] ** 2).sum() <= 0.25e-6 * 1.0 * 1e-3 < (floor[t - 1:] ** 2).sum()
-    assert need(floor, 4, 1e-16) == 108                                          # nothing is small enough: 2.5e-20 < 1e-18
-    assert need(floor, 4, 4.1e-12) == 8                                          # exactly the floor (100 x 1e-18 = 1e-16 <= 1.025e-15 ... and 1e-14 more is too much)
+    assert 4 <= t <= 8 and (floor[t:] ** 2).sum() <= 1e-6 * 1.0 * 1e-3 < (floor[t - 1:] ** 2).sum()
+    assert need(floor, 4, 1e-16) == 108                                          # nothing is small enough: 1e-19 < 1e-18
+    assert need(floor, 4, 1.02e-12) == 8                                         # exactly the floor (100 x 1e-18 = 1e-16 <= 1.02e-15 ... and 1e-14 more is too much)
     assert need(floor, 108, 1.0) == 108 and need(floor, 0, 1.0) == 108           # every column wanted / no K: all
     assert need(np.full(20, 1.0), 5, 1.0) >= 5                                   # never fewer than K
     # the perturbation bound on an explicit factor: rows of R in pivot order, graded, the last 30 small
     R = rng.standard_normal((40, 60)) * np.concatenate([2.0 ** -np.arange(10.0), np.full(30, 1e-6)])[:, None]
     full = np.linalg.svd(R, compute_uv=False); cut = np.linalg.svd(R[:10], compute_uv=False); tau = (R[10:] ** 2).sum()
     assert np.all(full[:10] >= cut * (1 - 1e-15)) and np.all(full[:10] - cut <= tau / (2 * cut) * (1 + 1e-9))
-    assert hm.hm_jacobi_truncation_holds(tau, cut[0], cut[9], tau / (cut[0] * cut[9]) * 1.01) == 1
-    assert hm.hm_jacobi_truncation_holds(tau, cut[0], cut[9], tau / (cut[0] * cut[9]) * 0.99) == 0
+    assert hm.hm_jacobi_truncation_holds(tau, cut[0], cut[9], tau / (4 * cut[0] * cut[9]) * 1.01) == 1
+    assert hm.hm_jacobi_truncation_holds(tau, cut[0], cut[9], tau / (4 * cut[0] * cut[9]) * 0.99) == 0
+
+
+def test_jacobi_columns_needed_spectral(hm):
+    """The sharper cut (host/jacobi_stop.hpp): the largest eigenvalue of the Gram matrix of the columns left out is bounded by
+    min(largest absolute row sum, Frobenius norm, trace) of every trailing block; a floor of many unrelated rows passes with
+    a trace far above the budget of the values, as long as the trace stays within the budget of the residual."""
+    rng = np.random.default_rng(12)
+    hm.hm_jacobi_columns_needed_spectral.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_double, C.c_double, C.c_void_p, C.c_void_p]
+    hm.hm_jacobi_columns_needed_spectral.restype = C.c_int
+    hm.hm_jacobi_truncation_holds_spectral.argtypes = [C.c_double] * 6
+    hm.hm_jacobi_truncation_holds_spectral.restype = C.c_int
+    N, r, K, c0 = 400, 120, 20, 30
+    scale = np.concatenate([2.0 ** -np.arange(40.0), np.full(80, 2.0 ** -40)])            # 40 graded rows over a floor of 80
+    R = rng.standard_normal((r, N)) / np.sqrt(N) * scale[:, None]
+    M = np.abs(R[c0:] @ R[c0:].T)
+    def cut(value, residual):
+        a = np.asfortranarray(M); tr, sp = C.c_double(), C.c_double()
+        t = hm.hm_jacobi_columns_needed_spectral(a.ctypes.data_as(C.c_void_p), r, c0, K, value, residual, C.byref(tr), C.byref(sp))
+        return t, tr.value, sp.value
+    def bounds(t):
+        B = M[t - c0:, t - c0:]
+        return min(B.sum(1).max(), np.linalg.norm(B), np.trace(B)), np.trace(B), np.linalg.eigvalsh(R[t:] @ R[t:].T)[-1]
+    floor_trace, floor_top = bounds(40)[1], bounds(40)[2]
+    assert floor_top < floor_trace / 10                                                   # 80 unrelated rows: the trace overstates what moves a value
+    # values may move by twice the floor's largest eigenvalue, the residual allows all of the floor: the cut takes the whole floor
+    # (and what graded rows fit), where the trace rule alone would stop inside it
+    t, tr, sp = cut(4 * floor_top, 2 * floor_trace)
+    assert c0 <= t <= 40 and tr > 4 * floor_top
+    b, trace, top = bounds(t)
+    assert np.isclose(sp, b, rtol=1e-12) and np.isclose(tr, trace, rtol=1e-12) and top <= sp <= 4 * floor_top and tr <= 2 * floor_trace
+    assert t == c0 or bounds(t - 1)[0] > 4 * floor_top or bounds(t - 1)[1] > 2 * floor_trace          # one more column would break a budget
+    # a residual budget below the budget of the values changes nothing: then the trace is held to the budget of the values
+    t2, tr2, _ = cut(4 * floor_top, 0.0)
+    assert t2 > t and tr2 <= 4 * floor_top and (bounds(t2 - 1)[1] > 4 * floor_top)
+    # nothing passes / everything in the window passes; never fewer than K columns kept
+    assert cut(0.0, 1.0)[0] == r and cut(1e30, 1e30)[0] == c0
+    a = np.asfortranarray(M); tr, sp = C.c_double(), C.c_double()
+    assert hm.hm_jacobi_columns_needed_spectral(a.ctypes.data_as(C.c_void_p), r, c0, 50, 1e30, 1e30, C.byref(tr), C.byref(sp)) == 50
+    # the test after the sweeps: eigenvalue bound within 4 eps sigma_1 sigma_K, and the trace within that or within 1 / 64 of what is outside
+    holds = hm.hm_jacobi_truncation_holds_spectral
+    assert holds(1e-3, 3.9e-6, 1.0, 1.0, 0.065, 1e-6) == 1 and holds(1e-3, 4.1e-6, 1.0, 1.0, 0.065, 1e-6) == 0
+    assert holds(1e-3, 3.9e-6, 1.0, 1.0, 0.063, 1e-6) == 0 and holds(3.9e-6, 3.9e-6, 1.0, 1.0, 0.0, 1e-6) == 1
 
 
 def test_jacobi_tail_rule(hm):
