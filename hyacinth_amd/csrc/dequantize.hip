@@ -54,9 +54,13 @@ __global__ __launch_bounds__(256) void dequantize_kernel(int32_t N, int32_t L, c
   using T = std::conditional_t<KIND == 0, float, double>;
   constexpr int W = (KIND == 2 ? 2 : 1) * (CPLX ? 2 : 1);
   using E = Elem<T, W>;
-  if (blockIdx.x > blockIdx.y) { return; }   /* tile row > tile column: below the diagonal */
+  /* workgroup b takes tile (row ty <= column tx) with b = ty + tx (tx + 1) / 2: only tiles on or above the diagonal are launched */
+  int tx = (int)((sqrtf(8.f * (float)blockIdx.x + 1.f) - 1.f) * 0.5f);
+  while ((uint32_t)(tx + 1) * (uint32_t)(tx + 2) / 2u <= blockIdx.x) { ++tx; }
+  while ((uint32_t)tx * (uint32_t)(tx + 1) / 2u > blockIdx.x) { --tx; }
+  const int ty = (int)(blockIdx.x - (uint32_t)tx * (uint32_t)(tx + 1) / 2u);
   __shared__ E tile[DQ_TILE][DQ_TILE + 1];   /* [x][y], one element of padding per row */
-  const int y0 = (int)blockIdx.x * DQ_TILE, x0 = (int)blockIdx.y * DQ_TILE, ti = threadIdx.x % DQ_TILE, tj = threadIdx.x / DQ_TILE;
+  const int y0 = ty * DQ_TILE, x0 = tx * DQ_TILE, ti = threadIdx.x % DQ_TILE, tj = threadIdx.x / DQ_TILE;
   E* G = reinterpret_cast<E*>(Gv);
   {
     const int y = y0 + ti; const int32_t ey = y < N ? vexp[y] : 0;
@@ -102,7 +106,7 @@ __global__ __launch_bounds__(256) void dequantize_kernel(int32_t N, int32_t L, c
 extern "C" int hykDequantize(hipStream_t stream, int32_t N, int32_t orderC, const uint64_t* C, const int32_t* vexp, int32_t Gtype, void* G, int64_t ldg) {
   if (N <= 0) { return 0; }
   if (orderC < 1 || orderC > 3 || N > 65535 || ldg < N) { return -1; }
-  const int64_t strideC = ((int64_t)N * N + N) / 2; const uint32_t tiles = (uint32_t)((N + DQ_TILE - 1) / DQ_TILE); dim3 grid(tiles, tiles);
+  const int64_t strideC = ((int64_t)N * N + N) / 2; const uint32_t tiles = (uint32_t)((N + DQ_TILE - 1) / DQ_TILE); dim3 grid(tiles * (tiles + 1) / 2);
   switch (Gtype) {
     case HYK_F32: dequantize_kernel<0, 0><<<grid, 256, 0, stream>>>(N, orderC, C, strideC, vexp, G, ldg); break;
     case HYK_F32C: dequantize_kernel<0, 1><<<grid, 256, 0, stream>>>(N, orderC, C, strideC, vexp, G, ldg); break;
