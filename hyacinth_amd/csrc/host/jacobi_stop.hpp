@@ -73,16 +73,19 @@ inline int jacobi_head(const std::vector<double>& norm, int kept) {
  * attained only when all the weight left out lies along the K-th vector), and the residual |A - A V V^H|^2, which depends on
  * the span of V alone, grows by at most tau_t (V spans the leading subspace of G - E with E positive semidefinite of trace
  * tau_t: tr((I - P) G) = tr((I - P)(G - E)) + tr((I - P) E) <= the optimum for G + tau_t).
- * jacobi_columns_needed guesses t from the column norms (largest norm for sigma_1, K-th largest norm for sigma_K, a quarter of
- * the bound for the guess: the norms of the columns are not the singular values); jacobi_truncation_holds is the test with
- * the values the sweeps have found, and the caller goes on with all columns when it fails.  A noise floor under the wanted
+ * jacobi_columns_needed guesses t from the column norms (largest norm for sigma_1, K-th largest norm for sigma_K, a quarter
+ * of the bound for the guess: the norms of the columns are not the singular values; the K-th largest norm was 3.8 times the
+ * K-th value on a dense spectrum with neighbours 1.8 % apart, which the quarter just covers; half the share takes twice the
+ * rows of a broad floor back in, whose sweeps cost far more than an occasional second cut); jacobi_truncation_holds is the test with the values the sweeps
+ * have found, and the caller takes columns back in when it fails.  A noise floor under the wanted
  * values, which costs a cyclic Jacobi method the most sweeps, and the graded columns beneath it are what this leaves out:
  * the work of a sweep goes with the square of the columns it takes. */
 constexpr double kTruncationBudget = 4.;   /* tau_t <= kTruncationBudget eps sigma'_1 sigma'_K */
+constexpr double kTruncationGuess = 0.25;  /* the share of it that the guess from the column norms may use */
 inline int jacobi_columns_needed(const std::vector<double>& norm, int K, double eps) {
   const int r = (int)norm.size(); if (K < 1 || K >= r) { return r; }
   std::vector<double> v(norm); std::nth_element(v.begin(), v.begin() + (K - 1), v.end(), std::greater<double>());
-  const double nuK = v[(size_t)(K - 1)], nu1 = *std::max_element(norm.begin(), norm.end()), bound = 0.25 * kTruncationBudget * eps * nu1 * nuK;
+  const double nuK = v[(size_t)(K - 1)], nu1 = *std::max_element(norm.begin(), norm.end()), bound = kTruncationGuess * kTruncationBudget * eps * nu1 * nuK;
   double sum = 0.; int t = r;
   while (t > K && sum + norm[(size_t)(t - 1)] * norm[(size_t)(t - 1)] <= bound) { sum += norm[(size_t)(t - 1)] * norm[(size_t)(t - 1)]; --t; }
   return t;

@@ -127,41 +127,47 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
      * jacobi_columns_needed picks the prefix from the column norms, and what the sweeps then find must confirm it
      * (jacobi_truncation_holds with the values themselves), or the sweeps go on with all columns. */
     int32_t cols = rank; double dropped2 = 0., droppedSpectral = 0.;
+    /* The cut for given budgets: the longest tail [t, rank), t >= atLeast, that passes the trace rule or the sharper rule
+     * (jacobi_columns_needed_spectral: what moves a value is the largest eigenvalue of the Gram matrix of the columns left
+     * out, which for the rows of a noise floor is a small part of their trace).  The Gram matrix is formed once, for the
+     * window [c0, rank) of columns that can pass at all under the first (largest) budgets: squared norm (a diagonal entry,
+     * below the largest eigenvalue) within the budget of the values, trace within the budget of the residual. */
+    std::vector<double> allNorms, absGram; int32_t c0 = rank;
+    auto choose_cut = [&](double valueBudget, double residualBudget, int32_t atLeast) {
+      int32_t t = rank; double sum = 0.;   /* trace rule */
+      while (t > atLeast && sum + allNorms[(size_t)(t - 1)] * allNorms[(size_t)(t - 1)] <= valueBudget) { sum += allNorms[(size_t)(t - 1)] * allNorms[(size_t)(t - 1)]; --t; }
+      cols = t; bool sharper = false;
+      if (!absGram.empty() && c0 < cols) {
+        const hyh::JacobiCut cut = hyh::jacobi_columns_needed_spectral(absGram, rank, c0, atLeast, valueBudget / 1.01, residualBudget);   /* 1 %: the products are rounded */
+        if (cut.cols < cols) { cols = cut.cols; droppedSpectral = 1.01 * cut.spectral; sharper = true; }
+      }
+      dropped2 = 0.; for (int32_t j = rank - 1; j >= cols; --j) { dropped2 = std::fma(allNorms[(size_t)j], allNorms[(size_t)j], dropped2); }
+      if (!sharper) { droppedSpectral = dropped2; }   /* the trace bounds the largest eigenvalue */
+      if (handle->logger && cols < rank) { std::fprintf((FILE*)handle->logger, "GESVJ: the last %d of %d columns (squared norms %.2le in all, largest eigenvalue of their Gram matrix at most %.2le) are left out of the sweeps\n", rank - cols, rank, dropped2, droppedSpectral); }
+    };
     if (K < rank && rank > 1) {
-      fetch_norms(before, rank); HYH_CHECK(hipStreamSynchronize(s)); if (!hyh::ok()) { return 0; }
-      cols = hyh::jacobi_columns_needed(before, K, eps);
-      /* The sharper cut (jacobi_columns_needed_spectral): what moves a value is the largest eigenvalue of the Gram matrix of
-       * the columns left out, which for the rows of a noise floor is a small part of their trace.  The window [c0, rank) holds
-       * the columns that can pass at all: squared norm (a diagonal entry, below the largest eigenvalue) within the budget of
-       * the values, trace within the budget of the residual. */
-      bool sharper = false;
-      {
-        std::vector<double> v(before); std::nth_element(v.begin(), v.begin() + (K - 1), v.end(), std::greater<double>());
-        const double nuK = v[(size_t)(K - 1)], nu1 = *std::max_element(before.begin(), before.end()), valueGuess = 0.25 * hyh::kTruncationBudget * eps * nu1 * nuK;
-        double outside = 0.; for (size_t j = (size_t)K; j < v.size(); ++j) { outside = std::fma(v[j], v[j], outside); }   /* the squared norms beyond the K largest */
-        const double residualGuess = outside / 256.;
-        int32_t c0 = rank; double suffix = 0.;
-        while (c0 > K) { const double w = before[(size_t)(c0 - 1)] * before[(size_t)(c0 - 1)]; if (w > valueGuess || suffix + w > std::max(valueGuess, residualGuess)) { break; } suffix += w; --c0; }
-        if (c0 < cols && gram.p) {
-          const int32_t d = rank - c0; const size_t elem = (size_t)(wideB ? 8 : 4) * (1 + Complex);
-          HYH_KERNEL(hykGemm(s, 'C', 'N', d, d, N, 1., Btype, (const char*)B.p + (size_t)c0 * N * elem, N, (const char*)B.p + (size_t)c0 * N * elem, N, 0., gram.p, d));
-          std::vector<char> raw((size_t)d * d * elem); std::vector<double> absGram((size_t)d * d);
-          HYH_CHECK(hipMemcpyAsync(raw.data(), gram.p, raw.size(), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s)); if (!hyh::ok()) { return 0; }
-          for (size_t i = 0; i < absGram.size(); ++i) {
-            double re, im = 0.;
-            if (wideB) { const double* q = reinterpret_cast<const double*>(raw.data()) + i * (1 + Complex); re = q[0]; if (Complex) { im = q[1]; } }
-            else { const float* q = reinterpret_cast<const float*>(raw.data()) + i * (1 + Complex); re = q[0]; if (Complex) { im = q[1]; } }
-            absGram[i] = Complex ? std::hypot(re, im) : std::fabs(re);
-          }
-          const hyh::JacobiCut cut = hyh::jacobi_columns_needed_spectral(absGram, rank, c0, K, valueGuess / 1.01, residualGuess);   /* 1 %: the products are rounded */
-          if (cut.cols < cols) { cols = cut.cols; droppedSpectral = 1.01 * cut.spectral; sharper = true; }
+      fetch_norms(allNorms, rank); HYH_CHECK(hipStreamSynchronize(s)); if (!hyh::ok()) { return 0; }
+      std::vector<double> v(allNorms); std::nth_element(v.begin(), v.begin() + (K - 1), v.end(), std::greater<double>());
+      const double nuK = v[(size_t)(K - 1)], nu1 = *std::max_element(allNorms.begin(), allNorms.end()), valueGuess = hyh::kTruncationGuess * hyh::kTruncationBudget * eps * nu1 * nuK;
+      double outside = 0.; for (size_t j = (size_t)K; j < v.size(); ++j) { outside = std::fma(v[j], v[j], outside); }   /* the squared norms beyond the K largest */
+      const double residualGuess = outside / 256.;
+      { double suffix = 0.; while (c0 > K) { const double w = allNorms[(size_t)(c0 - 1)] * allNorms[(size_t)(c0 - 1)]; if (w > valueGuess || suffix + w > std::max(valueGuess, residualGuess)) { break; } suffix += w; --c0; } }
+      if (c0 < hyh::jacobi_columns_needed(allNorms, K, eps) && gram.p) {   /* the sharper rule can reach further than the trace rule */
+        const int32_t d = rank - c0; const size_t elem = (size_t)(wideB ? 8 : 4) * (1 + Complex);
+        HYH_KERNEL(hykGemm(s, 'C', 'N', d, d, N, 1., Btype, (const char*)B.p + (size_t)c0 * N * elem, N, (const char*)B.p + (size_t)c0 * N * elem, N, 0., gram.p, d));
+        std::vector<char> raw((size_t)d * d * elem); absGram.resize((size_t)d * d);
+        HYH_CHECK(hipMemcpyAsync(raw.data(), gram.p, raw.size(), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s)); if (!hyh::ok()) { return 0; }
+        for (size_t i = 0; i < absGram.size(); ++i) {
+          double re, im = 0.;
+          if (wideB) { const double* q = reinterpret_cast<const double*>(raw.data()) + i * (1 + Complex); re = q[0]; if (Complex) { im = q[1]; } }
+          else { const float* q = reinterpret_cast<const float*>(raw.data()) + i * (1 + Complex); re = q[0]; if (Complex) { im = q[1]; } }
+          absGram[i] = Complex ? std::hypot(re, im) : std::fabs(re);
         }
       }
-      for (int32_t j = rank - 1; j >= cols; --j) { dropped2 = std::fma(before[(size_t)j], before[(size_t)j], dropped2); }
-      if (!sharper) { droppedSpectral = dropped2; }   /* the trace bounds the largest eigenvalue */
-      before.resize((size_t)cols);
-      if (handle->logger && cols < rank) { std::fprintf((FILE*)handle->logger, "GESVJ: the last %d of %d columns (squared norms %.2le in all, largest eigenvalue of their Gram matrix at most %.2le) are left out of the sweeps\n", rank - cols, rank, dropped2, droppedSpectral); }
+      choose_cut(valueGuess, residualGuess, K);
+      before.assign(allNorms.begin(), allNorms.begin() + cols);
     }
+    bool recut = false;
     for (;;) {
       double lastCosine2 = 0.;
       const bool watchOutput = K < cols;   /* with every column handed out only the cosines can end the sweeps */
@@ -195,8 +201,14 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
       const double sigmaK = top[(size_t)(K - 1)], sigma1 = *std::max_element(sig.begin(), sig.end());
       double outside2 = 0.; for (size_t j = (size_t)K; j < top.size(); ++j) { outside2 = std::fma(top[j], top[j], outside2); }   /* the squared values that are not handed out */
       if (hyh::jacobi_truncation_holds_spectral(dropped2, droppedSpectral, sigma1, sigmaK, outside2, eps)) { break; }
-      if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ: value %d is %.2le: the columns left out weigh too much, the sweeps go on with all %d\n", K, sigmaK, rank); }
-      cols = rank; dropped2 = droppedSpectral = 0.; fetch_norms(before, rank); HYH_CHECK(hipStreamSynchronize(s)); if (!hyh::ok()) { return 0; }
+      /* The guess from the column norms left out too much.  The first time, the cut is made again with half of the budget
+       * that the values found allow (the columns taken back in are the unrotated ones next to the cut; the others stay as the
+       * sweeps left them); should that fail too, the sweeps go on with all columns. */
+      const int32_t had = cols;
+      if (!recut) { recut = true; choose_cut(0.5 * hyh::kTruncationBudget * eps * sigma1 * sigmaK, outside2 / 128., had); } else { cols = rank; dropped2 = droppedSpectral = 0.; }
+      if (cols <= had) { cols = rank; dropped2 = droppedSpectral = 0.; }
+      if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ: value %d is %.2le: the %d columns left out weigh too much, the sweeps go on with %d of %d\n", K, sigmaK, rank - had, cols, rank); }
+      fetch_norms(before, cols); HYH_CHECK(hipStreamSynchronize(s)); if (!hyh::ok()) { return 0; }
     }
     std::vector<int32_t> order((size_t)cols); std::iota(order.begin(), order.end(), 0);
     std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return sig[a] > sig[b]; });

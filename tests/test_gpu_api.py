@@ -286,10 +286,10 @@ def _kahan(n, c):
 @pytest.mark.parametrize("case", ["floor left out", "floor taken back in"])
 def test_gevd_leaves_out_floor_columns(case, capfd, monkeypatch):
     """hyacinXGevd (src/gram_evd.cu:94-142) with fewer values wanted than the Cholesky factor has rows: the rows of a noise
-    floor are left out of the Jacobi sweeps when what they weigh is below eps sigma_1 sigma_K (first case: the log says so,
-    and the values still agree with numpy's to 10 eps sigma_1).  The choice is made from the row norms; in the second case
+    floor are left out of the Jacobi sweeps when they cannot move a value by more than 2 eps sigma_1 (first case: the log says
+    so, and the values still agree with numpy's to 10 eps sigma_1).  The choice is made from the row norms; in the second case
     they mislead (a Kahan matrix: its last singular value is 3e-5 of its last row's norm), the test with the values found
-    fails, and the sweeps must go on with all rows: value K is then the floor's, not the Kahan block's."""
+    fails, and the sweeps must take rows back in: value K is then the floor's, not the Kahan block's."""
     import hyacinth_amd as ha
     from gpu_util import dev, zeros, ptr, stream, sync, host
     rng = np.random.default_rng(8)
@@ -318,7 +318,7 @@ def test_gevd_leaves_out_floor_columns(case, capfd, monkeypatch):
     S = host(dS, np.float64, (K,))
     X = host(dX, np.float64, (K, N))[:rank]
     assert "are left out of the sweeps" in log
-    assert ("go on with all" in log) == (case == "floor taken back in")
+    assert ("weigh too much, the sweeps go on with" in log) == (case == "floor taken back in")
     assert 0 < rank <= K and np.abs(S[:rank] - want[:rank]).max() <= 10 * eps * want[0]
     assert np.abs(X @ X.T - np.eye(rank)).max() <= max(1e-12, eps)            # rotations stop at cosines of eps / 16
     if case == "floor taken back in":

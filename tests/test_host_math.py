@@ -255,8 +255,8 @@ def test_jacobi_head(hm):
 
 def test_jacobi_columns_needed(hm):
     """Which prefix of the factor's columns the SVD works on (host/jacobi_stop.hpp): the trailing columns whose squared norms
-    sum to at most eps nu_1 nu_K (a quarter of the 4 eps sigma_1 sigma_K the values found must confirm) are left out, never fewer
-    than K columns kept.  The bound behind it, checked on an
+    sum to at most eps nu_1 nu_K (a quarter of the 4 eps sigma_1 sigma_K the values found must confirm) are left out, never
+    fewer than K columns kept.  The bound behind it, checked on an
     explicit matrix: dropping rows of R of squared Frobenius norm tau moves every singular value down, by at most
     tau / (2 sigma') (sigma' the value without them)."""
     rng = np.random.default_rng(11)
