@@ -31,7 +31,7 @@ API_SYMBOLS = [
 KERNEL_SYMBOLS = [
     "hykColumnExponents", "hykSliceRange", "hykQuantizeLimbs", "hykQuantizeCrt", "hykZeroRows",
     "hykGramWorkspaceBytes", "hykGramWorkspaceClear", "hykGramCrt", "hykGramLimbs", "hykGramSetSlab",
-    "hykGramProfile", "hykGramProfileRead", "hykMfmaCeiling", "hykGramRange", "hykDequantize", "hykPotrfpWorkspaceBytes", "hykPotrfp", "hykPotrfpLeftLooking", "hykPotrfpSetPlainLaunch", "hykPotrfpStaticMaxN", "hykPotrfpStatic", "hykFactorToB", "hykJacobiSweep", "hykJacobiSweepCarry", "hykJacobiSweepTop", "hykJacobiCarryBytes", "hykJacobiSetVariant", "hykJacobiSetSplitTest",
+    "hykGramProfile", "hykGramProfileRead", "hykMfmaCeiling", "hykGramRange", "hykDequantize", "hykPotrfpWorkspaceBytes", "hykPotrfp", "hykPotrfpLeftLooking", "hykPotrfpWanted", "hykMirrorLower", "hykPotrfpSetPlainLaunch", "hykPotrfpStaticMaxN", "hykPotrfpStatic", "hykFactorToB", "hykJacobiSweep", "hykJacobiSweepCarry", "hykJacobiSweepTop", "hykJacobiCarryBytes", "hykJacobiSetVariant", "hykJacobiSetSplitTest",
     "hykColumnNorms", "hykBasisOut", "hykValuesOut", "hykInterpSolve", "hykInterpOut", "hykMatcopy",
     "hykSumSquares", "hykMatmulCf16", "hykGemm", "hykOrthonormalize", "hykLastStatus", "hykTestFailAllocation", "hykColumnExponentsOp", "hykQuantizeLimbsOp", "hykQuantizeCrtOp",
     "hykQuantizeScaleBatchOp", "hykHerkBatchOp", "hykLastHerkPlan", "hykMaxCosine",
@@ -108,6 +108,8 @@ def lib():
         L.hykPotrfpWorkspaceBytes.argtypes = [i32, i32]; L.hykPotrfpWorkspaceBytes.restype = C.c_size_t
         L.hykPotrfp.argtypes = [vp, i32, dbl, i32, i32, i32, vp, i64, vp, i32, vp, vp, vp]
         L.hykPotrfpLeftLooking.argtypes = [vp, i32, dbl, i32, i32, i32, vp, i64, vp, i32, vp, vp, vp]
+        L.hykPotrfpWanted.argtypes = [vp, i32, dbl, i32, i32, dbl, i32, i32, vp, i64, vp, i32, vp, vp, vp, vp]
+        L.hykMirrorLower.argtypes = [vp, i32, i32, vp, i64]
         L.hykPotrfpSetPlainLaunch.argtypes = [i32]
         L.hykPotrfpStaticMaxN.argtypes = []; L.hykPotrfpStaticMaxN.restype = i32
         L.hykPotrfpStatic.argtypes = [vp, i32, dbl, i32, i32, i32, vp, i64, vp, i32, vp, vp]

@@ -41,14 +41,17 @@ struct Factor {
 
 const char* type_tag(int t) { switch (t) { case HYACIN_F64: return "FP64"; case HYACIN_F64_COMPLEX: return "FP64-COMPLEX"; case HYACIN_DD: return "FP128-DD"; default: return "FP128-DD-COMPLEX"; } }
 
-int32_t run_potrfp(const hyacinHandle_t* h, Factor& f, double eps, int32_t K, int32_t N, int32_t* jpiv) {
+/* wanted / cut / left: hykPotrfpWanted (the factorization may end early for a caller that uses `wanted` values only; *left is
+ * then the trace of what it did not factor) */
+int32_t run_potrfp(const hyacinHandle_t* h, Factor& f, double eps, int32_t K, int32_t N, int32_t* jpiv, int32_t wanted = 0, double cut = 0., double* left = nullptr) {
   int32_t* word = (int32_t*)h->pinnedWorkspace; if (!word) { hyh::fail(-1, "pivoted Cholesky", "the handle has no pinned word (hyacinCreate not called?)", __FILE__, __LINE__); }
   if (!hyh::ok()) { return 0; }
-  *word = 0;
-  HYH_KERNEL(hykPotrfp(h->hipStream, h->DeviceSMs, eps, K, N, f.type, f.G, f.ldg, f.Rt.p, f.ldr, jpiv, f.work.p, word));
+  double* trace = reinterpret_cast<double*>(word + 2);   /* the pinned block is 64 bytes */
+  *word = 0; *trace = 0.;
+  HYH_KERNEL(hykPotrfpWanted(h->hipStream, h->DeviceSMs, eps, K, wanted, cut, N, f.type, f.G, f.ldg, f.Rt.p, f.ldr, jpiv, f.work.p, word, trace));
   HYH_CHECK(hipStreamSynchronize(h->hipStream));
   if (!hyh::ok()) { return 0; }
-  int32_t rank = *word;
+  int32_t rank = *word; if (left) { *left = *trace; }
   if (rank < 0) {   /* the workgroups lost each other (a bounded wait inside the kernel gave up): no basis rather than a wrong one */
     hyh::fail(-5, "pivoted Cholesky", "a workgroup gave up waiting for the others; no factor was produced", __FILE__, __LINE__);
     return 0;
@@ -72,10 +75,18 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
   eps = std::min(std::max(std::fabs(eps), machineEps), 1.);
 
   hyh::Scratch jpiv(handle, sizeof(int32_t) * (size_t)N);
-  int32_t rank;
-  { Factor f(handle, N, N, (int)Gtype, G, ldg);
-    rank = run_potrfp(handle, f, lrqr ? eps : 0., N, N, jpiv.as<int32_t>());
+  int32_t rank = 0;
+  /* First with a factorization that may end early (hykPotrfpWanted: K values are wanted, and a floor right under them is
+   * not worth its rows); if the values found then say that what was not factored weighs too much, once more in full. */
+  for (int attempt = 0; attempt < 2; ++attempt) {
+    bool again = false;
+    Factor f(handle, N, N, (int)Gtype, G, ldg);
+    if (attempt > 0 && !f.widened.p) { HYH_KERNEL(hykMirrorLower(s, N, f.type, f.G, f.ldg)); }   /* the first factorization has used the strict upper triangle of G */
+    const bool mayEndEarly = attempt == 0 && lrqr && K < N;
+    double unfactored = 0.;
+    rank = run_potrfp(handle, f, lrqr ? eps : 0., N, N, jpiv.as<int32_t>(), mayEndEarly ? K : 0, mayEndEarly ? hyh::kTruncationGuess * hyh::kTruncationBudget * eps : 0., &unfactored);
     if (rank <= 0 || !hyh::ok()) { return 0; }
+    if (handle->logger && unfactored > 0.) { std::fprintf((FILE*)handle->logger, "POTRFP: ended after %d columns, what is left of G has trace %.2le\n", rank, unfactored); }
     /* B = (R P^T)^H, N x rank, in the precision of the output storage type: doubles for FP64, floats for FP32 and FP16
      * (reference: src/gram_evd.cu:96-98) */
     const bool wideB = (int)Atype == HYACIN_F64 || (int)Atype == HYACIN_F64_COMPLEX; const int Btype = (wideB ? HYACIN_F64 : HYACIN_F32) + Complex;
@@ -134,17 +145,18 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
      * below the largest eigenvalue) within the budget of the values, trace within the budget of the residual. */
     std::vector<double> allNorms, absGram; int32_t c0 = rank;
     auto choose_cut = [&](double valueBudget, double residualBudget, int32_t atLeast) {
-      int32_t t = rank; double sum = 0.;   /* trace rule */
+      int32_t t = rank; double sum = unfactored;   /* trace rule; what the Cholesky left unfactored counts as rows left out, with its trace as the bound of its largest eigenvalue */
       while (t > atLeast && sum + allNorms[(size_t)(t - 1)] * allNorms[(size_t)(t - 1)] <= valueBudget) { sum += allNorms[(size_t)(t - 1)] * allNorms[(size_t)(t - 1)]; --t; }
       cols = t; bool sharper = false;
       if (!absGram.empty() && c0 < cols) {
-        const hyh::JacobiCut cut = hyh::jacobi_columns_needed_spectral(absGram, rank, c0, atLeast, valueBudget / 1.01, residualBudget);   /* 1 %: the products are rounded */
-        if (cut.cols < cols) { cols = cut.cols; droppedSpectral = 1.01 * cut.spectral; sharper = true; }
+        const hyh::JacobiCut cut = hyh::jacobi_columns_needed_spectral(absGram, rank, c0, atLeast, (valueBudget - unfactored) / 1.01, residualBudget - unfactored);   /* 1 %: the products are rounded */
+        if (cut.cols < cols) { cols = cut.cols; droppedSpectral = 1.01 * cut.spectral + unfactored; sharper = true; }
       }
-      dropped2 = 0.; for (int32_t j = rank - 1; j >= cols; --j) { dropped2 = std::fma(allNorms[(size_t)j], allNorms[(size_t)j], dropped2); }
+      dropped2 = unfactored; for (int32_t j = rank - 1; j >= cols; --j) { dropped2 = std::fma(allNorms[(size_t)j], allNorms[(size_t)j], dropped2); }
       if (!sharper) { droppedSpectral = dropped2; }   /* the trace bounds the largest eigenvalue */
       if (handle->logger && cols < rank) { std::fprintf((FILE*)handle->logger, "GESVJ: the last %d of %d columns (squared norms %.2le in all, largest eigenvalue of their Gram matrix at most %.2le) are left out of the sweeps\n", rank - cols, rank, dropped2, droppedSpectral); }
     };
+    dropped2 = droppedSpectral = unfactored;
     if (K < rank && rank > 1) {
       fetch_norms(allNorms, rank); HYH_CHECK(hipStreamSynchronize(s)); if (!hyh::ok()) { return 0; }
       std::vector<double> v(allNorms); std::nth_element(v.begin(), v.begin() + (K - 1), v.end(), std::greater<double>());
@@ -196,7 +208,7 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
       }
       fetch_norms(sig, cols); HYH_CHECK(hipStreamSynchronize(s));
       if (!hyh::ok()) { return 0; }
-      if (cols == rank) { break; }
+      if (cols == rank && unfactored == 0.) { break; }
       std::vector<double> top(sig); std::nth_element(top.begin(), top.begin() + (K - 1), top.end(), std::greater<double>());
       const double sigmaK = top[(size_t)(K - 1)], sigma1 = *std::max_element(sig.begin(), sig.end());
       double outside2 = 0.; for (size_t j = (size_t)K; j < top.size(); ++j) { outside2 = std::fma(top[j], top[j], outside2); }   /* the squared values that are not handed out */
@@ -204,11 +216,16 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
       /* The guess from the column norms left out too much.  The first time, the cut is made again with half of the budget
        * that the values found allow (the columns taken back in are the unrotated ones next to the cut; the others stay as the
        * sweeps left them); should that fail too, the sweeps go on with all columns. */
+      if (unfactored > 0. && !hyh::jacobi_truncation_holds_spectral(unfactored, unfactored, sigma1, sigmaK, outside2, eps)) { again = true; break; }   /* no cut of the rows at hand can make up for the rows that were never factored */
       const int32_t had = cols;
-      if (!recut) { recut = true; choose_cut(0.5 * hyh::kTruncationBudget * eps * sigma1 * sigmaK, outside2 / 128., had); } else { cols = rank; dropped2 = droppedSpectral = 0.; }
-      if (cols <= had) { cols = rank; dropped2 = droppedSpectral = 0.; }
+      if (!recut) { recut = true; choose_cut(0.5 * hyh::kTruncationBudget * eps * sigma1 * sigmaK, outside2 / 128., had); } else { cols = rank; dropped2 = droppedSpectral = unfactored; }
+      if (cols <= had) { cols = rank; dropped2 = droppedSpectral = unfactored; }
       if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ: value %d is %.2le: the %d columns left out weigh too much, the sweeps go on with %d of %d\n", K, sigmaK, rank - had, cols, rank); }
       fetch_norms(before, cols); HYH_CHECK(hipStreamSynchronize(s)); if (!hyh::ok()) { return 0; }
+    }
+    if (again) {
+      if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ: what the Cholesky left unfactored (%.2le) weighs too much against the values found: factoring again, in full\n", unfactored); }
+      continue;
     }
     std::vector<int32_t> order((size_t)cols); std::iota(order.begin(), order.end(), 0);
     std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return sig[a] > sig[b]; });
@@ -227,6 +244,7 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
     HYH_CHECK(hipStreamSynchronize(s));   /* Sout / order are host temporaries */
     if (!hyh::ok()) { return 0; }
     if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ-%s [eps=%.1le] [M=%d] [N=%d] [K=%d] [sweeps=%d] [SVD-rank=%d]\n", wideB ? (Complex ? "FP64-COMPLEX" : "FP64") : (Complex ? "FP32-COMPLEX" : "FP32"), eps, N, rank, K, used, svdRank); }
+    break;
   }
   return hyh::ok() ? rank : 0;
 }

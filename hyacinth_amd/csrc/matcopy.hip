@@ -92,6 +92,32 @@ extern "C" int hykMatcopy(hipStream_t stream, char mode, int64_t M, int64_t N, i
 }
 
 /* *out += sum of squares of the M x N FP64 matrix (a complex matrix is passed as 2M x N) */
+/* G[y, x] = conj(G[x, y]) for y < x: the strict upper triangle of a Hermitian matrix written again from its lower one.
+ * W doubles per real or imaginary part (1: FP64, 2: double-double).  A thread per entry, adjacent threads along y. */
+template <int W, bool CPLX>
+__global__ __launch_bounds__(256) void mirror_lower_kernel(int32_t N, double* __restrict__ G, int64_t ldg) {
+  constexpr int WE = W * (CPLX ? 2 : 1);
+  const int y = (int)(blockIdx.x * 256 + threadIdx.x), x = (int)blockIdx.y;
+  if (y >= x || x >= N) { return; }
+  const double* src = &G[((int64_t)x + (int64_t)y * ldg) * WE]; double* dst = &G[((int64_t)y + (int64_t)x * ldg) * WE];
+  #pragma unroll
+  for (int w = 0; w < WE; ++w) { dst[w] = (CPLX && w >= W) ? -src[w] : src[w]; }
+}
+
+extern "C" int hykMirrorLower(hipStream_t stream, int32_t N, int32_t Gtype, void* G, int64_t ldg) {
+  if (N <= 1) { return 0; }
+  if (!G || ldg < N || N > 65535) { return -1; }
+  dim3 grid((uint32_t)((N + 255) / 256), (uint32_t)N);
+  switch (Gtype) {
+    case HYK_F64: mirror_lower_kernel<1, false><<<grid, 256, 0, stream>>>(N, (double*)G, ldg); break;
+    case HYK_F64C: mirror_lower_kernel<1, true><<<grid, 256, 0, stream>>>(N, (double*)G, ldg); break;
+    case HYK_DD: mirror_lower_kernel<2, false><<<grid, 256, 0, stream>>>(N, (double*)G, ldg); break;
+    case HYK_DDC: mirror_lower_kernel<2, true><<<grid, 256, 0, stream>>>(N, (double*)G, ldg); break;
+    default: return -1;
+  }
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
 extern "C" int hykSumSquares(hipStream_t stream, int64_t M, int64_t N, const double* A, int64_t lda, double* out) {
   if (M <= 0 || N <= 0) { return 0; }
   dim3 grid((uint32_t)((M + 255) / 256 < 64 ? (M + 255) / 256 : 64), (uint32_t)(N < 256 ? N : 256));

@@ -67,7 +67,7 @@ constexpr int SPIN_LIMIT = 1 << 22;   /* polls of one record before the run is g
 struct PotrfArgs {
   int32_t N, K, ldr; double eps2;
   const double* G; int64_t ldg;
-  double* Rt; double* D; int32_t* jpiv; int32_t* pos; Record* records; int32_t* rankOut;
+  double* Rt; double* D; int32_t* jpiv; int32_t* pos; Record* records; int32_t* rankOut; double* traceOut;
 };
 
 /* scalar types: value = re (+ i im), each part a dd_t (lo part unused in FP64 mode) */
@@ -281,7 +281,7 @@ __global__ __launch_bounds__(P_THREADS) void potrfp_kernel(const PotrfArgs a) {
     }
     rank = k + 1;
   }
-  if (wg == 0 && tid == 0) { *a.rankOut = alive ? rank : -1; }
+  if (wg == 0 && tid == 0) { *a.rankOut = alive ? rank : -1; if (a.traceOut) { *a.traceOut = 0.; } }   /* this kernel has no cut (hykPotrfpWanted) */
 }
 
 /* one-time per kernel: how many workgroups may be co-resident */
@@ -338,6 +338,9 @@ constexpr int CTL_COUNTER = 32, CTL_TIMING = 40;
 struct Args {
   int32_t N, K, ldr, agents; double eps2;
   double* G; int64_t ldg; double* Rt; int32_t* jpiv; uint64_t* records; uint64_t* ctl; int32_t* rankOut;
+  /* wanted / cut: a caller that uses the `wanted` leading values of the factor only lets the factorization end once what is
+   * left of G weighs little against them (hykPotrfpWanted); traceOut: the trace of what is left when the factorization ends */
+  int32_t wanted; double cut; double* traceOut;
 };
 
 __device__ __forceinline__ uint64_t ld_shared_u64(const uint64_t* p) { return __hip_atomic_load(const_cast<uint64_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
@@ -540,7 +543,7 @@ __global__ __launch_bounds__(THREADS) void potrfp_blocked_kernel(const Args a) {
 
   /* agent state */
   R d = R::zero(); bool dead = !mine; uint32_t epoch = 0; RC cur, nxt, seen, seen2; cur.clear(); nxt.clear(); seen.clear(); seen2.clear();
-  double thresh = 0.; int k = 0; bool failed = false, stop = false; int mypiv = 0;
+  double thresh = 0., traceFirst = 0., normFirst2 = 0., traceWanted = 0.; int k = 0; bool failed = false, stop = false, cutInForce = false; int mypiv = 0;
   /* what was fetched for the runner-up: its column of G' and (lane t) its factor entry t of this panel */
   int specCol = -1; R specGre = R::zero(), specGim = R::zero(); double specRow[WE], specNew[WE];
   #pragma unroll
@@ -569,6 +572,17 @@ __global__ __launch_bounds__(THREADS) void potrfp_blocked_kernel(const Args a) {
         HYK_STAMP(0);
         while (!failed && !stop && k < kb + PB) {
           HYK_COUNT(9);
+          /* the second way to end (hykPotrfpWanted): a step takes the squared norm of its row of the factor off the trace of
+           * what is left, so the traces around steps 1 and `wanted` give the norms nu_1 and nu_w of those rows, and
+           * b = cut nu_1 nu_w; after `wanted` steps it becomes the threshold if what is left of G is within 32 b already (a floor
+           * right under the wanted values).  Every agent holds the same record, so all decide alike. */
+          if (k == 0) { traceFirst = cur.tr; }
+          if (k == 1) { normFirst2 = traceFirst - cur.tr; }
+          if (k + 1 == a.wanted) { traceWanted = cur.tr; }
+          if (a.cut > 0. && k == a.wanted) {
+            const double normWanted2 = traceWanted - cur.tr, b = (normFirst2 > 0. && normWanted2 > 0.) ? a.cut * sqrt(normFirst2 * normWanted2) : 0.;
+            if (cur.tr <= 32. * b && thresh < b) { thresh = b; cutInForce = true; }
+          }
           const int c = cur.bi, j = k - kb; R dc{ dd_t{ cur.bx, cur.by } }, sq, rho; sqrt_rsqrt<DD>(dc, sq, rho);
           const bool hit = specCol == c; const bool work = !dead && l != c;
           if (lane == j) { mypiv = c; }
@@ -791,7 +805,10 @@ __global__ __launch_bounds__(THREADS) void potrfp_blocked_kernel(const Args a) {
     if (tid == 0) { info[3] = k; }   /* the agent's count of columns done */
     __syncthreads();
     for (int i = tid; i < N; i += THREADS) { a.jpiv[i] = (int32_t)order[i] + 1; }
-    if (tid == 0) { *a.rankOut = failed ? -1 : ((N - info[3] == 1) ? info[3] + 1 : info[3]); }
+    if (tid == 0) {
+      *a.rankOut = failed ? -1 : ((N - info[3] == 1) ? info[3] + 1 : info[3]);
+      if (a.traceOut) { *a.traceOut = (!cutInForce || failed || N - info[3] <= 1 || !(cur.tr > 0.)) ? 0. : cur.tr; }   /* the trace of what is left of G (the first agent's copy of the last record) */
+    }
   }
 }
 
@@ -824,11 +841,11 @@ constexpr size_t EXCHANGE_BYTES = 2 * blk::MAX_AGENTS * blk::REC_WORDS * 8 + blk
 static_assert(EXCHANGE_BYTES >= 2 * MAX_WORKGROUPS * sizeof(Record), "the exchange area holds the records of either kernel");
 size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 
-int run_potrfp(hipStream_t stream, bool blocked, int32_t computeUnits, double eps, int32_t K, int32_t N, int32_t Gtype, void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, void* workspace, int32_t* rankOut) {
+int run_potrfp(hipStream_t stream, bool blocked, int32_t computeUnits, double eps, int32_t K, int32_t N, int32_t Gtype, void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, void* workspace, int32_t* rankOut, int32_t wanted = 0, double cut = 0., double* traceOut = nullptr) {
   if (N <= 0) { return 0; }
   if (!workspace || !G || !Rt || !jpiv || !rankOut) { return -1; }
   if (K <= 0 || K > N) { K = N; }
-  if (ldg < N || ldr < (K < N ? K + 1 : N) || computeUnits < 1) { return -1; }
+  if (ldg < N || ldr < (K < N ? K + 1 : N) || computeUnits < 1 || !(cut >= 0.)) { return -1; }
   const bool dd = (Gtype & ~1) == HYK_DD, cplx = Gtype & 1;
   if (!dd && (Gtype & ~1) != HYK_F64) { return -1; }
   char* w = (char*)workspace; int32_t* pos = (int32_t*)w; w += align256((size_t)N * 4); uint64_t* exchange = (uint64_t*)w; w += EXCHANGE_BYTES; double* D = (double*)w;
@@ -837,10 +854,11 @@ int run_potrfp(hipStream_t stream, bool blocked, int32_t computeUnits, double ep
   if (blocked && N <= blk::MAX_N && agents <= grid) {
     blk::Args b; b.N = N; b.K = K; b.ldr = ldr; b.agents = agents; b.eps2 = eps * eps; b.G = (double*)G; b.ldg = ldg; b.Rt = (double*)Rt; b.jpiv = jpiv;
     b.records = exchange; b.ctl = exchange + 2 * blk::MAX_AGENTS * blk::REC_WORDS; b.rankOut = rankOut;
+    b.wanted = (wanted > 0 && wanted < N) ? wanted : 0; b.cut = b.wanted ? cut : 0.; b.traceOut = traceOut;
     if (dd) { return cplx ? blk::launch<true, true>(stream, b, computeUnits) : blk::launch<true, false>(stream, b, computeUnits); }
     return cplx ? blk::launch<false, true>(stream, b, computeUnits) : blk::launch<false, false>(stream, b, computeUnits);
   }
-  PotrfArgs a; a.N = N; a.K = K; a.ldr = ldr; a.eps2 = eps * eps; a.G = (const double*)G; a.ldg = ldg; a.Rt = (double*)Rt; a.jpiv = jpiv; a.rankOut = rankOut;
+  PotrfArgs a; a.N = N; a.K = K; a.ldr = ldr; a.eps2 = eps * eps; a.G = (const double*)G; a.ldg = ldg; a.Rt = (double*)Rt; a.jpiv = jpiv; a.rankOut = rankOut; a.traceOut = traceOut;
   a.D = D; a.pos = pos; a.records = (Record*)exchange;
   if (dd) { return cplx ? launch<true, true>(stream, a, computeUnits) : launch<true, false>(stream, a, computeUnits); }
   return cplx ? launch<false, true>(stream, a, computeUnits) : launch<false, false>(stream, a, computeUnits);
@@ -857,6 +875,10 @@ extern "C" size_t hykPotrfpWorkspaceBytes(int32_t N, int32_t Gtype) {
 
 extern "C" int hykPotrfp(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, int32_t N, int32_t Gtype, void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, void* workspace, int32_t* rankOut) {
   return run_potrfp(stream, true, computeUnits, eps, K, N, Gtype, G, ldg, Rt, ldr, jpiv, workspace, rankOut);
+}
+
+extern "C" int hykPotrfpWanted(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, int32_t wanted, double cut, int32_t N, int32_t Gtype, void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, void* workspace, int32_t* rankOut, double* traceOut) {
+  return run_potrfp(stream, true, computeUnits, eps, K, N, Gtype, G, ldg, Rt, ldr, jpiv, workspace, rankOut, wanted, cut, traceOut);
 }
 
 extern "C" int hykPotrfpLeftLooking(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, int32_t N, int32_t Gtype, void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, void* workspace, int32_t* rankOut) {

@@ -96,6 +96,20 @@ int hykDequantize(hipStream_t stream, int32_t N, int32_t orderC, const uint64_t*
 size_t hykPotrfpWorkspaceBytes(int32_t N, int32_t Gtype);
 int hykPotrfp(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, int32_t N, int32_t Gtype, void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, void* workspace, int32_t* rankOut);
 int hykPotrfpLeftLooking(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, int32_t N, int32_t Gtype, void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, void* workspace, int32_t* rankOut);
+/* hykPotrfp for a caller that will use the `wanted` leading singular values of the factor only (the SVD tail with K < N;
+ * no counterpart in the reference, whose factorization always runs to its eps rule, src/gram_evd.cu:105).  The rows never
+ * computed are rows left out of G = R^H R: they take what is left of G (positive semidefinite, trace t) off it, which moves
+ * a singular value by at most t / (2 sigma).  With b = cut nu_1 nu_w (the norms of rows 1 and w = wanted of the factor, which
+ * are what steps 1 and w take off the trace of what is left): if t <= 32 b after
+ * `wanted` steps (a floor right under the wanted values), the factorization also ends as soon as t <= b, one step later
+ * at the earliest.  Otherwise it
+ * runs to its eps rule as hykPotrfp does: the whole budget then stays with a caller that can bound the rows it leaves out
+ * more sharply than by their trace.  nu_1 nu_w only estimates sigma_1 sigma_w: the caller has to test t against the values
+ * it finds and, should the test fail, factor again without a cut (hykMirrorLower restores G for that: the factorization
+ * changes the strict upper triangle only).  traceOut (device or pinned host memory, may be null): t when the factorization
+ * ended if the second rule was in force (by whichever rule it then ended), else 0.  wanted <= 0, wanted >= N or cut == 0:
+ * hykPotrfp.  The left-looking kernel (N > 8192, few compute units) ignores wanted / cut and reports 0. */
+int hykPotrfpWanted(hipStream_t stream, int32_t computeUnits, double eps, int32_t K, int32_t wanted, double cut, int32_t N, int32_t Gtype, void* G, int64_t ldg, void* Rt, int32_t ldr, int32_t* jpiv, void* workspace, int32_t* rankOut, double* traceOut);
 /* Process-wide launch mode of the two kernels above (no counterpart in the reference).  They are launched cooperatively by
  * default.  enable != 0: a grid that fits the device by the occupancy query is started with a plain launch.  For runs under
  * profilers whose kernel tracing does not get along with cooperative launches (rocprofv3 --kernel-trace: the process then
@@ -172,6 +186,10 @@ int hykInterpOut(hipStream_t stream, int32_t N, int32_t K, int32_t Atype, const 
 
 /* Converting copy / transpose.  Replaces scatter_matcopy modes 'A', 'T', 'C', src/matcopy.cu:23-44,58-96. */
 int hykMatcopy(hipStream_t stream, char mode, int64_t M, int64_t N, int32_t srcType, const void* A, int64_t lda, int32_t dstType, void* B, int64_t ldb);
+
+/* G[y, x] = conj(G[x, y]) for y < x (Gtype: FP64 or double-double, real or complex): writes the strict upper triangle of a
+ * Hermitian matrix again from its lower one, which hykPotrfp leaves as it was.  No counterpart in the reference. */
+int hykMirrorLower(hipStream_t stream, int32_t N, int32_t Gtype, void* G, int64_t ldg);
 
 /* *out += sum of squares.  Replaces cublasDnrm2_64, src/lra.cpp:170,204. */
 int hykSumSquares(hipStream_t stream, int64_t M, int64_t N, const double* A, int64_t lda, double* out);

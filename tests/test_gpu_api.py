@@ -283,8 +283,9 @@ def _kahan(n, c):
     return (s ** np.arange(n))[:, None] * (np.triu(-c * np.ones((n, n)), 1) + np.eye(n)) * (1.0 - 1e-3 * np.arange(n))[None, :]
 
 
+@pytest.mark.parametrize("gtype", [0, 6])                     # Gram in FP64, in double-double
 @pytest.mark.parametrize("case", ["floor left out", "floor taken back in"])
-def test_gevd_leaves_out_floor_columns(case, capfd, monkeypatch):
+def test_gevd_leaves_out_floor_columns(case, gtype, capfd, monkeypatch):
     """hyacinXGevd (src/gram_evd.cu:94-142) with fewer values wanted than the Cholesky factor has rows: the rows of a noise
     floor are left out of the Jacobi sweeps when they cannot move a value by more than 2 eps sigma_1 (first case: the log says
     so, and the values still agree with numpy's to 10 eps sigma_1).  The choice is made from the row norms; in the second case
@@ -307,9 +308,10 @@ def test_gevd_leaves_out_floor_columns(case, capfd, monkeypatch):
     monkeypatch.setenv("HYACIN_VERBOSE", "1")
     h = ha.create_handle(stream=stream().value)
     try:
-        dG, dS, dX = dev(np.ascontiguousarray(G.T)), zeros(8 * K), zeros(8 * N * K)
+        raw = np.zeros((N, N, 2 if gtype == 6 else 1)); raw[..., 0] = G.T
+        dG, dS, dX = dev(raw), zeros(8 * K), zeros(8 * N * K)
         capfd.readouterr()
-        rank = ha.lib().hyacinXGevd(C.byref(h), eps, N, K, 0, ptr(dX), N, ptr(dS), 0, ptr(dG), N)
+        rank = ha.lib().hyacinXGevd(C.byref(h), eps, N, K, 0, ptr(dX), N, ptr(dS), gtype, ptr(dG), N)
         sync()
         C.CDLL(None).fflush(None)                       # the log goes through the C library's buffered stdout
         log = capfd.readouterr().out
@@ -319,6 +321,9 @@ def test_gevd_leaves_out_floor_columns(case, capfd, monkeypatch):
     X = host(dX, np.float64, (K, N))[:rank]
     assert "are left out of the sweeps" in log
     assert ("weigh too much, the sweeps go on with" in log) == (case == "floor taken back in")
+    # in the second case the Cholesky itself ends early at first (what is left after K steps is the floor, well within its
+    # estimate of the budget), the values found refute the estimate, and the matrix is factored again in full
+    assert ("POTRFP: ended after" in log and "factoring again, in full" in log) == (case == "floor taken back in")
     assert 0 < rank <= K and np.abs(S[:rank] - want[:rank]).max() <= 10 * eps * want[0]
     assert np.abs(X @ X.T - np.eye(rank)).max() <= max(1e-12, eps)            # rotations stop at cosines of eps / 16
     if case == "floor taken back in":

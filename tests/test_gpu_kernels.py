@@ -410,6 +410,61 @@ def test_potrfp_plain_launch(gl, entry, gbase, cplx, N):
     assert outs[0][0] > 0 and outs[0][0] == outs[1][0] and np.array_equal(outs[0][1], outs[1][1]) and np.array_equal(outs[0][2], outs[1][2])
 
 
+@pytest.mark.parametrize("gbase,cplx", [(0, 0), (0, 1), (6, 0), (6, 1)])
+def test_potrfp_wanted(gl, gbase, cplx):
+    """hykPotrfpWanted: the factorization for a caller that uses `wanted` values only.  Twelve graded values over a floor of
+    288 columns of 1e-6: what is left of G after twelve steps (2.9e-10) is within 32 b for cut = 1e-6 (b = 1e-6 nu_1 nu_w, the norms
+    of rows 1 and w of the factor: about 2e-10), so the factorization ends at the first step that leaves at most b, with the
+    pivots of the full run up to there and the trace of what is left in traceOut.  With cut = 1e-8 the floor is far above 32 b
+    and with cut = 0 there is no rule: both give the full run's rank and pivots and report 0."""
+    from gpu_util import dev, zeros, ptr, stream, sync, host
+    rng = np.random.default_rng(47 + cplx + gbase)
+    gtype, N, wanted = gbase + cplx, 300, 12
+    raw = spd_raw(rng, N, wanted, cplx, gbase, 1e-6)
+    width = raw.shape[2]
+    def run(cut):
+        Rt, jp, rk, tr, ws, dG = zeros(N * N * width * 8), zeros(N * 4), zeros(4), zeros(8), zeros(gl.L.hykPotrfpWorkspaceBytes(N, gtype)), dev(raw)
+        print("hykPotrfpWanted gtype", gtype, "cut", cut, flush=True)
+        assert gl.L.hykPotrfpWanted(stream(), 256, 1e-9, N, wanted, cut, N, gtype, ptr(dG), N, ptr(Rt), N, ptr(jp), ptr(ws), ptr(rk), ptr(tr)) == 0
+        sync()
+        R = host(Rt, np.float64, (N, N, width))[..., 0] + (1j * host(Rt, np.float64, (N, N, width))[..., 2 if gbase == 6 else 1] if cplx else 0)   # [column][row]
+        return int(host(rk, np.int32)[0]), host(jp, np.int32).copy(), float(host(tr, np.float64)[0]), R
+    full = run(0.0)
+    assert full[0] == N and full[2] == 0.0
+    far = run(1e-8)
+    assert far[0] == full[0] and np.array_equal(far[1], full[1]) and far[2] == 0.0
+    rank, piv, left, R = run(1e-6)
+    rows2 = (np.abs(full[3]) ** 2).sum(axis=0)                                   # squared norms of the rows of the full factor, in pivot order
+    b = 1e-6 * np.sqrt(rows2[0] * rows2[wanted - 1])
+    assert wanted < rank < N and np.array_equal(piv[:rank], full[1][:rank])
+    tail = lambda t: rows2[t:].sum()                                             # the trace of what is left after t steps
+    ideal = next(t for t in range(wanted + 1, N) if tail(t) <= b)                # the first step that leaves at most b
+    assert abs(rank - ideal) <= 1                                                # (the kernel's running trace carries the rounding of its updates: a step of the floor is 0.5 % of b)
+    assert abs(left - tail(rank)) <= 1e-2 * tail(rank)
+    assert np.allclose(R[:, :rank], full[3][:, :rank], rtol=0, atol=1e-13)
+
+
+@pytest.mark.parametrize("gtype", [0, 1, 6, 7])
+def test_mirror_lower(gl, gtype):
+    """hykMirrorLower: the strict upper triangle written again as the conjugate of the lower one; diagonal and lower triangle
+    untouched, also with a padded leading dimension."""
+    from gpu_util import dev, ptr, stream, sync, host
+    rng = np.random.default_rng(48 + gtype)
+    N, ld, cplx, w = 77, 80, gtype & 1, 2 if gtype >= 6 else 1
+    raw = rng.standard_normal((N, ld, w * (1 + cplx)))                          # [column][row][words]
+    d = dev(raw)
+    print("hykMirrorLower gtype", gtype, flush=True)
+    assert gl.L.hykMirrorLower(stream(), N, gtype, ptr(d), ld) == 0
+    sync()
+    got, want = host(d, np.float64, raw.shape), raw.copy()
+    for x in range(N):
+        for y in range(x):
+            want[x, y] = raw[y, x]
+            if cplx:
+                want[x, y, w:] = -raw[y, x, w:]
+    assert np.array_equal(got, want)
+
+
 @pytest.mark.parametrize("cplx", [0, 1])
 @pytest.mark.parametrize("opA", ["N", "T", "C"])
 @pytest.mark.parametrize("M,N,K,pad", [(300, 70, 45, 0), (128, 128, 64, 0), (1000, 260, 333, 8), (257, 129, 1, 0), (96, 40, 200, 3)])
