@@ -10,14 +10,14 @@ from oracle import closed_form as cf
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 SRC = os.path.join(ROOT, "tests", "host_math", "host_math.cpp")
-LIB = os.path.join(ROOT, "tests", "host_math", "libhost_math.so")
+LIB = os.environ.get("HYACIN_HOST_MATH_LIBRARY") or os.path.join(ROOT, "tests", "host_math", "libhost_math.so")   # (the variable: a build made elsewhere, e.g. with a sanitizer)
 
 
 @pytest.fixture(scope="module")
 def hm():
     hdr = os.path.join(ROOT, "hyacinth_amd", "csrc", "hyk_common.h")
     stop = os.path.join(ROOT, "hyacinth_amd", "csrc", "host", "jacobi_stop.hpp")
-    if not os.path.exists(LIB) or os.path.getmtime(LIB) < max(os.path.getmtime(SRC), os.path.getmtime(hdr), os.path.getmtime(stop)):
+    if not os.environ.get("HYACIN_HOST_MATH_LIBRARY") and (not os.path.exists(LIB) or os.path.getmtime(LIB) < max(os.path.getmtime(SRC), os.path.getmtime(hdr), os.path.getmtime(stop))):
         subprocess.check_call(["g++", "-O2", "-std=c++17", "-shared", "-fPIC", "-I", os.path.join(ROOT, "hyacinth_amd", "csrc"), SRC, "-o", LIB])
     L = C.CDLL(LIB)
     L.hm_frexp.restype = C.c_int32
