@@ -135,8 +135,8 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
      * columns of B) out of the SVD takes a positive semidefinite matrix of trace tau (the sum of their squared norms) off
      * G: every eigenvalue moves down by at most tau, a singular value by at most tau / (2 sigma'), sigma' being the value
      * found without them.  The columns of a noise floor under the values that are wanted are not worth their rotations:
-     * jacobi_columns_needed picks the prefix from the column norms, and what the sweeps then find must confirm it
-     * (jacobi_truncation_holds with the values themselves), or the sweeps go on with all columns. */
+     * the prefix is picked from the column norms (choose_cut below), and what the sweeps then find must confirm it
+     * (jacobi_truncation_holds_spectral with the values themselves), or columns are taken back in. */
     int32_t cols = rank; double dropped2 = 0., droppedSpectral = 0.;
     /* The cut for given budgets: the longest tail [t, rank), t >= atLeast, that passes the trace rule or the sharper rule
      * (jacobi_columns_needed_spectral: what moves a value is the largest eigenvalue of the Gram matrix of the columns left
