@@ -284,13 +284,15 @@ def _kahan(n, c):
 
 
 @pytest.mark.parametrize("gtype", [0, 6])                     # Gram in FP64, in double-double
-@pytest.mark.parametrize("case", ["floor left out", "floor taken back in"])
+@pytest.mark.parametrize("case", ["floor left out", "floor taken back in", "floor never factored"])
 def test_gevd_leaves_out_floor_columns(case, gtype, capfd, monkeypatch):
     """hyacinXGevd (src/gram_evd.cu:94-142) with fewer values wanted than the Cholesky factor has rows: the rows of a noise
     floor are left out of the Jacobi sweeps when they cannot move a value by more than 2 eps sigma_1 (first case: the log says
     so, and the values still agree with numpy's to 10 eps sigma_1).  The choice is made from the row norms; in the second case
     they mislead (a Kahan matrix: its last singular value is 3e-5 of its last row's norm), the test with the values found
-    fails, and the sweeps must take rows back in: value K is then the floor's, not the Kahan block's."""
+    fails, and the sweeps must take rows back in: value K is then the floor's, not the Kahan block's.  Third case: a floor
+    right under the K wanted values, light enough for the Cholesky itself to end after K + 1 columns (hykPotrfpWanted); the
+    values found confirm it, and they are within (trace left) / (2 sigma_K) of numpy's."""
     import hyacinth_amd as ha
     from gpu_util import dev, zeros, ptr, stream, sync, host
     rng = np.random.default_rng(8)
@@ -298,6 +300,10 @@ def test_gevd_leaves_out_floor_columns(case, gtype, capfd, monkeypatch):
         N, K, eps = 300, 20, 1e-8
         V = haar(rng, N, N, False)
         R = (np.concatenate([10.0 ** -np.linspace(0, 6, 40), np.full(N - 40, 1e-8)])[:, None]) * V.T     # singular values: 40 graded ones over a floor
+    elif case == "floor never factored":
+        N, K, eps = 300, 20, 1e-4
+        V = haar(rng, N, N, False)
+        R = (np.concatenate([10.0 ** -np.linspace(0, 2, K), np.full(N - K, 1e-5)])[:, None]) * V.T       # 20 values down to 1e-2 over a floor of 1e-5
     else:
         N, K, eps = 64, 24, 1e-6
         R = np.zeros((N, N))
@@ -320,6 +326,9 @@ def test_gevd_leaves_out_floor_columns(case, gtype, capfd, monkeypatch):
     S = host(dS, np.float64, (K,))
     X = host(dX, np.float64, (K, N))[:rank]
     assert "are left out of the sweeps" in log
+    if case == "floor never factored":
+        assert "POTRFP: ended after %d columns" % (K + 1) in log and "factoring again" not in log
+        assert rank == K and np.abs(S - want[:K]).max() <= (N - K) * 1e-10 / (2 * want[K - 1]) + 1e-14
     assert ("weigh too much, the sweeps go on with" in log) == (case == "floor taken back in")
     # in the second case the Cholesky itself ends early at first (what is left after K steps is the floor, well within its
     # estimate of the budget), the values found refute the estimate, and the matrix is factored again in full
