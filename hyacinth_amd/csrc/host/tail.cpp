@@ -114,7 +114,9 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
      * sweep ends "settled" depends on the data, and an allocation in the middle of the loop would make the calls that can
      * fail depend on it too; needed only when fewer values are handed out than the factor has columns) */
     const bool mayCheck = K < rank && rank > 1;
-    hyh::Scratch gram(handle, mayCheck ? (size_t)rank * rank * (wideB ? 8 : 4) * (1 + Complex) : 0), dMark(handle, mayCheck ? sizeof(int32_t) * (size_t)rank : 0), dOut(handle, mayCheck ? 64 : 0);
+    const size_t elemB = (size_t)(wideB ? 8 : 4) * (1 + Complex);
+    hyh::Scratch gram(handle, mayCheck ? (size_t)rank * rank * elemB : 0), dMark(handle, mayCheck ? sizeof(int32_t) * (size_t)rank : 0), dOut(handle, mayCheck ? 64 : 0);
+    hyh::Scratch polishA(handle, mayCheck ? (size_t)N * K * elemB : 0), polishB(handle, mayCheck ? (size_t)N * K * elemB : 0), dPolishOrder(handle, mayCheck ? sizeof(int32_t) * (size_t)K : 0);
     if (!hyh::ok()) { return 0; }
     auto handed_out_defect = [&](const std::vector<double>& norm, int32_t ncols) -> double {
       std::vector<int32_t> order((size_t)ncols), mark((size_t)ncols, 0); std::iota(order.begin(), order.end(), 0);
@@ -131,13 +133,55 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
       return std::sqrt(cos2);
     };
     const double orthogonalTo = std::sqrt(eps);
+    /* When the values have settled and only the orthogonality of the vectors is short of its mark (a cluster of values that K
+     * cuts through: the sweeps bring its vectors apart slowly, and which basis of the cluster's span is handed out is
+     * immaterial), the columns that are handed out are made orthonormal directly instead of by further sweeps: normalised
+     * into a copy V and taken through V <- V (3 I - V^H V) / 2 (the Newton-Schulz step towards the orthonormal factor of V's
+     * polar decomposition: same span, so the same projection residual; a defect d becomes about d^2 per step).  At most two
+     * steps, then the largest cosine is measured again; if it is still above the mark the copy is dropped and the sweeps
+     * go on.  polished: the first `polishedCols` columns of `polished` are what is handed out, in the order `polishOrder`. */
+    int32_t cols = rank; double dropped2 = 0., droppedSpectral = 0.;
+    /* rank cut (reference: find_srank_kernel, src/gram_evd.cu:44-70): with the values in descending order (`order`), keep i < K
+     * while sum_{j>=i} sigma_j^2 > eps^2 sum_j sigma_j^2; the columns left out of the sweeps count with what they weigh (the sum
+     * over all values is the trace of G either way).  Returns how many are kept. */
+    auto rank_cut = [&](const std::vector<double>& value, std::vector<int32_t>& order) -> int32_t {
+      const int32_t n = (int32_t)value.size(); order.resize((size_t)n); std::iota(order.begin(), order.end(), 0);
+      std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return value[(size_t)a] > value[(size_t)b]; });
+      std::vector<double> suffix((size_t)n + 1, dropped2); for (int32_t i = n - 1; i >= 0; --i) { const double v = value[(size_t)order[(size_t)i]]; suffix[(size_t)i] = std::fma(v, v, suffix[(size_t)i + 1]); }
+      const double resid = eps * eps * suffix[0]; int32_t kept = 0;
+      for (int32_t i = 0; i < K && i < n; ++i) { if (resid < suffix[(size_t)i]) { ++kept; } }
+      return kept;
+    };
+    void* polished = nullptr; int32_t polishedCols = 0; std::vector<int32_t> polishOrder;
+    auto polish = [&](const std::vector<double>& norm, int32_t ncols) -> bool {
+      /* exactly the columns that the rank cut will hand out: a column made orthogonal to one that is then dropped would
+       * take a share of its direction out of the span */
+      const int32_t k = rank_cut(std::vector<double>(norm.begin(), norm.begin() + ncols), polishOrder); if (k < 2 || !polishA.p) { return false; }
+      HYH_CHECK(hipMemcpyAsync(dPolishOrder.p, polishOrder.data(), sizeof(int32_t) * (size_t)k, hipMemcpyHostToDevice, s));
+      void* cur = polishA.p; void* nxt = polishB.p;
+      HYH_KERNEL(hykBasisOut(s, N, k, Btype, Btype, B.p, sigma.as<double>(), dPolishOrder.as<int32_t>(), cur, N));   /* sigma holds the norms of the sweep just finished */
+      double cos2 = 1.;
+      for (int step = 0; step < 2 && hyh::ok(); ++step) {
+        HYH_KERNEL(hykGemm(s, 'C', 'N', k, k, N, 1., Btype, cur, N, cur, N, 0., gram.p, k));
+        HYH_KERNEL(hykMatcopy(s, 'A', N, k, Btype, cur, N, Btype, nxt, N));
+        HYH_KERNEL(hykGemm(s, 'N', 'N', N, k, k, -0.5, Btype, cur, N, gram.p, k, 1.5, nxt, N));
+        std::swap(cur, nxt);
+        HYH_KERNEL(hykGramWorkspaceClear(s, dOut.p, 64));
+        HYH_KERNEL(hykGemm(s, 'C', 'N', k, k, N, 1., Btype, cur, N, cur, N, 0., gram.p, k));
+        HYH_KERNEL(hykMaxDefect(s, Btype, k, gram.p, k, dOut.as<double>()));   /* every entry of V^H V - I, the diagonal included: a step leaves the norms off by about d^2 too */
+        HYH_CHECK(hipMemcpyAsync(&cos2, dOut.p, sizeof(double), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
+        if (!hyh::ok()) { return false; }
+        if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ: the %d columns that are handed out after orthonormalisation step %d: largest entry of V^H V - I %.2le\n", k, step + 1, std::sqrt(cos2)); }
+        if (std::sqrt(cos2) <= orthogonalTo) { polished = cur; polishedCols = k; return true; }
+      }
+      return false;
+    };
     /* Only the K largest values and their vectors are handed out.  Leaving the last rows of the Cholesky factor (the last
      * columns of B) out of the SVD takes a positive semidefinite matrix of trace tau (the sum of their squared norms) off
      * G: every eigenvalue moves down by at most tau, a singular value by at most tau / (2 sigma'), sigma' being the value
      * found without them.  The columns of a noise floor under the values that are wanted are not worth their rotations:
      * the prefix is picked from the column norms (choose_cut below), and what the sweeps then find must confirm it
      * (jacobi_truncation_holds_spectral with the values themselves), or columns are taken back in. */
-    int32_t cols = rank; double dropped2 = 0., droppedSpectral = 0.;
     /* The cut for given budgets: the longest tail [t, rank), t >= atLeast, that passes the trace rule or the sharper rule
      * (jacobi_columns_needed_spectral: what moves a value is the largest eigenvalue of the Gram matrix of the columns left
      * out, which for the rows of a noise floor is a small part of their trace).  The Gram matrix is formed once, for the
@@ -202,6 +246,8 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
             const double defect = handed_out_defect(after, cols); if (!hyh::ok()) { return 0; }
             if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: largest cosine among the columns that can be handed out %.2le (wanted: %.2le)\n", used, defect, orthogonalTo); }
             if (defect <= orthogonalTo) { break; }
+            if (defect <= 0.25 && polish(after, cols)) { break; }
+            if (!hyh::ok()) { return 0; }
           }
         }
         lastCosine2 = seen.cosine2; before.swap(after);
@@ -217,6 +263,7 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
        * that the values found allow (the columns taken back in are the unrotated ones next to the cut; the others stay as the
        * sweeps left them); should that fail too, the sweeps go on with all columns. */
       if (unfactored > 0. && !hyh::jacobi_truncation_holds_spectral(unfactored, unfactored, sigma1, sigmaK, outside2, eps)) { again = true; break; }   /* no cut of the rows at hand can make up for the rows that were never factored */
+      polished = nullptr; polishedCols = 0;   /* (it held columns of a cut that did not stand) */
       const int32_t had = cols;
       if (!recut) { recut = true; choose_cut(0.5 * hyh::kTruncationBudget * eps * sigma1 * sigmaK, outside2 / 128., had); } else { cols = rank; dropped2 = droppedSpectral = unfactored; }
       if (cols <= had) { cols = rank; dropped2 = droppedSpectral = unfactored; }
@@ -227,20 +274,17 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
       if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ: what the Cholesky left unfactored (%.2le) weighs too much against the values found: factoring again, in full\n", unfactored); }
       continue;
     }
-    std::vector<int32_t> order((size_t)cols); std::iota(order.begin(), order.end(), 0);
-    std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return sig[a] > sig[b]; });
-    /* rank cut (reference: find_srank_kernel, src/gram_evd.cu:44-70): keep i < K while sum_{j>=i} sigma_j^2 > eps^2 sum_j sigma_j^2;
-     * the columns left out count with what they weigh (the sum over all values is the trace of G either way) */
-    std::vector<double> suffix((size_t)cols + 1, dropped2); for (int32_t i = cols - 1; i >= 0; --i) { const double v = sig[order[i]]; suffix[i] = std::fma(v, v, suffix[i + 1]); }
-    const double resid = eps * eps * suffix[0]; std::vector<double> Sout((size_t)K, 0.); int32_t kept = 0;
-    for (int32_t i = 0; i < K; ++i) { if (i < cols && resid < suffix[i]) { Sout[i] = sig[order[i]]; ++kept; } }
+    std::vector<int32_t> order; const int32_t kept = rank_cut(sig, order);
+    std::vector<double> Sout((size_t)K, 0.); for (int32_t i = 0; i < kept; ++i) { Sout[(size_t)i] = sig[(size_t)order[(size_t)i]]; }
     const int32_t svdRank = kept; rank = std::min(rank, kept);
     hyh::Scratch dS(handle, sizeof(double) * (size_t)K), dOrder(handle, sizeof(int32_t) * (size_t)std::max(1, rank));
     if (!hyh::ok()) { return 0; }
     HYH_CHECK(hipMemcpyAsync(dS.p, Sout.data(), sizeof(double) * (size_t)K, hipMemcpyHostToDevice, s));
     if (rank > 0) { HYH_CHECK(hipMemcpyAsync(dOrder.p, order.data(), sizeof(int32_t) * (size_t)rank, hipMemcpyHostToDevice, s)); }
     HYH_KERNEL(hykValuesOut(s, K, (int32_t)Atype, dS.as<double>(), S));
-    if (rank > 0) { HYH_KERNEL(hykBasisOut(s, N, rank, (int32_t)Atype, Btype, B.p, sigma.as<double>(), dOrder.as<int32_t>(), X, ldx)); }
+    if (polished && !(rank == polishedCols && std::equal(order.begin(), order.begin() + rank, polishOrder.begin()))) { polished = nullptr; }   /* (the norms are those of the sweep the copy was made after, so cut and order agree) */
+    if (rank > 0 && polished) { HYH_KERNEL(hykMatcopy(s, 'A', N, rank, Btype, polished, N, (int32_t)Atype, X, ldx)); }
+    else if (rank > 0) { HYH_KERNEL(hykBasisOut(s, N, rank, (int32_t)Atype, Btype, B.p, sigma.as<double>(), dOrder.as<int32_t>(), X, ldx)); }
     HYH_CHECK(hipStreamSynchronize(s));   /* Sout / order are host temporaries */
     if (!hyh::ok()) { return 0; }
     if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ-%s [eps=%.1le] [M=%d] [N=%d] [K=%d] [sweeps=%d] [SVD-rank=%d]\n", wideB ? (Complex ? "FP64-COMPLEX" : "FP64") : (Complex ? "FP32-COMPLEX" : "FP32"), eps, N, rank, K, used, svdRank); }

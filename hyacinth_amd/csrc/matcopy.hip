@@ -91,7 +91,6 @@ extern "C" int hykMatcopy(hipStream_t stream, char mode, int64_t M, int64_t N, i
   }
 }
 
-/* *out += sum of squares of the M x N FP64 matrix (a complex matrix is passed as 2M x N) */
 /* G[y, x] = conj(G[x, y]) for y < x: the strict upper triangle of a Hermitian matrix written again from its lower one.
  * W doubles per real or imaginary part (1: FP64, 2: double-double).  A thread per entry, adjacent threads along y. */
 template <int W, bool CPLX>
@@ -118,6 +117,7 @@ extern "C" int hykMirrorLower(hipStream_t stream, int32_t N, int32_t Gtype, void
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
+/* *out += sum of squares of the M x N FP64 matrix (a complex matrix is passed as 2M x N) */
 extern "C" int hykSumSquares(hipStream_t stream, int64_t M, int64_t N, const double* A, int64_t lda, double* out) {
   if (M <= 0 || N <= 0) { return 0; }
   dim3 grid((uint32_t)((M + 255) / 256 < 64 ? (M + 255) / 256 : 64), (uint32_t)(N < 256 ? N : 256));

@@ -178,11 +178,17 @@ extern "C" int hykColumnNorms(hipStream_t stream, int32_t Btype, int32_t N, int3
 
 /* the largest squared cosine among the marked columns, from their Gram matrix: G column-major n x n (complex interleaved),
  * mark[p] != 0 for the columns that count; out: one double, zero before the call, raised by an integer maximum on its bits */
-template <bool CPLX, typename GT>
+/* DEFECT: the largest |G[p, q] - delta_pq|^2 over all p <= q instead (how far columns that should be orthonormal are from it; no marks) */
+template <bool CPLX, typename GT, bool DEFECT = false>
 __global__ __launch_bounds__(T_THREADS) void max_cosine_kernel(int32_t n, const GT* __restrict__ G, int64_t ldg, const int32_t* __restrict__ mark, double* __restrict__ out) {
   __shared__ double scratch[T_THREADS / 64]; constexpr int W = CPLX ? 2 : 1;
   const int q = blockIdx.x; double worst = 0.;
-  if (mark[q]) {
+  if constexpr (DEFECT) {
+    for (int p = threadIdx.x; p <= q; p += T_THREADS) {
+      const GT* g = &G[((int64_t)p + (int64_t)q * ldg) * W]; const double g0 = (double)g[0] - (p == q ? 1. : 0.); double g2 = g0 * g0; if constexpr (CPLX) { const double g1 = g[1]; g2 = fma(g1, g1, g2); }
+      worst = fmax(worst, g2);
+    }
+  } else if (mark[q]) {
     const double gqq = G[((int64_t)q + (int64_t)q * ldg) * W];
     for (int p = threadIdx.x; p < q; p += T_THREADS) {
       if (!mark[p]) { continue; }
@@ -205,6 +211,15 @@ extern "C" int hykMaxCosine(hipStream_t stream, int32_t Gtype, int32_t n, const 
   const bool Complex = Gtype & 1;
   if ((Gtype & ~1) == HYK_F32) { if (Complex) { max_cosine_kernel<true, float><<<n, T_THREADS, 0, stream>>>(n, (const float*)G, ldg, mark, out); } else { max_cosine_kernel<false, float><<<n, T_THREADS, 0, stream>>>(n, (const float*)G, ldg, mark, out); } }
   else if (Complex) { max_cosine_kernel<true, double><<<n, T_THREADS, 0, stream>>>(n, (const double*)G, ldg, mark, out); } else { max_cosine_kernel<false, double><<<n, T_THREADS, 0, stream>>>(n, (const double*)G, ldg, mark, out); }
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
+extern "C" int hykMaxDefect(hipStream_t stream, int32_t Gtype, int32_t n, const void* G, int64_t ldg, double* out) {
+  if (n <= 0) { return 0; }
+  if (ldg < n || !btype_ok(Gtype)) { return -1; }
+  const bool Complex = Gtype & 1;
+  if ((Gtype & ~1) == HYK_F32) { if (Complex) { max_cosine_kernel<true, float, true><<<n, T_THREADS, 0, stream>>>(n, (const float*)G, ldg, nullptr, out); } else { max_cosine_kernel<false, float, true><<<n, T_THREADS, 0, stream>>>(n, (const float*)G, ldg, nullptr, out); } }
+  else if (Complex) { max_cosine_kernel<true, double, true><<<n, T_THREADS, 0, stream>>>(n, (const double*)G, ldg, nullptr, out); } else { max_cosine_kernel<false, double, true><<<n, T_THREADS, 0, stream>>>(n, (const double*)G, ldg, nullptr, out); }
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 

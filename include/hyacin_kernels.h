@@ -174,6 +174,9 @@ int hykColumnNorms(hipStream_t stream, int32_t Btype, int32_t N, int32_t r, cons
  * HYK_F32 / HYK_F32C, complex interleaved), mark[p] != 0 selects the columns that count; *out (device, zero before the call) receives the largest
  * |G[p, q]|^2 / (G[p, p] G[q, q]) over the marked pairs p < q. */
 int hykMaxCosine(hipStream_t stream, int32_t Gtype, int32_t n, const void* G, int64_t ldg, const int32_t* mark, double* out);
+/* How far n columns are from orthonormal, from their Gram matrix (same types): *out (device, zero before the call) receives
+ * the largest |G[p, q] - delta_pq|^2 over p <= q.  No counterpart in the reference. */
+int hykMaxDefect(hipStream_t stream, int32_t Gtype, int32_t n, const void* G, int64_t ldg, double* out);
 int hykBasisOut(hipStream_t stream, int32_t N, int32_t rank, int32_t Atype, int32_t Btype, const void* B, const double* sigma, const int32_t* order, void* X, int64_t ldx);
 int hykValuesOut(hipStream_t stream, int32_t K, int32_t Atype, const double* S, void* out);
 

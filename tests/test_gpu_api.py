@@ -359,6 +359,40 @@ def test_fit_hands_out_orthogonal_vectors(env, at):
     assert defect <= max(np.sqrt(eps), 1e-5 if at >= 2 else 0.0)
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_orthonormalised_vectors_keep_their_span(env, seed, capfd, monkeypatch):
+    """A fit whose values settle before its vectors are orthogonal and whose energy cut hands out fewer than K vectors (nearly
+    all columns wanted, the last few below the cut).  The vectors are then made orthonormal directly (the log says so), and
+    that has to happen to exactly the vectors that are handed out: orthonormalised together with vectors that are dropped
+    afterwards they would carry a share of those directions and lose as much of their own, which shows as a projection
+    residual far above the oracle's (complex FP64 at eps = 1e-13: 6e-22 against 2e-26 when it went wrong)."""
+    from oracle import ho as oracle
+    from util import as_complex
+    ha, h = env
+    rng = np.random.default_rng(600 + seed)
+    M, N, K, eps = 2267, 373, 364, 8.9e-14
+    A0, _ = low_rank(rng, M, N, 0.68, cplx=True, noise=eps * 1e-2)
+    A = to_storage(A0, 1)
+    monkeypatch.setenv("HYACIN_VERBOSE", "1")
+    h2 = ha.create_handle(stream=h.hipStream)
+    try:
+        capfd.readouterr()
+        rank, S, V, err, nrm = run_tsvd((ha, h2), A, eps, K, "C")
+        C.CDLL(None).fflush(None)
+        log = capfd.readouterr().out
+    finally:
+        ha.destroy_handle(h2)
+    r_o, S_o, V_o, g = oracle.tsvd_fit(A, eps, K)
+    k = min(rank, r_o)
+    print("rank", rank, "oracle", r_o, "orthonormalised" if "after orthonormalisation step" in log else "by sweeps alone", flush=True)
+    assert 0 < rank < K and abs(rank - r_o) <= 4
+    assert "after orthonormalisation step" in log
+    Ac = as_complex(A).astype(np.complex128)
+    mine, ref = oracle.check_norm(Ac, V), oracle.check_norm(Ac, V_o[:, :k])
+    assert mine <= 2 * ref + (100 * eps * S_o[0]) ** 2, (mine, ref)
+    assert np.abs(V[:, :rank].conj().T @ V[:, :rank] - np.eye(rank)).max() <= 2 * np.sqrt(eps)
+
+
 @pytest.mark.parametrize("at,eps", [(0, 1e-12), (1, 1e-9), (2, 1e-5)])
 def test_fit_with_global_rows(env, at, eps):
     """globalM above M (the rows of other devices, include/hyacin.h:67-113): the integer Gram gets the head-room of

@@ -228,3 +228,38 @@ def test_max_cosine(L, cplx, n, pad, wide):
     got = host(out, np.float64)[0]
     assert abs(got - want) <= 1e-12 * want
     assert L.hykMaxCosine(stream(), (0 if wide else 2) + cplx, n, ptr(dG), n - 1, ptr(dM), ptr(out)) == -1
+
+
+@pytest.mark.parametrize("cplx", [0, 1])
+@pytest.mark.parametrize("wide", [1, 0])
+@pytest.mark.parametrize("n,pad", [(1, 0), (37, 3), (300, 0)])
+def test_max_defect(L, cplx, n, pad, wide):
+    """hykMaxDefect: the largest |G[p, q] - delta_pq|^2 over p <= q of the Gram matrix of nearly orthonormal columns, against
+    numpy; once with the largest entry on the diagonal (a column whose norm is off), once off it."""
+    from gpu_util import dev, zeros, ptr, stream, sync, host
+    rng = np.random.default_rng(75 + n)
+    for where in ("diagonal", "off"):
+        Q, _ = np.linalg.qr(rng.standard_normal((2 * n + 3, n)) + (1j * rng.standard_normal((2 * n + 3, n)) if cplx else 0))
+        X = Q + 1e-3 * (rng.standard_normal(Q.shape) + (1j * rng.standard_normal(Q.shape) if cplx else 0)) / np.sqrt(Q.shape[0])
+        if where == "diagonal":
+            X[:, n // 2] *= 1.01
+        elif n > 1:
+            X[:, 0] += 0.02 * X[:, n - 1]
+        G = X.conj().T @ X
+        ld = n + pad
+        buf = np.full((n, ld, 2) if cplx else (n, ld), np.nan, np.float64 if wide else np.float32)   # [column][row]
+        if cplx:
+            buf[:, :n, 0] = G.real.T
+            buf[:, :n, 1] = G.imag.T
+        else:
+            buf[:, :n] = G.T
+        dG, out = dev(buf), zeros(8)
+        assert L.hykMaxDefect(stream(), (0 if wide else 2) + cplx, n, ptr(dG), ld, ptr(out)) == 0
+        sync()
+        if not wide:                                                # what the kernel saw
+            G = (buf[:, :n, 0] + 1j * buf[:, :n, 1]).T.astype(np.complex128) if cplx else buf[:, :n].T.astype(np.float64)
+        want = (np.abs(np.triu(G - np.eye(n)).T) ** 2).max()        # entries p <= q (column q, row p)
+        got = host(out, np.float64)[0]
+        assert abs(got - want) <= 1e-12 * want
+        assert (np.argmax(np.abs(G - np.eye(n))) % (n + 1) == 0) == (where == "diagonal" or n == 1)
+    assert L.hykMaxDefect(stream(), (0 if wide else 2) + cplx, 5, ptr(dG), 4, ptr(out)) == -1
