@@ -37,12 +37,18 @@ inline bool jacobi_sweeps_done(int rotations, double cosine2, double lastCosine2
  * its singular value squared.  So the iteration may end after a sweep in which
  *   (i)  no kept value moved by more than eps sigma_max / 4, and
  *   (ii) the kept columns gained at most 1 / 32 of what is left outside them (the residual bound has stopped improving).
+ * (i) also counts as met one sweep early when the iteration is visibly in its fast phase: lastMoved is what the kept values
+ * moved by in the sweep before (0: unknown); if this sweep's move is at most 1 / 64 of it and, shrunk once more by no more
+ * than the same ratio (the method contracts faster from sweep to sweep there, so this overstates the next move: by two
+ * orders of magnitude where it was watched), stays within the same eps sigma_max / 4, the sweep that would only confirm it
+ * is not run: the values are already as far from their
+ * limits as that next move.
  * A noise floor of hundreds of nearly equal small columns, which a cyclic Jacobi method needs ten and more sweeps to resolve
  * and which is never handed out, then no longer decides when the sweeps end.  With nothing left outside (kept = all columns
  * and a zero cut) rule (ii) never holds and the rules above decide alone.
  * before / after: the column norms (not squared) at the start and at the end of the sweep, in the same column order.
  * seen (optional): { largest move of a kept value, what the kept columns gained, what is left outside } for the log. */
-inline bool jacobi_output_settled(const std::vector<double>& before, const std::vector<double>& after, int kept, double eps, double* seen = nullptr) {
+inline bool jacobi_output_settled(const std::vector<double>& before, const std::vector<double>& after, int kept, double eps, double* seen = nullptr, double lastMoved = 0.) {
   const size_t r = after.size(); if (before.size() != r || r == 0 || kept <= 0 || (size_t)kept >= r) { return false; }
   std::vector<double> a(before), b(after);
   std::sort(a.begin(), a.end(), std::greater<double>()); std::sort(b.begin(), b.end(), std::greater<double>());
@@ -51,7 +57,8 @@ inline bool jacobi_output_settled(const std::vector<double>& before, const std::
   for (size_t i = r; i-- > (size_t)kept;) { outsideBefore += a[i] * a[i]; outsideAfter += b[i] * b[i]; }
   const double gained = outsideBefore - outsideAfter;
   if (seen) { seen[0] = moved; seen[1] = gained; seen[2] = outsideAfter; }
-  return moved <= 0.25 * eps * b[0] && gained <= outsideAfter / 32.;
+  const bool still = moved <= 0.25 * eps * b[0] || (lastMoved > 0. && moved <= lastMoved / 64. && moved * (moved / lastMoved) <= 0.25 * eps * b[0]);
+  return still && gained <= outsideAfter / 32.;
 }
 
 /* The columns whose pairs the caller waits for: one past the last index among the `kept` largest column norms.  Pairs of two

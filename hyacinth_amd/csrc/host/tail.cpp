@@ -225,7 +225,7 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
     }
     bool recut = false;
     for (;;) {
-      double lastCosine2 = 0.;
+      double lastCosine2 = 0., lastMoved = 0.;
       const bool watchOutput = K < cols;   /* with every column handed out only the cosines can end the sweeps */
       for (int32_t sw = 0; sw < maxSweeps && cols > 1; ++sw) {
         const int32_t top = watchOutput ? hyh::jacobi_tail_start(before, K, eps) : cols;   /* a broad floor of small columns is left alone */
@@ -240,7 +240,7 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
         if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: %d rotations, largest cosine %.2le among pairs with a column before %d%s\n", used, seen.rotations, std::sqrt(seen.cosine2), headCols, top < cols ? " (floor of small columns left alone)" : ""); }
         if (hyh::jacobi_sweeps_done(seen.rotations, seen.cosine2, lastCosine2, rotateAbove)) { break; }
         if (watchOutput) {
-          double moved[3] = { 0., 0., 0. }; const bool settled = hyh::jacobi_output_settled(before, after, K, eps, moved);
+          double moved[3] = { 0., 0., 0. }; const bool settled = hyh::jacobi_output_settled(before, after, K, eps, moved, lastMoved); lastMoved = moved[0];
           if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: the %d values handed out moved by at most %.2le, their columns gained %.2le of %.2le outside%s\n", used, K, moved[0], moved[1], moved[2], settled ? ": settled" : ""); }
           if (settled) {
             const double defect = handed_out_defect(after, cols); if (!hyh::ok()) { return 0; }

@@ -97,6 +97,7 @@ int hm_jacobi_done(int rotations, double cosine2, double lastCosine2, double rot
 /* ... and for ending them when what is handed out has settled */
 int hm_jacobi_tail_start(const double* norm, int r, int K, double eps) { return hyh::jacobi_tail_start(std::vector<double>(norm, norm + r), K, eps); }
 int hm_jacobi_settled(const double* before, const double* after, int r, int kept, double eps) { return hyh::jacobi_output_settled(std::vector<double>(before, before + r), std::vector<double>(after, after + r), kept, eps) ? 1 : 0; }
+int hm_jacobi_settled_after(const double* before, const double* after, int r, int kept, double eps, double lastMoved) { return hyh::jacobi_output_settled(std::vector<double>(before, before + r), std::vector<double>(after, after + r), kept, eps, nullptr, lastMoved) ? 1 : 0; }
 int hm_jacobi_columns_needed(const double* norm, int r, int K, double eps) { return hyh::jacobi_columns_needed(std::vector<double>(norm, norm + r), K, eps); }
 int hm_jacobi_truncation_holds(double dropped2, double sigma1, double sigmaK, double eps) { return hyh::jacobi_truncation_holds(dropped2, sigma1, sigmaK, eps) ? 1 : 0; }
 int hm_jacobi_columns_needed_spectral(const double* absGram, int r, int c0, int K, double valueBudget, double residualBudget, double* traceOut, double* spectralOut) {

@@ -334,7 +334,7 @@ def test_gevd_leaves_out_floor_columns(case, gtype, capfd, monkeypatch):
     # estimate of the budget), the values found refute the estimate, and the matrix is factored again in full
     assert ("POTRFP: ended after" in log and "factoring again, in full" in log) == (case == "floor taken back in")
     assert 0 < rank <= K and np.abs(S[:rank] - want[:rank]).max() <= 10 * eps * want[0]
-    assert np.abs(X @ X.T - np.eye(rank)).max() <= max(1e-12, eps)            # rotations stop at cosines of eps / 16
+    assert np.abs(X @ X.T - np.eye(rank)).max() <= max(1e-12, np.sqrt(eps))   # what is guaranteed with K below the factor's rank (the sweeps may end on the values)
     if case == "floor taken back in":
         assert rank >= 23 and abs(S[rank - 1] - want[rank - 1]) <= 1e-11 and (rank < 24 or abs(S[23] - 1e-5) <= 1e-11)
     # the basis captures the matrix up to the values that are not handed out

@@ -239,6 +239,21 @@ def test_jacobi_output_settled_rule(hm):
     # a flat floor that keeps mixing (its norms move among themselves, their sum stays) does not hold the end back
     floor = np.concatenate([s[:10], np.full(30, 1e-9)]); mixed = floor.copy(); mixed[10:] = 1e-9 * np.sqrt(np.linspace(0.5, 1.5, 30))
     assert abs((mixed[10:] ** 2).sum() - (floor[10:] ** 2).sum()) < 1e-30 and settled(floor, mixed, 10, 1e-12) == 1
+    # one sweep early in the fast phase: this sweep moved the values by 2.4e-12 (above eps sigma_max / 4 = 2.5e-13) after 3.7e-8
+    # in the sweep before: contraction 6.5e-5, the next move at that rate 1.6e-16 <= eps sigma_max / 4
+    hm.hm_jacobi_settled_after.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_double, C.c_double]
+    hm.hm_jacobi_settled_after.restype = C.c_int
+    def after_move(before, after, kept, eps, last):
+        a, b = np.ascontiguousarray(before, dtype=np.float64), np.ascontiguousarray(after, dtype=np.float64)
+        return hm.hm_jacobi_settled_after(_p(a), _p(b), len(b), kept, eps, last)
+    moved = s.copy(); moved[3] += 2.4e-12
+    assert settled(s, moved, 10, 1e-12) == 0 and after_move(s, moved, 10, 1e-12, 0.0) == 0
+    assert after_move(s, moved, 10, 1e-12, 3.7e-8) == 1
+    assert after_move(s, moved, 10, 1e-12, 1e-10) == 0                               # contraction 1 / 42 only: not the fast phase
+    moved = s.copy(); moved[3] += 4e-9
+    assert after_move(s, moved, 10, 1e-12, 1e-6) == 0                                # fast (1 / 250), but the next move at that rate, 1.6e-11, is too large
+    out = s.copy(); out[3] += 2.4e-12; out[10:] *= 0.9
+    assert after_move(s, out, 10, 1e-12, 3.7e-8) == 0                                # the other condition still has to hold
 
 
 def test_jacobi_head(hm):
