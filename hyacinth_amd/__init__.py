@@ -34,7 +34,7 @@ KERNEL_SYMBOLS = [
     "hykGramProfile", "hykGramProfileRead", "hykMfmaCeiling", "hykGramRange", "hykDequantize", "hykPotrfpWorkspaceBytes", "hykPotrfp", "hykPotrfpLeftLooking", "hykPotrfpWanted", "hykMirrorLower", "hykPotrfpSetPlainLaunch", "hykPotrfpStaticMaxN", "hykPotrfpStatic", "hykFactorToB", "hykJacobiSweep", "hykJacobiSweepCarry", "hykJacobiSweepTop", "hykJacobiCarryBytes", "hykJacobiSetVariant", "hykJacobiSetSplitTest",
     "hykColumnNorms", "hykBasisOut", "hykValuesOut", "hykInterpSolve", "hykInterpOut", "hykMatcopy",
     "hykSumSquares", "hykMatmulCf16", "hykGemm", "hykOrthonormalize", "hykLastStatus", "hykTestFailAllocation", "hykColumnExponentsOp", "hykQuantizeLimbsOp", "hykQuantizeCrtOp",
-    "hykQuantizeScaleBatchOp", "hykHerkBatchOp", "hykLastHerkPlan", "hykMaxCosine", "hykMaxDefect",
+    "hykQuantizeScaleBatchOp", "hykHerkBatchOp", "hykLastHerkPlan", "hykMaxCosine", "hykMaxDefect", "hykNewtonSchulzFactor",
 ]
 
 
@@ -123,6 +123,7 @@ def lib():
         L.hykQuantizeCrtOp.argtypes = [vp, ch, i32, i32, i32, i32, vp, i64, vp, vp, i64, i32]
         L.hykMaxCosine.argtypes = [vp, i32, i32, vp, i64, vp, vp]
         L.hykMaxDefect.argtypes = [vp, i32, i32, vp, i64, vp]
+        L.hykNewtonSchulzFactor.argtypes = [vp, i32, i32, vp, i64]
         L.hykQuantizeScaleBatchOp.argtypes = [HP, ch, i32, i32, i32, i32, i32, vp, i64, i32, vp]; L.hykQuantizeScaleBatchOp.restype = None
         L.hykHerkBatchOp.argtypes = [HP, ch, i32, i32, i32, i32, i32, vp, i64, i32, vp, i32, i32, vp]; L.hykHerkBatchOp.restype = None
         L.hykLastHerkPlan.argtypes = [C.POINTER(HerkPlan)]

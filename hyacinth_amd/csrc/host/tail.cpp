@@ -105,41 +105,19 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
       HYH_KERNEL(hykColumnNorms(s, Btype, N, cols, B.p, sigma.as<double>()));
       HYH_CHECK(hipMemcpyAsync(v.data(), sigma.p, sizeof(double) * (size_t)cols, hipMemcpyDeviceToHost, s));
     };
-    /* How far the columns that can be handed out (the K largest norms) are from orthogonal: the largest cosine among them,
-     * from their Gram matrix.  The sweeps may end on the values alone (jacobi_output_settled), which settle with the square
-     * of what the vectors still lack: singular values 2 % apart leave their vectors several per cent away from orthogonal
-     * when the values have long stopped moving.  What is handed out as singular vectors is held to sqrt(eps): the
-     * projector V V^H is then right to eps. */
-    /* (its scratch -- the Gram matrix of the columns, the marks, the result word -- is taken once, before the sweeps: whether a
-     * sweep ends "settled" depends on the data, and an allocation in the middle of the loop would make the calls that can
-     * fail depend on it too; needed only when fewer values are handed out than the factor has columns) */
+    /* The sweeps may end on the values alone (jacobi_output_settled), which settle with the square of what the vectors still
+     * lack: singular values 2 % apart leave their vectors several per cent away from orthogonal when the values have long
+     * stopped moving.  What is handed out as singular vectors is held to sqrt(eps) in every entry of V^H V - I: the
+     * projector V V^H is then right to eps.
+     * (The scratch for that -- a Gram matrix, two copies of the vectors, their order, the result word -- is taken once, before
+     * the sweeps: whether a sweep ends "settled" depends on the data, and an allocation in the middle of the loop would make
+     * the calls that can fail depend on it too; needed only when fewer values are handed out than the factor has columns.) */
     const bool mayCheck = K < rank && rank > 1;
     const size_t elemB = (size_t)(wideB ? 8 : 4) * (1 + Complex);
-    hyh::Scratch gram(handle, mayCheck ? (size_t)rank * rank * elemB : 0), dMark(handle, mayCheck ? sizeof(int32_t) * (size_t)rank : 0), dOut(handle, mayCheck ? 64 : 0);
+    hyh::Scratch gram(handle, mayCheck ? (size_t)rank * rank * elemB : 0), dOut(handle, mayCheck ? 64 : 0);
     hyh::Scratch polishA(handle, mayCheck ? (size_t)N * K * elemB : 0), polishB(handle, mayCheck ? (size_t)N * K * elemB : 0), dPolishOrder(handle, mayCheck ? sizeof(int32_t) * (size_t)K : 0);
     if (!hyh::ok()) { return 0; }
-    auto handed_out_defect = [&](const std::vector<double>& norm, int32_t ncols) -> double {
-      std::vector<int32_t> order((size_t)ncols), mark((size_t)ncols, 0); std::iota(order.begin(), order.end(), 0);
-      const int32_t kept = std::min(K, ncols);
-      std::nth_element(order.begin(), order.begin() + (kept - 1), order.end(), [&](int32_t a, int32_t b) { return norm[(size_t)a] > norm[(size_t)b]; });
-      for (int32_t i = 0; i < kept; ++i) { mark[(size_t)order[(size_t)i]] = 1; }
-      if (!gram.p || !hyh::ok()) { return 0.; }
-      double cos2 = 0.;
-      HYH_CHECK(hipMemcpyAsync(dMark.p, mark.data(), sizeof(int32_t) * (size_t)ncols, hipMemcpyHostToDevice, s));
-      HYH_KERNEL(hykGramWorkspaceClear(s, dOut.p, 64));
-      HYH_KERNEL(hykGemm(s, 'C', 'N', ncols, ncols, N, 1., Btype, B.p, N, B.p, N, 0., gram.p, ncols));
-      HYH_KERNEL(hykMaxCosine(s, Btype, ncols, gram.p, ncols, dMark.as<int32_t>(), dOut.as<double>()));
-      HYH_CHECK(hipMemcpyAsync(&cos2, dOut.p, sizeof(double), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
-      return std::sqrt(cos2);
-    };
     const double orthogonalTo = std::sqrt(eps);
-    /* When the values have settled and only the orthogonality of the vectors is short of its mark (a cluster of values that K
-     * cuts through: the sweeps bring its vectors apart slowly, and which basis of the cluster's span is handed out is
-     * immaterial), the columns that are handed out are made orthonormal directly instead of by further sweeps: normalised
-     * into a copy V and taken through V <- V (3 I - V^H V) / 2 (the Newton-Schulz step towards the orthonormal factor of V's
-     * polar decomposition: same span, so the same projection residual; a defect d becomes about d^2 per step).  At most two
-     * steps, then the largest cosine is measured again; if it is still above the mark the copy is dropped and the sweeps
-     * go on.  polished: the first `polishedCols` columns of `polished` are what is handed out, in the order `polishOrder`. */
     int32_t cols = rank; double dropped2 = 0., droppedSpectral = 0.;
     /* rank cut (reference: find_srank_kernel, src/gram_evd.cu:44-70): with the values in descending order (`order`), keep i < K
      * while sum_{j>=i} sigma_j^2 > eps^2 sum_j sigma_j^2; the columns left out of the sweeps count with what they weigh (the sum
@@ -152,29 +130,37 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
       for (int32_t i = 0; i < K && i < n; ++i) { if (resid < suffix[(size_t)i]) { ++kept; } }
       return kept;
     };
+    /* Once the values have settled, the vectors that will be handed out (the rank cut applied to the norms as they are) are
+     * normalised into a copy V and every entry of V^H V - I is measured.  Within sqrt(eps): done.  Short of that by a
+     * cluster of values that K cuts through (the sweeps bring its vectors apart slowly, and which basis of the cluster's
+     * span is handed out is immaterial): V is made orthonormal directly, V <- V (3 I - V^H V) / 2 (the Newton-Schulz step
+     * towards the orthonormal factor of V's polar decomposition: same span, so the same projection residual; a defect d
+     * becomes about d^2 per step), at most two steps, measured again after each.  It has to be exactly the vectors that are
+     * handed out: a vector made orthogonal to one that is then dropped would carry a share of that direction and lose as
+     * much of its own.  Returns 0: not orthogonal, the sweeps go on; 1: orthogonal as the columns are; 2: the first
+     * `polishedCols` columns of `polished` are what is handed out, in the order `polishOrder`. */
     void* polished = nullptr; int32_t polishedCols = 0; std::vector<int32_t> polishOrder;
-    auto polish = [&](const std::vector<double>& norm, int32_t ncols) -> bool {
-      /* exactly the columns that the rank cut will hand out: a column made orthogonal to one that is then dropped would
-       * take a share of its direction out of the span */
-      const int32_t k = rank_cut(std::vector<double>(norm.begin(), norm.begin() + ncols), polishOrder); if (k < 2 || !polishA.p) { return false; }
+    auto orthonormal = [&](const std::vector<double>& norm, int32_t ncols) -> int {
+      const int32_t k = rank_cut(std::vector<double>(norm.begin(), norm.begin() + ncols), polishOrder); if (k < 2 || !polishA.p) { return 1; }
       HYH_CHECK(hipMemcpyAsync(dPolishOrder.p, polishOrder.data(), sizeof(int32_t) * (size_t)k, hipMemcpyHostToDevice, s));
       void* cur = polishA.p; void* nxt = polishB.p;
       HYH_KERNEL(hykBasisOut(s, N, k, Btype, Btype, B.p, sigma.as<double>(), dPolishOrder.as<int32_t>(), cur, N));   /* sigma holds the norms of the sweep just finished */
-      double cos2 = 1.;
-      for (int step = 0; step < 2 && hyh::ok(); ++step) {
-        HYH_KERNEL(hykGemm(s, 'C', 'N', k, k, N, 1., Btype, cur, N, cur, N, 0., gram.p, k));
-        HYH_KERNEL(hykMatcopy(s, 'A', N, k, Btype, cur, N, Btype, nxt, N));
-        HYH_KERNEL(hykGemm(s, 'N', 'N', N, k, k, -0.5, Btype, cur, N, gram.p, k, 1.5, nxt, N));
-        std::swap(cur, nxt);
+      for (int step = 0; step <= 2 && hyh::ok(); ++step) {
+        double defect2 = 1.;
         HYH_KERNEL(hykGramWorkspaceClear(s, dOut.p, 64));
         HYH_KERNEL(hykGemm(s, 'C', 'N', k, k, N, 1., Btype, cur, N, cur, N, 0., gram.p, k));
-        HYH_KERNEL(hykMaxDefect(s, Btype, k, gram.p, k, dOut.as<double>()));   /* every entry of V^H V - I, the diagonal included: a step leaves the norms off by about d^2 too */
-        HYH_CHECK(hipMemcpyAsync(&cos2, dOut.p, sizeof(double), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
-        if (!hyh::ok()) { return false; }
-        if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ: the %d columns that are handed out after orthonormalisation step %d: largest entry of V^H V - I %.2le\n", k, step + 1, std::sqrt(cos2)); }
-        if (std::sqrt(cos2) <= orthogonalTo) { polished = cur; polishedCols = k; return true; }
+        HYH_KERNEL(hykMaxDefect(s, Btype, k, gram.p, k, dOut.as<double>()));   /* the diagonal included: a step leaves the norms off by about d^2 too */
+        HYH_CHECK(hipMemcpyAsync(&defect2, dOut.p, sizeof(double), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
+        if (!hyh::ok()) { return 0; }
+        const double defect = std::sqrt(defect2);
+        if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: the %d vectors to be handed out%s: largest entry of V^H V - I %.2le (wanted: %.2le)\n", used, k, step ? " after an orthonormalisation step" : "", defect, orthogonalTo); }
+        if (defect <= orthogonalTo) { if (step == 0) { return 1; } polished = cur; polishedCols = k; return 2; }
+        if (defect > 0.25 || step == 2) { return 0; }
+        HYH_KERNEL(hykNewtonSchulzFactor(s, Btype, k, gram.p, k));
+        HYH_KERNEL(hykGemm(s, 'N', 'N', N, k, k, 1., Btype, cur, N, gram.p, k, 0., nxt, N));
+        std::swap(cur, nxt);
       }
-      return false;
+      return 0;
     };
     /* Only the K largest values and their vectors are handed out.  Leaving the last rows of the Cholesky factor (the last
      * columns of B) out of the SVD takes a positive semidefinite matrix of trace tau (the sum of their squared norms) off
@@ -243,11 +229,8 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
           double moved[3] = { 0., 0., 0. }; const bool settled = hyh::jacobi_output_settled(before, after, K, eps, moved, lastMoved); lastMoved = moved[0];
           if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: the %d values handed out moved by at most %.2le, their columns gained %.2le of %.2le outside%s\n", used, K, moved[0], moved[1], moved[2], settled ? ": settled" : ""); }
           if (settled) {
-            const double defect = handed_out_defect(after, cols); if (!hyh::ok()) { return 0; }
-            if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: largest cosine among the columns that can be handed out %.2le (wanted: %.2le)\n", used, defect, orthogonalTo); }
-            if (defect <= orthogonalTo) { break; }
-            if (defect <= 0.25 && polish(after, cols)) { break; }
-            if (!hyh::ok()) { return 0; }
+            const int state = orthonormal(after, cols); if (!hyh::ok()) { return 0; }
+            if (state != 0) { break; }
           }
         }
         lastCosine2 = seen.cosine2; before.swap(after);

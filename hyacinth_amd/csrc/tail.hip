@@ -214,6 +214,25 @@ extern "C" int hykMaxCosine(hipStream_t stream, int32_t Gtype, int32_t n, const 
   return hipGetLastError() == hipSuccess ? 0 : -3;
 }
 
+/* G <- (3 I - G) / 2 in place: the factor of the Newton-Schulz step V <- V (3 I - V^H V) / 2 from the Gram matrix G = V^H V */
+template <bool CPLX, typename GT>
+__global__ __launch_bounds__(T_THREADS) void newton_schulz_factor_kernel(int32_t n, GT* __restrict__ G, int64_t ldg) {
+  constexpr int W = CPLX ? 2 : 1; const int q = blockIdx.x;
+  for (int p = threadIdx.x; p < n; p += T_THREADS) {
+    GT* g = &G[((int64_t)p + (int64_t)q * ldg) * W];
+    g[0] = (GT)((p == q ? 1.5 : 0.) - 0.5 * (double)g[0]); if constexpr (CPLX) { g[1] = (GT)(-0.5 * (double)g[1]); }
+  }
+}
+
+extern "C" int hykNewtonSchulzFactor(hipStream_t stream, int32_t Gtype, int32_t n, void* G, int64_t ldg) {
+  if (n <= 0) { return 0; }
+  if (ldg < n || !btype_ok(Gtype)) { return -1; }
+  const bool Complex = Gtype & 1;
+  if ((Gtype & ~1) == HYK_F32) { if (Complex) { newton_schulz_factor_kernel<true, float><<<n, T_THREADS, 0, stream>>>(n, (float*)G, ldg); } else { newton_schulz_factor_kernel<false, float><<<n, T_THREADS, 0, stream>>>(n, (float*)G, ldg); } }
+  else if (Complex) { newton_schulz_factor_kernel<true, double><<<n, T_THREADS, 0, stream>>>(n, (double*)G, ldg); } else { newton_schulz_factor_kernel<false, double><<<n, T_THREADS, 0, stream>>>(n, (double*)G, ldg); }
+  return hipGetLastError() == hipSuccess ? 0 : -3;
+}
+
 extern "C" int hykMaxDefect(hipStream_t stream, int32_t Gtype, int32_t n, const void* G, int64_t ldg, double* out) {
   if (n <= 0) { return 0; }
   if (ldg < n || !btype_ok(Gtype)) { return -1; }

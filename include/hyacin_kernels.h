@@ -177,6 +177,9 @@ int hykMaxCosine(hipStream_t stream, int32_t Gtype, int32_t n, const void* G, in
 /* How far n columns are from orthonormal, from their Gram matrix (same types): *out (device, zero before the call) receives
  * the largest |G[p, q] - delta_pq|^2 over p <= q.  No counterpart in the reference. */
 int hykMaxDefect(hipStream_t stream, int32_t Gtype, int32_t n, const void* G, int64_t ldg, double* out);
+/* G <- (3 I - G) / 2 in place (same types): with G = V^H V, the factor T of the Newton-Schulz step V <- V T towards
+ * orthonormal columns of the same span.  No counterpart in the reference. */
+int hykNewtonSchulzFactor(hipStream_t stream, int32_t Gtype, int32_t n, void* G, int64_t ldg);
 int hykBasisOut(hipStream_t stream, int32_t N, int32_t rank, int32_t Atype, int32_t Btype, const void* B, const double* sigma, const int32_t* order, void* X, int64_t ldx);
 int hykValuesOut(hipStream_t stream, int32_t K, int32_t Atype, const double* S, void* out);
 

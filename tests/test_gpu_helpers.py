@@ -263,3 +263,11 @@ def test_max_defect(L, cplx, n, pad, wide):
         assert abs(got - want) <= 1e-12 * want
         assert (np.argmax(np.abs(G - np.eye(n))) % (n + 1) == 0) == (where == "diagonal" or n == 1)
     assert L.hykMaxDefect(stream(), (0 if wide else 2) + cplx, 5, ptr(dG), 4, ptr(out)) == -1
+    # hykNewtonSchulzFactor: G <- (3 I - G) / 2 in place, padding rows untouched
+    assert L.hykNewtonSchulzFactor(stream(), (0 if wide else 2) + cplx, n, ptr(dG), ld) == 0
+    sync()
+    got = host(dG, buf.dtype, buf.shape)
+    T = (got[:, :n, 0] + 1j * got[:, :n, 1]).T if cplx else got[:, :n].T
+    assert np.allclose(T, (3 * np.eye(n) - G) / 2, rtol=0, atol=1e-6 if not wide else 1e-15)
+    assert np.isnan(got[:, n:]).all()
+    assert L.hykNewtonSchulzFactor(stream(), (0 if wide else 2) + cplx, 5, ptr(dG), 4) == -1
