@@ -117,7 +117,7 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
     hyh::Scratch gram(handle, mayCheck ? (size_t)rank * rank * elemB : 0), dOut(handle, mayCheck ? 64 : 0);
     hyh::Scratch polishA(handle, mayCheck ? (size_t)N * K * elemB : 0), polishB(handle, mayCheck ? (size_t)N * K * elemB : 0), dPolishOrder(handle, mayCheck ? sizeof(int32_t) * (size_t)K : 0);
     if (!hyh::ok()) { return 0; }
-    const double orthogonalTo = std::sqrt(eps);
+    const double orthogonalTo = std::sqrt(eps), tightTo = std::max(eps, 64. * (wideB ? 2.220446049250313e-16 : 1.1920928955078125e-07));
     int32_t cols = rank; double dropped2 = 0., droppedSpectral = 0.;
     /* rank cut (reference: find_srank_kernel, src/gram_evd.cu:44-70): with the values in descending order (`order`), keep i < K
      * while sum_{j>=i} sigma_j^2 > eps^2 sum_j sigma_j^2; the columns left out of the sweeps count with what they weigh (the sum
@@ -135,7 +135,9 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
      * cluster of values that K cuts through (the sweeps bring its vectors apart slowly, and which basis of the cluster's
      * span is handed out is immaterial): V is made orthonormal directly, V <- V (3 I - V^H V) / 2 (the Newton-Schulz step
      * towards the orthonormal factor of V's polar decomposition: same span, so the same projection residual; a defect d
-     * becomes about d^2 per step), at most two steps, measured again after each.  It has to be exactly the vectors that are
+     * becomes about d^2 per step), measured again after each step.  sqrt(eps) is what is needed for the sweeps to end; the
+     * steps (three at most) go on to eps, or to the rounding of the copy's type, while they gain: the reference's vectors,
+     * a product of rotations, are orthonormal to rounding whatever state its sweeps end in.  It has to be exactly the vectors that are
      * handed out: a vector made orthogonal to one that is then dropped would carry a share of that direction and lose as
      * much of its own.  Returns 0: not orthogonal, the sweeps go on; 1: orthogonal as the columns are; 2: the first
      * `polishedCols` columns of `polished` are what is handed out, in the order `polishOrder`. */
@@ -145,22 +147,25 @@ extern "C" int32_t hyacinXGevd(const hyacinHandle_t* handle, double eps, int32_t
       HYH_CHECK(hipMemcpyAsync(dPolishOrder.p, polishOrder.data(), sizeof(int32_t) * (size_t)k, hipMemcpyHostToDevice, s));
       void* cur = polishA.p; void* nxt = polishB.p;
       HYH_KERNEL(hykBasisOut(s, N, k, Btype, Btype, B.p, sigma.as<double>(), dPolishOrder.as<int32_t>(), cur, N));   /* sigma holds the norms of the sweep just finished */
-      for (int step = 0; step <= 2 && hyh::ok(); ++step) {
+      double defect = 1., before_ = 2.; int steps = 0;
+      for (;; ++steps) {
         double defect2 = 1.;
         HYH_KERNEL(hykGramWorkspaceClear(s, dOut.p, 64));
         HYH_KERNEL(hykGemm(s, 'C', 'N', k, k, N, 1., Btype, cur, N, cur, N, 0., gram.p, k));
         HYH_KERNEL(hykMaxDefect(s, Btype, k, gram.p, k, dOut.as<double>()));   /* the diagonal included: a step leaves the norms off by about d^2 too */
         HYH_CHECK(hipMemcpyAsync(&defect2, dOut.p, sizeof(double), hipMemcpyDeviceToHost, s)); HYH_CHECK(hipStreamSynchronize(s));
         if (!hyh::ok()) { return 0; }
-        const double defect = std::sqrt(defect2);
-        if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: the %d vectors to be handed out%s: largest entry of V^H V - I %.2le (wanted: %.2le)\n", used, k, step ? " after an orthonormalisation step" : "", defect, orthogonalTo); }
-        if (defect <= orthogonalTo) { if (step == 0) { return 1; } polished = cur; polishedCols = k; return 2; }
-        if (defect > 0.25 || step == 2) { return 0; }
+        defect = std::sqrt(defect2);
+        if (handle->logger) { std::fprintf((FILE*)handle->logger, "GESVJ sweep %d: the %d vectors to be handed out%s: largest entry of V^H V - I %.2le (needed: %.2le, aimed at: %.2le)\n", used, k, steps ? " after an orthonormalisation step" : "", defect, orthogonalTo, tightTo); }
+        if (defect <= tightTo || steps == 3 || defect > 0.25 || defect > 0.25 * before_) { break; }   /* there, or out of steps, or too far for the step to converge, or no longer gaining */
+        before_ = defect;
         HYH_KERNEL(hykNewtonSchulzFactor(s, Btype, k, gram.p, k));
         HYH_KERNEL(hykGemm(s, 'N', 'N', N, k, k, 1., Btype, cur, N, gram.p, k, 0., nxt, N));
         std::swap(cur, nxt);
       }
-      return 0;
+      if (!hyh::ok() || defect > orthogonalTo) { return 0; }
+      if (steps == 0) { return 1; }
+      polished = cur; polishedCols = k; return 2;
     };
     /* Only the K largest values and their vectors are handed out.  Leaving the last rows of the Cholesky factor (the last
      * columns of B) out of the SVD takes a positive semidefinite matrix of trace tau (the sum of their squared norms) off
